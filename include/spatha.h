@@ -1,0 +1,168 @@
+/*
+ * spatha.h -- C ABI of the MI355X (gfx950) Spatha library: the V:N:M sparse
+ * format builder and the V:N:M sparse x dense SpMM.
+ *
+ * Plain C: pointers, sizes and an opaque handle.  Every entry point returns a
+ * spatha_status (0 = success), never exits the process and never throws.
+ * Host-side format functions take host pointers; spmm functions take device
+ * pointers and a HIP stream (passed as void* so that the header needs no HIP
+ * include; NULL is the default stream) and are stream ordered: no hidden
+ * synchronisation.  The caller owns every buffer it passes in; a handle owns
+ * only the copies it derives itself.
+ *
+ * Each declaration names the interface of the reference (UDC-GAC/venom) that it
+ * stands in for.
+ */
+#ifndef SPATHA_H
+#define SPATHA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum spatha_status {
+    SPATHA_OK = 0,
+    SPATHA_ERR_BAD_ARGUMENT = 1,   /* null pointer, negative size, n != 2, ...              */
+    SPATHA_ERR_BAD_SHAPE = 2,      /* rows % V, V % 32, m < 4, N alignment, ...             */
+    SPATHA_ERR_UNSUPPORTED = 3,    /* valid format, but no kernel for it (e.g. V = 32)      */
+    SPATHA_ERR_HIP = 4,            /* a HIP runtime call failed; see spatha_last_hip_error  */
+    SPATHA_ERR_NO_DEVICE = 5,      /* no HIP device visible                                 */
+    SPATHA_ERR_TOO_LARGE = 6       /* beyond a fixed capacity of the entry point            */
+} spatha_status;
+
+const char* spatha_status_string(int status);
+/* hipError_t of the last failing HIP call made by this library on this thread. */
+int spatha_last_hip_error(void);
+/* "major.minor.patch" */
+const char* spatha_version(void);
+
+/* ------------------------------------------------------------------------ *
+ * Format geometry.
+ * Replaces the size arithmetic of Format_sr_nm<T>::init
+ * (src/format/format_sr_nm.cpp:45-60) and SrNMTensor.to_sparse_sr_nm
+ * (end2end/grouped_nmv_tensor.py:709-719).
+ * ------------------------------------------------------------------------ */
+typedef struct spatha_vnm_geometry {
+    int32_t rows, cols, n, m, v;
+    int32_t ksp;          /* stored values per row: ROUND_UP(ceil(cols/m)*n, 16) */
+    int64_t n_values;     /* rows * ksp                                           */
+    int64_t n_metadata;   /* (rows/2) * (ksp/8) 32-bit words                      */
+    int64_t n_columns;    /* (rows/v) * (ksp/n) * 4 32-bit words                  */
+} spatha_vnm_geometry;
+
+int spatha_vnm_geometry_init(int rows, int cols, int n, int m, int v, spatha_vnm_geometry* out);
+
+/* ------------------------------------------------------------------------ *
+ * Host format builder (CPU; OpenMP over V-row blocks; threads <= 0 = all).
+ * ------------------------------------------------------------------------ */
+
+/* Random V:N:M pattern drawn from the C library's rand() in the reference's
+ * order, so that an un-seeded process produces the reference benchmark's
+ * pattern.  Replaces Format_sr_nm<T>::random_mask
+ * (src/format/format_sr_nm.cpp:151-237) and BlockwiseSpMatrix::random_mask
+ * (include/spatha/block_sparse/spmm/blockwise_format.h:159-246).
+ * metadata / columns must hold n_metadata / n_columns words, zero-filled. */
+int spatha_vnm_random_pattern(int rows, int cols, int n, int m, int v, uint32_t* metadata, uint32_t* columns);
+
+/* (float)(rand() % 9 - 4) fill used for A's values and for B by the reference
+ * benchmark (src/format/format_sr_nm.cpp:64-68, src/util/matrix_utils.h:88-97). */
+int spatha_fill_rand_small_ints_f16(uint16_t* out, int64_t count);
+
+/* Dense -> V:N:M.  dense is row-major rows x cols; columns holds, per V-row
+ * block and per m-column group, the 4 selected column offsets (ascending).
+ * mask == NULL: an entry is kept when it is non-zero
+ *   (Format_sr_nm<T>::to_sparse_sr_nm, src/format/format_sr_nm.cpp:419-543);
+ * mask != NULL (int32 rows x cols, 0/1): an entry is kept when its mask is set
+ *   (to_sparse_sr_nm / func2, end2end/grouped_nmv_tensor.py:487-675).
+ * A (row, group) with fewer than n kept entries gets zero-valued entries at the
+ * lowest unused positions (the reference leaves stale data there); more than n
+ * kept entries is an error (SPATHA_ERR_BAD_ARGUMENT). */
+int spatha_vnm_encode_f32(const float* dense, const int32_t* mask, const uint32_t* columns, int rows, int cols, int n,
+                          int m, int v, float* values, uint32_t* metadata, int threads);
+int spatha_vnm_encode_f16(const uint16_t* dense, const int32_t* mask, const uint32_t* columns, int rows, int cols,
+                          int n, int m, int v, uint16_t* values, uint32_t* metadata, int threads);
+
+/* V:N:M -> dense (dense is overwritten, zeros where nothing is stored).
+ * Replaces Format_sr_nm<T>::to_dense (src/format/format_sr_nm.cpp:327-417) and
+ * to_dense / func3 (end2end/grouped_nmv_tensor.py:345-485). */
+int spatha_vnm_decode_f32(const float* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
+                          int n, int m, int v, float* dense, int threads);
+int spatha_vnm_decode_f16(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows,
+                          int cols, int n, int m, int v, uint16_t* dense, int threads);
+
+/* Magnitude selector: per V-row block and m-column group pick the 4 columns
+ * that maximise the sum over rows of the n largest magnitudes; emits the 0/1
+ * mask and the column offsets.  dense_abs holds |A| as fp32.  masks (rows x
+ * cols) and columns (n_columns) must be zero-filled by the caller.
+ * Replaces group_n_m2 / func and nm_vector_mask_sparsify
+ * (end2end/grouped_nmv_tensor.py:81-343, :746-779). */
+int spatha_vnm_select_columns_f32(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
+                                  int32_t* columns, int threads);
+
+/* Layout of the single "metadata + column-loc" device blob the reference
+ * uploads: metadata words first, column-loc words at the next multiple of 8
+ * words.  Replaces BlockwiseSpMatrix<T>::transform_and_sync_device
+ * (include/spatha/block_sparse/spmm/blockwise_format.h:327-373) and
+ * Format_sr_nm<T>::transform_and_sync_device (src/format/format_sr_nm.cpp:239-285).
+ * blob may be NULL to query sizes only. */
+int spatha_vnm_pack_meta_blob(const uint32_t* metadata, int64_t n_metadata, const uint32_t* columns,
+                              int64_t n_columns, uint32_t* blob, int64_t* columns_offset_words,
+                              int64_t* blob_words);
+
+/* ------------------------------------------------------------------------ *
+ * SpMM on the GPU:  C[rows x N] = A_vnm[rows x cols] * B[cols x N],
+ * fp16 operands, fp32 accumulation, fp16 result (round to nearest even).
+ * ------------------------------------------------------------------------ */
+typedef struct spatha_spmm_plan spatha_spmm_plan;
+
+/* Builds a plan from the three canonical arrays, which are DEVICE pointers
+ * (values fp16[n_values], metadata u32[n_metadata], columns u32[n_columns]).
+ * The plan keeps derived copies laid out for the gfx950 sparse matrix
+ * instructions; the canonical arrays are not referenced after the call's work
+ * on `stream` has completed.  Replaces SpmmNMInitFn / SpmmBlockwiseOp::initialize
+ * (include/spatha/block_sparse/spmm/blockwise_op.h:98-161, :209-223) together
+ * with BlockwiseSpMatrix::init_sparse_device (blockwise_format.h:285-325). */
+int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint16_t* values_dev,
+                            const uint32_t* metadata_dev, const uint32_t* columns_dev, void* stream,
+                            spatha_spmm_plan** out);
+int spatha_spmm_plan_destroy(spatha_spmm_plan* plan);
+
+#define SPATHA_OUT_ROW_MAJOR 0   /* C[rows][N]           (benchmark path)                  */
+#define SPATHA_OUT_TRANSPOSED 1  /* C^T[N][rows] + bias  (PyTorch extension path)          */
+
+/* Runs one SpMM.  B is row-major cols x N (N contiguous), N % 8 == 0.
+ * out_layout SPATHA_OUT_ROW_MAJOR writes C[rows][N]; bias must be NULL
+ *   (SpmmNMExecFn, blockwise_op.h:233-238; main loop blockwise_kernel.h:739-944).
+ * out_layout SPATHA_OUT_TRANSPOSED writes C^T[N][rows] and, when bias != NULL,
+ *   adds bias[row] in fp16 to the rounded product (spmm_cuda,
+ *   end2end/spatha_mod/block_sparse/spmm/blockwise_library.cu:294-389, fused
+ *   epilogue end2end/spatha_mod/block_sparse/spmm/blockwise_kernel.h:294-343).
+ * variant selects a kernel: 0 = automatic. */
+int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
+                    uint16_t* out_dev, int out_layout, int variant, void* stream);
+
+/* Name / tile shape of the kernel `variant` (or of the automatic choice for N
+ * when variant == 0) would use, for logs; returns NULL if unsupported. */
+const char* spatha_spmm_kernel_name(const spatha_spmm_plan* plan, int N, int out_layout, int variant);
+
+/* Times `iters` back-to-back launches with HIP events on `stream` after
+ * `warmup` untimed ones; *ms_per_launch is the mean.  Replaces cuTime
+ * (src/cuda_utils.h:61-87) as used by Spatha<T,T2>::spmm
+ * (src/spmm/spatha_spmm.cpp:55-82). */
+int spatha_spmm_time(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
+                     uint16_t* out_dev, int out_layout, int variant, int warmup, int iters, void* stream,
+                     float* ms_per_launch);
+
+/* Dense fp16 GEMM C[rows x N] = A[rows x cols] * B[cols x N] (fp32 accumulate)
+ * on the GPU: the dense baseline and --check product of the benchmark.
+ * Replaces Cublas_gemm<half,half,float>::sgemm (src/gemm/cublas_gemm.cpp:54-96). */
+int spatha_dense_gemm_f16(const uint16_t* A_dev, const uint16_t* B_dev, int rows, int cols, int N, uint16_t* C_dev,
+                          void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPATHA_H */

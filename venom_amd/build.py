@@ -1,0 +1,59 @@
+"""Build recipe of the native library (venom_amd/lib/libspatha.so) and of the
+benchmark_spmm driver.
+
+    python -m venom_amd.build          # compile everything for gfx950
+
+Host-only sources go through g++ (OpenMP via libgomp), HIP sources through
+hipcc --offload-arch=gfx950; hipcc links.  Everything is built in-tree.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+OBJDIR = os.path.join(HERE, "build")
+LIB = os.path.join(LIBDIR, "libspatha.so")
+BENCH = os.path.join(LIBDIR, "benchmark_spmm")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ARCH = "gfx950"
+# packed fp32 VALU ops are kept off for every device compile
+HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
+             "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fopenmp", "-Wall"]
+
+HIP_SOURCES = ["spmm_kernels.hip", "dense_gemm.hip", "spatha_api.cpp"]
+CXX_SOURCES = ["vnm_format.cpp"]
+
+
+def _run(cmd, verbose):
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build(verbose=False, with_driver=True):
+    os.makedirs(LIBDIR, exist_ok=True)
+    os.makedirs(OBJDIR, exist_ok=True)
+    objs = []
+    for src in CXX_SOURCES:
+        obj = os.path.join(OBJDIR, src + ".o")
+        _run(["g++"] + CXX_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj], verbose)
+        objs.append(obj)
+    for src in HIP_SOURCES:
+        obj = os.path.join(OBJDIR, src + ".o")
+        lang = ["-x", "hip"] if src.endswith(".hip") else []
+        _run([HIPCC] + HIP_FLAGS + lang + ["-c", os.path.join(CSRC, src), "-o", obj], verbose)
+        objs.append(obj)
+    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB] + objs + ["-lgomp"], verbose)
+    if with_driver and os.path.exists(os.path.join(CSRC, "benchmark_spmm.cpp")):
+        _run([HIPCC] + HIP_FLAGS + [os.path.join(CSRC, "benchmark_spmm.cpp"), "-o", BENCH, "-L" + LIBDIR, "-lspatha",
+                                    "-Wl,-rpath,$ORIGIN", "-lgomp"], verbose)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(verbose=True)
+    sys.exit(0)

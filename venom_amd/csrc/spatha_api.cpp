@@ -1,0 +1,219 @@
+// C ABI of the library (see include/spatha.h): argument checking, plan
+// management and kernel selection.  No torch types, no exceptions across the
+// boundary, no exit().
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+
+#include "../../include/spatha.h"
+#include "spmm_kernels.h"
+#include "vnm_format.h"
+
+struct spatha_spmm_plan {
+    spatha_vnm_geometry geo;
+    int S;                 // k-steps of 64 compressed B rows
+    int device;
+    uint16_t* apack;
+    uint32_t* ipack;
+    uint32_t* rowtab;
+};
+
+namespace {
+thread_local int g_last_hip_error = 0;
+
+inline int hip_fail(hipError_t e) {
+    g_last_hip_error = (int)e;
+    return SPATHA_ERR_HIP;
+}
+
+int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
+    using namespace spatha;
+    (void)N;
+    const int v = plan->geo.v;
+    if (variant == SPMM_VARIANT_AUTO) {
+        if (v % 128 == 0) return SPMM_VARIANT_128x128;
+        if (v % 64 == 0) return SPMM_VARIANT_64x256;
+        return -1;
+    }
+    if (variant < 0 || variant >= SPMM_VARIANT_COUNT) return -1;
+    if (v % spmm_variant_bm(variant) != 0) return -1;
+    return variant;
+}
+}  // namespace
+
+extern "C" {
+
+const char* spatha_status_string(int status) {
+    switch (status) {
+        case SPATHA_OK: return "ok";
+        case SPATHA_ERR_BAD_ARGUMENT: return "bad argument";
+        case SPATHA_ERR_BAD_SHAPE: return "shape not representable in V:N:M (rows % V, V % 32, m >= 4, N % 8)";
+        case SPATHA_ERR_UNSUPPORTED: return "no kernel for this configuration";
+        case SPATHA_ERR_HIP: return "HIP runtime error";
+        case SPATHA_ERR_NO_DEVICE: return "no HIP device";
+        case SPATHA_ERR_TOO_LARGE: return "size beyond the entry point's capacity";
+        default: return "unknown status";
+    }
+}
+
+int spatha_last_hip_error(void) { return g_last_hip_error; }
+
+const char* spatha_version(void) { return "0.1.0"; }
+
+int spatha_vnm_geometry_init(int rows, int cols, int n, int m, int v, spatha_vnm_geometry* out) {
+    return spatha::geometry_init(rows, cols, n, m, v, out);
+}
+
+int spatha_vnm_random_pattern(int rows, int cols, int n, int m, int v, uint32_t* metadata, uint32_t* columns) {
+    return spatha::random_pattern(rows, cols, n, m, v, metadata, columns);
+}
+
+int spatha_fill_rand_small_ints_f16(uint16_t* out, int64_t count) {
+    if (!out || count < 0) return SPATHA_ERR_BAD_ARGUMENT;
+    // fp16 bit patterns of -4..4
+    static const uint16_t enc[9] = {0xC400, 0xC200, 0xC000, 0xBC00, 0x0000, 0x3C00, 0x4000, 0x4200, 0x4400};
+    for (int64_t i = 0; i < count; i++) out[i] = enc[std::rand() % 9];
+    return SPATHA_OK;
+}
+
+int spatha_vnm_encode_f32(const float* dense, const int32_t* mask, const uint32_t* columns, int rows, int cols, int n,
+                          int m, int v, float* values, uint32_t* metadata, int threads) {
+    return spatha::encode_f32(dense, mask, columns, rows, cols, n, m, v, values, metadata, threads);
+}
+int spatha_vnm_encode_f16(const uint16_t* dense, const int32_t* mask, const uint32_t* columns, int rows, int cols,
+                          int n, int m, int v, uint16_t* values, uint32_t* metadata, int threads) {
+    return spatha::encode_f16(dense, mask, columns, rows, cols, n, m, v, values, metadata, threads);
+}
+int spatha_vnm_decode_f32(const float* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
+                          int n, int m, int v, float* dense, int threads) {
+    return spatha::decode_f32(values, metadata, columns, rows, cols, n, m, v, dense, threads);
+}
+int spatha_vnm_decode_f16(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows,
+                          int cols, int n, int m, int v, uint16_t* dense, int threads) {
+    return spatha::decode_f16(values, metadata, columns, rows, cols, n, m, v, dense, threads);
+}
+int spatha_vnm_select_columns_f32(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
+                                  int32_t* columns, int threads) {
+    return spatha::select_columns_f32(dense_abs, rows, cols, n, m, v, masks, columns, threads);
+}
+int spatha_vnm_pack_meta_blob(const uint32_t* metadata, int64_t n_metadata, const uint32_t* columns,
+                              int64_t n_columns, uint32_t* blob, int64_t* columns_offset_words,
+                              int64_t* blob_words) {
+    return spatha::pack_meta_blob(metadata, n_metadata, columns, n_columns, blob, columns_offset_words, blob_words);
+}
+
+int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint16_t* values_dev,
+                            const uint32_t* metadata_dev, const uint32_t* columns_dev, void* stream,
+                            spatha_spmm_plan** out) {
+    if (!out) return SPATHA_ERR_BAD_ARGUMENT;
+    *out = nullptr;
+    spatha_vnm_geometry geo;
+    int st = spatha::geometry_init(rows, cols, n, m, v, &geo);
+    if (st) return st;
+    if (!values_dev || !metadata_dev || !columns_dev) return SPATHA_ERR_BAD_ARGUMENT;
+    if (v % 64 != 0) return SPATHA_ERR_UNSUPPORTED;   // kernels own 64-row wave tiles inside one V block
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    if (e != hipSuccess || ndev == 0) { g_last_hip_error = (int)e; return SPATHA_ERR_NO_DEVICE; }
+    spatha_spmm_plan* plan = new (std::nothrow) spatha_spmm_plan();
+    if (!plan) return SPATHA_ERR_BAD_ARGUMENT;
+    plan->geo = geo;
+    plan->S = (geo.ksp + 31) / 32;
+    plan->apack = nullptr; plan->ipack = nullptr; plan->rowtab = nullptr;
+    e = hipGetDevice(&plan->device);
+    if (e != hipSuccess) { delete plan; return hip_fail(e); }
+    const size_t a_bytes = (size_t)(rows / 64) * plan->S * 256 * 16;
+    const size_t i_bytes = (size_t)(rows / 64) * plan->S * 64 * 8;
+    const size_t r_bytes = (size_t)(rows / v) * plan->S * 64 * 4;
+    if ((e = hipMalloc((void**)&plan->apack, a_bytes)) != hipSuccess ||
+        (e = hipMalloc((void**)&plan->ipack, i_bytes)) != hipSuccess ||
+        (e = hipMalloc((void**)&plan->rowtab, r_bytes)) != hipSuccess) {
+        spatha_spmm_plan_destroy(plan);
+        return hip_fail(e);
+    }
+    e = spatha::launch_pack(values_dev, metadata_dev, columns_dev, rows, cols, m, v, geo.ksp, plan->S, plan->apack,
+                            plan->ipack, plan->rowtab, (hipStream_t)stream);
+    if (e != hipSuccess) { spatha_spmm_plan_destroy(plan); return hip_fail(e); }
+    *out = plan;
+    return SPATHA_OK;
+}
+
+int spatha_spmm_plan_destroy(spatha_spmm_plan* plan) {
+    if (!plan) return SPATHA_OK;
+    hipError_t first = hipSuccess, e;
+    if (plan->apack && (e = hipFree(plan->apack)) != hipSuccess && first == hipSuccess) first = e;
+    if (plan->ipack && (e = hipFree(plan->ipack)) != hipSuccess && first == hipSuccess) first = e;
+    if (plan->rowtab && (e = hipFree(plan->rowtab)) != hipSuccess && first == hipSuccess) first = e;
+    delete plan;
+    return first == hipSuccess ? SPATHA_OK : hip_fail(first);
+}
+
+int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
+                    uint16_t* out_dev, int out_layout, int variant, void* stream) {
+    if (!plan || !B_dev || !out_dev || N <= 0) return SPATHA_ERR_BAD_ARGUMENT;
+    if (out_layout != SPATHA_OUT_ROW_MAJOR && out_layout != SPATHA_OUT_TRANSPOSED) return SPATHA_ERR_BAD_ARGUMENT;
+    if (out_layout == SPATHA_OUT_ROW_MAJOR && bias_dev) return SPATHA_ERR_BAD_ARGUMENT;
+    if (N % 8 != 0) return SPATHA_ERR_BAD_SHAPE;      // 16-byte row segments of B and C
+    if (((uintptr_t)B_dev & 15) || ((uintptr_t)out_dev & 15) || ((uintptr_t)bias_dev & 15)) return SPATHA_ERR_BAD_ARGUMENT;
+    int var = pick_variant(plan, N, variant);
+    if (var < 0) return SPATHA_ERR_UNSUPPORTED;
+    spatha::SpmmParams p;
+    p.apack = plan->apack; p.ipack = plan->ipack; p.rowtab = plan->rowtab;
+    p.B = B_dev; p.bias = bias_dev; p.C = out_dev;
+    p.rows = plan->geo.rows; p.cols = plan->geo.cols; p.N = N; p.S = plan->S; p.v = plan->geo.v;
+    const int bm = spatha::spmm_variant_bm(var), bn = spatha::spmm_variant_bn(var);
+    p.tiles_m = plan->geo.rows / bm;
+    p.tiles_n = (N + bn - 1) / bn;
+    hipError_t e = spatha::launch_spmm(var, out_layout, p, (hipStream_t)stream);
+    return e == hipSuccess ? SPATHA_OK : hip_fail(e);
+}
+
+const char* spatha_spmm_kernel_name(const spatha_spmm_plan* plan, int N, int out_layout, int variant) {
+    (void)out_layout;
+    if (!plan) return nullptr;
+    int var = pick_variant(plan, N, variant);
+    return var < 0 ? nullptr : spatha::spmm_variant_name(var);
+}
+
+int spatha_spmm_time(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
+                     uint16_t* out_dev, int out_layout, int variant, int warmup, int iters, void* stream,
+                     float* ms_per_launch) {
+    if (!ms_per_launch || iters <= 0 || warmup < 0) return SPATHA_ERR_BAD_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    for (int i = 0; i < warmup; i++) {
+        int st = spatha_spmm_run(plan, B_dev, N, bias_dev, out_dev, out_layout, variant, stream);
+        if (st) return st;
+    }
+    hipEvent_t t0, t1;
+    hipError_t e;
+    if ((e = hipEventCreate(&t0)) != hipSuccess) return hip_fail(e);
+    if ((e = hipEventCreate(&t1)) != hipSuccess) { (void)hipEventDestroy(t0); return hip_fail(e); }
+    int st = SPATHA_OK;
+    e = hipEventRecord(t0, s);
+    for (int i = 0; i < iters && e == hipSuccess && st == SPATHA_OK; i++)
+        st = spatha_spmm_run(plan, B_dev, N, bias_dev, out_dev, out_layout, variant, stream);
+    if (e == hipSuccess) e = hipEventRecord(t1, s);
+    if (e == hipSuccess) e = hipEventSynchronize(t1);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    if (st) return st;
+    if (e != hipSuccess) return hip_fail(e);
+    *ms_per_launch = ms / (float)iters;
+    return SPATHA_OK;
+}
+
+int spatha_dense_gemm_f16(const uint16_t* A_dev, const uint16_t* B_dev, int rows, int cols, int N, uint16_t* C_dev,
+                          void* stream) {
+    if (!A_dev || !B_dev || !C_dev || rows <= 0 || cols <= 0 || N <= 0) return SPATHA_ERR_BAD_ARGUMENT;
+    if (N % 8 != 0 || cols % 8 != 0) return SPATHA_ERR_BAD_SHAPE;
+    hipError_t e = spatha::launch_dense_gemm(A_dev, B_dev, rows, cols, N, C_dev, (hipStream_t)stream);
+    return e == hipSuccess ? SPATHA_OK : hip_fail(e);
+}
+
+}  // extern "C"

@@ -1,0 +1,29 @@
+// Host-side V:N:M format builder (C++ interface behind the C ABI of spatha.h).
+#pragma once
+
+#include <cstdint>
+
+#include "../../include/spatha.h"
+
+namespace spatha {
+
+int geometry_init(int rows, int cols, int n, int m, int v, spatha_vnm_geometry* out);
+
+int random_pattern(int rows, int cols, int n, int m, int v, uint32_t* metadata, uint32_t* columns);
+
+int encode_f32(const float* dense, const int32_t* mask, const uint32_t* columns, int rows, int cols, int n, int m,
+               int v, float* values, uint32_t* metadata, int threads);
+int encode_f16(const uint16_t* dense, const int32_t* mask, const uint32_t* columns, int rows, int cols, int n, int m,
+               int v, uint16_t* values, uint32_t* metadata, int threads);
+int decode_f32(const float* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols, int n,
+               int m, int v, float* dense, int threads);
+int decode_f16(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols, int n,
+               int m, int v, uint16_t* dense, int threads);
+
+int select_columns_f32(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
+                       int32_t* columns, int threads);
+
+int pack_meta_blob(const uint32_t* metadata, int64_t n_metadata, const uint32_t* columns, int64_t n_columns,
+                   uint32_t* blob, int64_t* columns_offset_words, int64_t* blob_words);
+
+}  // namespace spatha

@@ -164,8 +164,10 @@ void encode_impl(const Geometry& g, const T* dense, const uint32_t* columns_in, 
                  uint32_t* meta_out, IsKept&& is_kept) {
     // Scratch that persists over the whole walk, as in format_sr_nm.cpp:437-439
     // (the reference leaves it uninitialised; zero is the only defined choice).
-    std::vector<T> vals(g.nelems, (T)0);
-    std::vector<uint32_t> idxs(g.nelems, 0u);
+    // A third kept entry is written one slot further on, where the next (row, group) of the
+    // walk overwrites it; the slack absorbs the one case that would leave the arrays.
+    std::vector<T> vals(g.nelems + 8, (T)0);
+    std::vector<uint32_t> idxs(g.nelems + 8, 0u);
     std::vector<uint32_t> cols(64, 0u);
     const int n = g.n, mrow_m = g.mrow_m, m_fixed = g.m_fixed;
     walk_tiles(g, [&](int bm_i, int mbrow_i, int mbrow_i2, int brow_i, int mcol_i, int mcol_kk, int mcol_k) {

@@ -1,0 +1,199 @@
+"""Parity of the gfx950 SpMM (through the C ABI) with the CPU oracle.
+
+Integer-valued operands make fp32 accumulation exact and order independent, so those cases
+must agree with the oracle BIT FOR BIT; Gaussian operands are held to max relative error
+1e-2 against the float64 product (the tolerance the task states for fp16 with fp32
+accumulation), measured as |got - exact| / max(|exact|, 1)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import golden_cases
+from venom_amd import _lib
+from venom_amd import format as F
+from venom_amd import spatha
+
+pytestmark = pytest.mark.gpu
+REL_TOL = 1e-2
+
+
+def _dev(a, gpu):
+    if a.dtype == np.uint32:
+        a = a.view(np.int32)
+    return torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+
+
+def _plan(vals, meta, columns, rows, cols, m, v, gpu):
+    return spatha.SpmmPlan(_dev(vals, gpu), _dev(meta, gpu), _dev(columns, gpu), rows, cols, 2, m, v)
+
+
+CASES = [
+    # rows, cols, N, m, v
+    (128, 256, 128, 8, 128),
+    (128, 256, 128, 8, 64),
+    (256, 512, 264, 16, 64),      # ragged N (not a multiple of any tile)
+    (256, 1024, 200, 8, 128),
+    (128, 48, 64, 8, 64),         # Ksp padded 12 -> 16: padding groups, half-filled last k-step
+    (256, 100, 72, 8, 128),       # cols % m != 0
+    (128, 64, 8, 4, 64),          # plain 2:4, N = 8
+    (256, 512, 16, 32, 128),      # m = 32, skinny N
+    (512, 640, 136, 20, 128),     # m not a power of two
+    (384, 416, 520, 8, 192),      # V = 192 (multiple of 64 only)
+]
+
+
+@pytest.mark.parametrize("rows,cols,N,m,v", CASES)
+@pytest.mark.parametrize("transposed", [False, True])
+def test_integer_operands_bit_exact(gpu, rows, cols, N, m, v, transposed):
+    print("case", rows, cols, N, m, v, transposed, flush=True)
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=rows + N, integer_values=True)
+    rng = np.random.default_rng(N)
+    B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+    bias = rng.integers(-3, 4, size=rows).astype(np.float16) if transposed else None
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias, transposed_out=transposed)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    for variant in (0, 1, 2):
+        if variant == 1 and v % 128:
+            continue
+        got = plan.run(_dev(B, gpu), bias=None if bias is None else _dev(bias, gpu), transposed_out=transposed,
+                       variant=variant)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16)), (variant,)
+
+
+@pytest.mark.parametrize("path", [p for p in golden_cases() if "_v64" in p or "_v128" in p],
+                         ids=lambda p: p.split("vnm_")[-1][:-4])
+def test_reference_encoded_matrices(gpu, path):
+    """Arrays written by the reference's own encoder go straight into the kernel."""
+    z = np.load(path)
+    n, m, v = int(z["n"]), int(z["m"]), int(z["v"])
+    rows, cols = z["dense"].shape
+    vals = z["values"].astype(np.float16)
+    rng = np.random.default_rng(1)
+    N = 72
+    B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+    exact = z["decoded"].astype(np.float16).astype(np.float64) @ B.astype(np.float64)
+    plan = _plan(vals, z["metadata"].view(np.uint32), z["columns"].astype(np.uint32), rows, cols, m, v, gpu)
+    got = plan.run(_dev(B, gpu)).cpu().numpy().astype(np.float64)
+    err = np.abs(got - exact) / np.maximum(np.abs(exact), 1.0)
+    assert err.max() <= REL_TOL
+    want = oracle.spmm(vals, z["metadata"].view(np.uint32), z["columns"].astype(np.uint32), rows, cols, n, m, v, B)
+    assert np.abs(got - want.astype(np.float64)).max() <= REL_TOL * np.maximum(np.abs(exact), 1.0).max()
+
+
+def test_config1_gaussian_within_tolerance(gpu):
+    """BASELINE config 1: 1024 x 4096 x 4096, 128:2:8, A ~ N(0,1), B ~ U(-1,1), seed 0."""
+    rows, cols, N, m, v = 1024, 4096, 4096, 8, 128
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=0, value_std=1.0)
+    rng = np.random.default_rng(0)
+    B = rng.uniform(-1, 1, size=(cols, N)).astype(np.float16)
+    dense = oracle.decode(vals, meta, columns, rows, cols, 2, m, v)
+    exact = dense.astype(np.float64) @ B.astype(np.float64)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    got = plan.run(_dev(B, gpu)).cpu().numpy().astype(np.float64)
+    err = np.abs(got - exact) / np.maximum(np.abs(exact), 1.0)
+    assert err.max() <= REL_TOL
+    # the reference's own acceptance rule (absolute 1.0 against the dense product)
+    assert oracle.check_results(got.astype(np.float16), exact.astype(np.float16)) == 0
+    # and against the oracle's fp32-accumulating SpMM on a slice of columns
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B[:, :256]).astype(np.float64)
+    assert (np.abs(got[:, :256] - want) / np.maximum(np.abs(exact[:, :256]), 1.0)).max() <= REL_TOL
+
+
+@pytest.mark.parametrize("rows,cols,N,m,v", [(4096, 1024, 16384, 8, 64), (1024, 4096, 16384, 8, 64),
+                                             (4096, 1024, 16384, 4, 128), (1024, 1024, 16384, 32, 128)])
+def test_full_size_checksums(gpu, rows, cols, N, m, v):
+    """BERT-large shapes at full size: row sums and column sums of C against products the CPU
+    can afford (C 1 = A (B 1), 1^T C = (1^T A) B), exact for small integers."""
+    print("full size", rows, cols, N, m, v, flush=True)
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=7, integer_values=True)
+    vals = np.clip(vals, -2, 2).astype(np.float16)
+    rng = np.random.default_rng(8)
+    B = rng.integers(-1, 2, size=(cols, N)).astype(np.float16)
+    dense = oracle.decode(vals, meta, columns, rows, cols, 2, m, v).astype(np.float64)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    C = plan.run(_dev(B, gpu))
+    Cd = C.double()
+    row_sums = Cd.sum(dim=1).cpu().numpy()
+    col_sums = Cd.sum(dim=0).cpu().numpy()
+    assert np.array_equal(row_sums, dense @ B.astype(np.float64).sum(axis=1))
+    assert np.array_equal(col_sums, dense.sum(axis=0) @ B.astype(np.float64))
+    # a random sample of full rows against the oracle
+    pick = rng.choice(rows, 4, replace=False)
+    want = dense[pick] @ B.astype(np.float64)
+    assert np.array_equal(C[torch.from_numpy(pick).to(gpu)].cpu().numpy().astype(np.float64), want)
+    # transposed output is the same numbers
+    Ct = plan.run(_dev(B, gpu), transposed_out=True)
+    assert torch.equal(Ct.t(), C)
+
+
+def test_linearity_in_B(gpu):
+    rows, cols, N, m, v = 512, 2048, 1024, 16, 128
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=3, integer_values=True)
+    rng = np.random.default_rng(4)
+    B1 = rng.integers(-2, 3, size=(cols, N)).astype(np.float16)
+    B2 = rng.integers(-2, 3, size=(cols, N)).astype(np.float16)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    c1 = plan.run(_dev(B1, gpu)).float()
+    c2 = plan.run(_dev(B2, gpu)).float()
+    c12 = plan.run(_dev(B1 + B2, gpu)).float()
+    assert torch.equal(c12, c1 + c2)
+
+
+def test_spmm_operator_signature(gpu):
+    """spatha.spmm with the reference's 15 arguments: transposed output plus bias."""
+    rows, cols, N, m, v = 256, 512, 384, 8, 64
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=5, integer_values=True)
+    rng = np.random.default_rng(6)
+    B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+    bias = rng.integers(-3, 4, size=rows).astype(np.float16)
+    out = spatha.spmm(_dev(meta, gpu), _dev(columns, gpu), _dev(vals, gpu), _dev(B, gpu), _dev(bias, gpu), rows, cols, N,
+                      v, 2, m, vals.size, 0, 32, 4)
+    assert tuple(out.shape) == (N, rows) and out.dtype == torch.float16
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias, transposed_out=True)
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_bias_rounding_is_one_fp16_add(gpu):
+    rows, cols, N, m, v = 128, 256, 64, 8, 64
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=9, value_std=1.0)
+    rng = np.random.default_rng(10)
+    B = rng.integers(-2, 3, size=(cols, N)).astype(np.float16)
+    bias = (rng.standard_normal(rows) * 3).astype(np.float16)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    raw = plan.run(_dev(B, gpu), transposed_out=True).cpu().numpy()
+    with_bias = plan.run(_dev(B, gpu), bias=_dev(bias, gpu), transposed_out=True).cpu().numpy()
+    want = oracle.add_half(raw.view(np.uint16), np.broadcast_to(bias.view(np.uint16)[None, :], raw.shape).copy())
+    assert np.array_equal(with_bias.view(np.uint16), want)
+
+
+def test_dense_gemm_baseline(gpu):
+    rng = np.random.default_rng(12)
+    rows, cols, N = 200, 328, 264
+    A = rng.integers(-4, 5, size=(rows, cols)).astype(np.float16)
+    B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+    dA, dB = _dev(A, gpu), _dev(B, gpu)
+    out = torch.empty((rows, N), dtype=torch.float16, device=gpu)
+    st = _lib.lib().spatha_dense_gemm_f16(dA.data_ptr(), dB.data_ptr(), rows, cols, N, out.data_ptr(),
+                                          torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), oracle.dense_gemm(A, B))
+
+
+def test_run_time_errors(gpu):
+    rows, cols, m, v = 128, 128, 8, 64
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=1, integer_values=True)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    B = torch.zeros((cols, 20), dtype=torch.float16, device=gpu)     # N % 8 != 0
+    with pytest.raises(_lib.SpathaError) as e:
+        plan.run(B)
+    assert e.value.status == 2
+    B = torch.zeros((cols, 16), dtype=torch.float16, device=gpu)
+    with pytest.raises(_lib.SpathaError) as e:
+        plan.run(B, variant=1)                                        # 128-row tile needs V % 128 == 0
+    assert e.value.status == 3
+    with pytest.raises(_lib.SpathaError) as e:
+        plan.run(B, bias=torch.zeros(rows, dtype=torch.float16, device=gpu))   # bias only with transposed output
+    assert e.value.status == 1

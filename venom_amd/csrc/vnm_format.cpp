@@ -106,6 +106,12 @@ int encode(const T* dense, const int32_t* mask, const uint32_t* columns, int row
                     uint32_t used = 0;
                     for (uint32_t c = 0; c < 4; c++) {
                         int64_t dcol = grp * m + cl[grp * 4 + c];
+                        // a column offset listed twice (the reference's selector leaves the fourth
+                        // offset of a 3-wide tail group at 0) names one matrix column: its first
+                        // listing is the entry, later listings add nothing
+                        bool repeat = false;
+                        for (uint32_t e = 0; e < c; e++) repeat |= (cl[grp * 4 + e] == cl[grp * 4 + c]);
+                        if (repeat && dcol < cols) continue;
                         if (dcol < cols) {
                             int64_t di = r * cols + dcol;
                             bool keep = mask ? (mask[di] != 0) : is_nonzero<T>(dense[di]);

@@ -1,0 +1,171 @@
+#!/usr/bin/env python3
+"""Headline benchmark: V:N:M SpMM at 64:2:8 on the BERT-large FFN-up shape.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one SpMM  C[4096 x 16384] = A_vnm[4096 x 1024] * B[1024 x 16384]  (fp16 operands,
+fp32 accumulation, fp16 result) with every operand already resident in HBM.  Prints ONE JSON
+line: dense-equivalent TFLOPS (2*M*K*N / t), microseconds per SpMM, the roofline of the SpMM
+kernel (HBM bound for this shape) and the CPU baseline (the CPU oracle's SpMM on a bounded
+sample of the same workload, timed on this host's cores)."""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+SMFMAC_PEAK_TFLOPS = 5033.0    # fp16 MFMA with 2:4 structured sparsity (dense fp16 peak 2516.6 x 2)
+
+
+def algorithmic_bytes(rows, cols, N, m, v, ksp):
+    """values + metadata + column-loc (as stored) + B read once + C written once."""
+    return 2 * rows * ksp + 4 * (rows // 2) * (ksp // 8) + 16 * (rows // v) * (ksp // 2) + 2 * cols * N + 2 * rows * N
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--rows", type=int, default=4096)
+    ap.add_argument("--cols", type=int, default=1024)
+    ap.add_argument("--n", type=int, default=16384, help="columns of B (tokens)")
+    ap.add_argument("--m", type=int, default=8)
+    ap.add_argument("--v", type=int, default=64)
+    ap.add_argument("--variant", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--extra", action="store_true", help="also time the other BASELINE shapes (reported under 'extra')")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the SpMM path has no multi-GPU part); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from venom_amd import _lib
+    from venom_amd import format as F
+    from venom_amd import spatha
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    L = _lib.lib()
+
+    def prepare(rows, cols, N, m, v, seed=0):
+        vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=seed, value_std=0.02)
+        g = F.geometry(rows, cols, 2, m, v)
+        plan = spatha.SpmmPlan(torch.from_numpy(vals).to(dev), torch.from_numpy(meta.view(np.int32)).to(dev),
+                               torch.from_numpy(columns.view(np.int32)).to(dev), rows, cols, 2, m, v)
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(seed)
+        B = torch.randn((cols, N), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+        C = torch.empty((rows, N), dtype=torch.float16, device=dev)
+        return dict(vals=vals, meta=meta, columns=columns, geo=g, plan=plan, B=B, C=C)
+
+    def timed(w, steps, warmup, variant=0):
+        """Wall clock around `steps` launches bracketed by synchronize, plus HIP events on the
+        launch stream over the same region (average kernel duration)."""
+        plan, B, C = w["plan"], w["B"], w["C"]
+        stream = torch.cuda.current_stream(dev)
+        sp = ctypes.c_void_p(stream.cuda_stream)
+        for _ in range(warmup):
+            _lib.check(L.spatha_spmm_run(plan._handle, B.data_ptr(), B.shape[1], None, C.data_ptr(), 0, variant, sp), "run")
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for _ in range(steps):
+            _lib.check(L.spatha_spmm_run(plan._handle, B.data_ptr(), B.shape[1], None, C.data_ptr(), 0, variant, sp), "run")
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+    rows, cols, N, m, v = args.rows, args.cols, args.n, args.m, args.v
+    w = prepare(rows, cols, N, m, v)
+    ms_wall, ms_kernel = timed(w, args.steps, args.warmup, args.variant)
+    ksp = w["geo"].ksp
+    flops_dense = 2.0 * rows * cols * N
+    flops_smfmac = 2.0 * rows * N * (2 * ksp)
+    nbytes = algorithmic_bytes(rows, cols, N, m, v, ksp)
+    tflops = flops_dense / (ms_wall * 1e-3) / 1e12
+    achieved_gbs = nbytes / (ms_kernel * 1e-3) / 1e9
+
+    out = {
+        "metric": "dense-equiv TFLOPS of the V:N:M SpMM at 64:2:8, BERT-large FFN",
+        "value": round(tflops, 2),
+        "unit": "TFLOPS (dense-equivalent, 2*M*K*N/t)",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_wall, 6),
+        "us_per_spmm": round(ms_wall * 1e3, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 (fp32 accumulate)",
+        "data": "synthetic (seed 0: A %d:2:%d random pattern, values ~N(0,0.02); B ~N(0,1))" % (v, m),
+        "config": {"workload": "spmm A %dx%d %d:2:%d (Ksp %d) x B %dx%d, row-major C" % (rows, cols, v, m, ksp, cols, N),
+                   "kernel": w["plan"].kernel_name(N, 0, args.variant)},
+        "pct_smfmac_peak": round(100.0 * flops_smfmac / (ms_kernel * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2),
+        "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes": nbytes, "kernel_us": round(ms_kernel * 1e3, 3)},
+    }
+
+    if args.extra:
+        extra = []
+        for (r2, c2, n2, m2, v2) in [(1024, 4096, 16384, 8, 64), (1024, 1024, 16384, 8, 64), (4096, 1024, 16384, 8, 128),
+                                     (1024, 4096, 4096, 8, 128), (4096, 1024, 16384, 4, 128),
+                                     (4096, 1024, 16384, 16, 64), (4096, 1024, 16384, 32, 64)]:
+            w2 = prepare(r2, c2, n2, m2, v2)
+            _, k2 = timed(w2, 50, 10)
+            by = algorithmic_bytes(r2, c2, n2, m2, v2, w2["geo"].ksp)
+            extra.append({"shape": "%dx%dx%d %d:2:%d" % (r2, c2, n2, v2, m2), "us": round(k2 * 1e3, 2),
+                          "dense_equiv_tflops": round(2.0 * r2 * c2 * n2 / (k2 * 1e-3) / 1e12, 1),
+                          "hbm_gbs": round(by / (k2 * 1e-3) / 1e9, 1),
+                          "pct_smfmac_peak": round(100 * 2.0 * r2 * n2 * 2 * w2["geo"].ksp / (k2 * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2)})
+            del w2
+        out["extra"] = extra
+
+    if not args.no_cpu_baseline:
+        import oracle
+
+        threads = min(oracle.num_threads(), os.cpu_count() or 1)
+        n_sample = min(N, 1024)
+        Bs = w["B"][:, :n_sample].contiguous().cpu().numpy()
+        t0 = time.perf_counter()
+        ref = oracle.spmm(w["vals"], w["meta"], w["columns"], rows, cols, 2, m, v, Bs, threads=threads)
+        t_spmm = time.perf_counter() - t0
+        # host format conversion of the same matrix, the reference's single-threaded way: decode + encode
+        t0 = time.perf_counter()
+        dense = oracle.decode(w["vals"], w["meta"], w["columns"], rows, cols, 2, m, v)
+        oracle.encode(dense, w["columns"], 2, m, v)
+        t_fmt = time.perf_counter() - t0
+        got = w["C"][:, :n_sample].cpu().numpy()
+        err = float(np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64)) /
+                           np.maximum(np.abs(ref.astype(np.float64)), 1.0)))
+        out["cpu_baseline"] = {
+            "value": round(2.0 * rows * cols * n_sample / t_spmm / 1e12, 5),
+            "unit": "TFLOPS (dense-equivalent)",
+            "cores": threads,
+            "kind": "port",
+            "sample": "oracle SpMM (compressed form, fp32 accumulate, OpenMP) on the first %d of %d columns of B: %.2f s; "
+                      "host format decode+encode of A, 1 thread: %.3f s; max rel err GPU vs oracle on the sample %.2e"
+                      % (n_sample, N, t_spmm, t_fmt, err),
+        }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -18,8 +18,9 @@ struct spatha_spmm_plan {
     int S;                 // k-steps of 64 compressed B rows
     int device;
     uint16_t* apack;
-    uint32_t* ipack;
     uint32_t* rowtab;
+    void* zeros;           // 1 KiB of zeros on the device
+    size_t apack_bytes, rowtab_bytes;
 };
 
 namespace {
@@ -41,6 +42,7 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
     }
     if (variant < 0 || variant >= SPMM_VARIANT_COUNT) return -1;
     if (v % spmm_variant_bm(variant) != 0) return -1;
+    if (spmm_variant_lds(variant, plan->S) > 160 * 1024) return -1;
     return variant;
 }
 }  // namespace
@@ -123,20 +125,21 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     if (!plan) return SPATHA_ERR_BAD_ARGUMENT;
     plan->geo = geo;
     plan->S = (geo.ksp + 31) / 32;
-    plan->apack = nullptr; plan->ipack = nullptr; plan->rowtab = nullptr;
+    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr;
     e = hipGetDevice(&plan->device);
     if (e != hipSuccess) { delete plan; return hip_fail(e); }
-    const size_t a_bytes = (size_t)(rows / 64) * plan->S * 256 * 16;
-    const size_t i_bytes = (size_t)(rows / 64) * plan->S * 64 * 8;
+    const size_t a_bytes = (size_t)(rows / 64) * plan->S * spatha::APACK_BLOCK;
     const size_t r_bytes = (size_t)(rows / v) * plan->S * 64 * 4;
+    plan->apack_bytes = a_bytes; plan->rowtab_bytes = r_bytes;
     if ((e = hipMalloc((void**)&plan->apack, a_bytes)) != hipSuccess ||
-        (e = hipMalloc((void**)&plan->ipack, i_bytes)) != hipSuccess ||
-        (e = hipMalloc((void**)&plan->rowtab, r_bytes)) != hipSuccess) {
+        (e = hipMalloc((void**)&plan->rowtab, r_bytes)) != hipSuccess ||
+        (e = hipMalloc(&plan->zeros, 1024)) != hipSuccess ||
+        (e = hipMemsetAsync(plan->zeros, 0, 1024, (hipStream_t)stream)) != hipSuccess) {
         spatha_spmm_plan_destroy(plan);
         return hip_fail(e);
     }
     e = spatha::launch_pack(values_dev, metadata_dev, columns_dev, rows, cols, m, v, geo.ksp, plan->S, plan->apack,
-                            plan->ipack, plan->rowtab, (hipStream_t)stream);
+                            plan->rowtab, (hipStream_t)stream);
     if (e != hipSuccess) { spatha_spmm_plan_destroy(plan); return hip_fail(e); }
     *out = plan;
     return SPATHA_OK;
@@ -146,8 +149,8 @@ int spatha_spmm_plan_destroy(spatha_spmm_plan* plan) {
     if (!plan) return SPATHA_OK;
     hipError_t first = hipSuccess, e;
     if (plan->apack && (e = hipFree(plan->apack)) != hipSuccess && first == hipSuccess) first = e;
-    if (plan->ipack && (e = hipFree(plan->ipack)) != hipSuccess && first == hipSuccess) first = e;
     if (plan->rowtab && (e = hipFree(plan->rowtab)) != hipSuccess && first == hipSuccess) first = e;
+    if (plan->zeros && (e = hipFree(plan->zeros)) != hipSuccess && first == hipSuccess) first = e;
     delete plan;
     return first == hipSuccess ? SPATHA_OK : hip_fail(first);
 }
@@ -162,12 +165,19 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
     int var = pick_variant(plan, N, variant);
     if (var < 0) return SPATHA_ERR_UNSUPPORTED;
     spatha::SpmmParams p;
-    p.apack = plan->apack; p.ipack = plan->ipack; p.rowtab = plan->rowtab;
-    p.B = B_dev; p.bias = bias_dev; p.C = out_dev;
+    p.apack = plan->apack; p.rowtab = plan->rowtab;
+    p.B = B_dev; p.bias = bias_dev; p.C = out_dev; p.zeros = plan->zeros;
     p.rows = plan->geo.rows; p.cols = plan->geo.cols; p.N = N; p.S = plan->S; p.v = plan->geo.v;
     const int bm = spatha::spmm_variant_bm(var), bn = spatha::spmm_variant_bn(var);
     p.tiles_m = plan->geo.rows / bm;
     p.tiles_n = (N + bn - 1) / bn;
+    {
+        const uint64_t bb = (uint64_t)plan->geo.cols * (uint64_t)N * 2u;
+        const bool fits32 = bb < 0xE0000000ull && plan->apack_bytes < 0xE0000000ull && plan->rowtab_bytes < 0xE0000000ull;
+        if (!fits32 && var >= spatha::SPMM_VARIANT_R128x128_S4) return SPATHA_ERR_UNSUPPORTED;
+        p.b_bytes = (uint32_t)bb; p.apack_bytes = (uint32_t)plan->apack_bytes; p.rowtab_bytes = (uint32_t)plan->rowtab_bytes;
+    }
+    { const char* d = std::getenv("SPATHA_DEBUG_KNOBS"); p.debug = d ? std::atoi(d) : 0; }
     hipError_t e = spatha::launch_spmm(var, out_layout, p, (hipStream_t)stream);
     return e == hipSuccess ? SPATHA_OK : hip_fail(e);
 }

@@ -8,28 +8,54 @@
 
 namespace spatha {
 
+enum { APACK_BLOCK = 4096 + 512 };
+
 struct SpmmParams {
-    const uint16_t* apack;    // packed A operands
-    const uint32_t* ipack;    // packed sparse-index fields
+    const uint16_t* apack;    // packed A operands + sparse-index words, APACK_BLOCK bytes per (64 rows, k-step)
     const uint32_t* rowtab;   // gathered B row per LDS row
     const uint16_t* B;        // cols x N, row-major
     const uint16_t* bias;     // rows, or null
+    const void* zeros;        // >= 1 KiB of zero bytes (source of zero-filled B rows)
     uint16_t* C;              // rows x N, or N x rows when transposed
     int rows, cols, N, S, v;
+    uint32_t b_bytes, apack_bytes, rowtab_bytes;   // sizes for buffer descriptors (persistent kernels)
     int tiles_m, tiles_n;
+    int debug;                // development knobs (0 in production): 1 = skip B loads, 2 = skip C stores
 };
 
-enum { SPMM_VARIANT_AUTO = 0, SPMM_VARIANT_128x128 = 1, SPMM_VARIANT_64x256 = 2, SPMM_VARIANT_COUNT = 3 };
+enum {
+    SPMM_VARIANT_AUTO = 0,
+    SPMM_VARIANT_128x128 = 1,      // register-staged, 2 LDS stages
+    SPMM_VARIANT_64x256 = 2,
+    SPMM_VARIANT_P128x128_S4 = 3,  // direct-to-LDS pipeline
+    SPMM_VARIANT_P128x128_S3 = 4,
+    SPMM_VARIANT_P64x256_S2 = 5,
+    SPMM_VARIANT_P64x256_S3 = 6,
+    SPMM_VARIANT_P128x128_S6 = 7,
+    SPMM_VARIANT_P64x256_S4 = 8,
+    SPMM_VARIANT_R128x128_S4 = 9,  // persistent, pipeline runs across tiles
+    SPMM_VARIANT_R128x128_S5 = 10,
+    SPMM_VARIANT_R128x128_S2 = 11,
+    SPMM_VARIANT_R64x256_S3 = 12,
+    SPMM_VARIANT_R64x256_S4 = 13,
+    SPMM_VARIANT_W128x128_S5 = 14,  // persistent + producer/consumer wave specialisation
+    SPMM_VARIANT_W128x128_S3 = 15,
+    SPMM_VARIANT_W128x128_S2 = 16,
+    SPMM_VARIANT_W128x256_S3 = 17,
+    SPMM_VARIANT_W64x256_S2 = 18,
+    SPMM_VARIANT_W64x256_S3 = 19,
+    SPMM_VARIANT_COUNT = 20
+};
 
 const char* spmm_variant_name(int variant);
 int spmm_variant_bm(int variant);
 int spmm_variant_bn(int variant);
+int spmm_variant_lds(int variant, int S);
 
 hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
-                       int m, int v, int ksp, int S, uint16_t* apack, uint32_t* ipack, uint32_t* rowtab,
-                       hipStream_t stream);
+                       int m, int v, int ksp, int S, uint16_t* apack, uint32_t* rowtab, hipStream_t stream);
 
 hipError_t launch_dense_gemm(const uint16_t* A, const uint16_t* B, int rows, int cols, int N, uint16_t* C,
                              hipStream_t stream);

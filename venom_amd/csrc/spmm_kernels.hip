@@ -23,8 +23,9 @@
 // row e; lane i receives column i of rows 0..3.
 //
 // Data layout produced once per matrix by pack_kernel (all "derived copies"):
-//   apack  half [rows/64][S][4 mb][64 lanes][8]   A operands, S = ceil(Ksp/32) k-steps
-//   ipack  u32  [rows/64][S][64 lanes][2]         idx fields: word d = mb 2d | mb 2d+1 << 16
+//   apack  [rows/64][S] blocks of APACK_BLOCK = 4608 bytes, S = ceil(Ksp/32) k-steps:
+//            half [4 mb][64 lanes][8]             A operands
+//            u32  [2 d][64 lanes]                 idx fields: word d = mb 2d | mb 2d+1 << 16
 //   rowtab u32  [rows/V][S*64]                    B row feeding LDS row rho of step s
 //                                                 (group*m + column-loc, or ~0 = zero row)
 // Inside a 64-row wave tile the sparse-instruction row (mb, i = 4*ib + r) holds
@@ -41,6 +42,7 @@ namespace spatha {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 half16_t __attribute__((ext_vector_type(16)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -53,7 +55,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 // One thread per (wave tile, step, mb, lane) for apack/ipack; rowtab separately.
 // ---------------------------------------------------------------------------
 __global__ void pack_a_kernel(const uint16_t* __restrict__ values, const uint32_t* __restrict__ metadata, int rows,
-                              int ksp, int S, uint16_t* __restrict__ apack, uint32_t* __restrict__ ipack) {
+                              int ksp, int S, uint16_t* __restrict__ apack) {
     const int64_t total = (int64_t)(rows / 64) * S * 4 * 64;
     const int ngroups = ksp / 2;
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
@@ -94,10 +96,10 @@ __global__ void pack_a_kernel(const uint16_t* __restrict__ values, const uint32_
         out.y = vals[2] | ((uint32_t)vals[3] << 16);
         out.z = vals[4] | ((uint32_t)vals[5] << 16);
         out.w = vals[6] | ((uint32_t)vals[7] << 16);
-        *(u32x4*)(apack + t * 8) = out;
-        // idx: [wt][s][lane][2] words, 16 bits per mb
-        uint16_t* ip16 = (uint16_t*)ipack;
-        ip16[((ws * 64 + lane) * 2 + (mb >> 1)) * 2 + (mb & 1)] = (uint16_t)idx16;
+        char* blk = (char*)apack + ws * APACK_BLOCK;
+        *(u32x4*)(blk + mb * 1024 + lane * 16) = out;
+        // index words: [d][lane] dwords after the operands, 16 bits per mb (mb = 2d + half)
+        *(uint16_t*)(blk + 4096 + (mb >> 1) * 256 + lane * 4 + (mb & 1) * 2) = (uint16_t)idx16;
     }
 }
 
@@ -152,8 +154,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_kernel(SpmmParams p) {
     const int S = p.S, N = p.N;
 
     const int64_t wt = (int64_t)(m0 / 64 + wm);                       // wave tile index along rows
-    const u32x4* a_ptr = (const u32x4*)p.apack + (wt * S) * 256 + lane;   // + s*256 + mb*64
-    const u32x2* i_ptr = (const u32x2*)p.ipack + (wt * S) * 64 + lane;    // + s*64
+    const char* a_blk = (const char*)p.apack + (wt * S) * APACK_BLOCK;   // + s*APACK_BLOCK
     const uint32_t* rt = p.rowtab + (int64_t)(m0 / p.v) * S * 64;
 
     // B loader coordinates
@@ -177,11 +178,12 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_kernel(SpmmParams p) {
         for (int i = 0; i < B_LOADS; i++) {
             uint32_t row = rows_next[i];
             u32x4 z = {0u, 0u, 0u, 0u};
-            breg[i] = (row != 0xffffffffu && bcol_ok) ? *(const u32x4*)(bbase + (int64_t)row * N) : z;
+            breg[i] = (row != 0xffffffffu && bcol_ok && !(p.debug & 1)) ? *(const u32x4*)(bbase + (int64_t)row * N) : z;
         }
 #pragma unroll
-        for (int mb = 0; mb < 4; mb++) areg[mb] = a_ptr[(int64_t)s * 256 + mb * 64];
-        ireg = i_ptr[(int64_t)s * 64];
+        for (int mb = 0; mb < 4; mb++) areg[mb] = *(const u32x4*)(a_blk + (int64_t)s * APACK_BLOCK + mb * 1024 + lane * 16);
+        ireg.x = *(const uint32_t*)(a_blk + (int64_t)s * APACK_BLOCK + 4096 + lane * 4);
+        ireg.y = *(const uint32_t*)(a_blk + (int64_t)s * APACK_BLOCK + 4096 + 256 + lane * 4);
     };
     auto store_lds = [&](int stage) {
         char* base = smem + stage * STAGE_B + br * PITCH_B + bc * 16;
@@ -299,9 +301,954 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_kernel(SpmmParams p) {
             const int row = 16 * (L & 3) + (L >> 2);
             const int col = n0 + wn * 64 + ch * 8;
             u32x4 v = *(const u32x4*)(st + L * PITCH_C + ch * 16);
-            if (col < N) *(u32x4*)(p.C + ((int64_t)m0 + wm * 64 + row) * N + col) = v;
+            if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)m0 + wm * 64 + row) * N + col) = v;
         }
     }
+}
+
+
+// ---------------------------------------------------------------------------
+// One k-step of a wave's 64 x 64 tile out of an LDS stage: 4 A operands + index words,
+// 4 B fragments (16 transposing reads), 16 sparse matrix instructions.  The B fragments are
+// double buffered in registers and `between` (the next stage's DMA issue) runs after the
+// first reads have been sent, so that LDS latency overlaps address arithmetic and matrix work
+// instead of being paid once per fragment.
+// ---------------------------------------------------------------------------
+template <int ROW_BYTES>
+__device__ __forceinline__ half16_t read_b_fragment(const char* st, int off) {
+    half16_t bf;
+#pragma unroll
+    for (int fb = 0; fb < 4; fb++) {
+        short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, st + off + fb * 16 * ROW_BYTES));
+        half4_t h4 = __builtin_bit_cast(half4_t, t4);
+        bf[fb * 4 + 0] = h4[0];
+        bf[fb * 4 + 1] = h4[1];
+        bf[fb * 4 + 2] = h4[2];
+        bf[fb * 4 + 3] = h4[3];
+    }
+    return bf;
+}
+
+#define SPATHA_MMA4(NB, BF)                                                                                   \
+    acc[0][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[0], BF, acc[0][NB], (int)i0, 0, 0);           \
+    acc[1][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], BF, acc[1][NB], (int)i0, 0, 1);           \
+    acc[2][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], BF, acc[2][NB], (int)i1, 0, 0);           \
+    acc[3][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], BF, acc[3][NB], (int)i1, 0, 1);
+
+template <int ROW_BYTES, class Between>
+__device__ __forceinline__ void mma_stage(const char* st, int a_off, int i_off, const int (&tr_off)[4],
+                                          float4_t (&acc)[4][4], Between&& between) {
+    half8_t a_cur[4];
+#pragma unroll
+    for (int mb = 0; mb < 4; mb++) a_cur[mb] = *(const half8_t*)(st + a_off + mb * 1024);
+    const uint32_t i0 = *(const uint32_t*)(st + i_off), i1 = *(const uint32_t*)(st + i_off + 256);
+    half16_t bf0 = read_b_fragment<ROW_BYTES>(st, tr_off[0]);
+    half16_t bf1 = read_b_fragment<ROW_BYTES>(st, tr_off[1]);
+    __builtin_amdgcn_sched_barrier(0);
+    between();
+    __builtin_amdgcn_sched_barrier(0);
+    SPATHA_MMA4(0, bf0)
+    __builtin_amdgcn_sched_barrier(0);
+    bf0 = read_b_fragment<ROW_BYTES>(st, tr_off[2]);
+    __builtin_amdgcn_sched_barrier(0);
+    SPATHA_MMA4(1, bf1)
+    __builtin_amdgcn_sched_barrier(0);
+    bf1 = read_b_fragment<ROW_BYTES>(st, tr_off[3]);
+    __builtin_amdgcn_sched_barrier(0);
+    SPATHA_MMA4(2, bf0)
+    SPATHA_MMA4(3, bf1)
+}
+
+// ---------------------------------------------------------------------------
+// Pipelined SpMM kernel.  Everything the k-loop consumes -- the gathered B rows, the packed
+// A operands and their index words -- is copied global -> LDS by the DMA path
+// (global_load_lds_dwordx4 / _dword: no VGPR staging, no LDS store instructions) NS-1
+// k-steps ahead of the step being multiplied.  One workgroup barrier per k-step.
+//
+// The DMA loads are issued from inline assembly on purpose: the compiler's wait-count
+// insertion treats every LDS read as a possible alias of every outstanding LDS-DMA write and
+// would drain the whole queue (vmcnt(0)) before the first read of each step, which removes
+// the overlap this kernel exists for.  No other vector-memory instruction is issued inside
+// the loop, so the explicit s_waitcnt vmcnt(k) below is the only bookkeeping: a wave issues
+// exactly LOADS_PER_STAGE DMA instructions per stage, in stage order.  The asm statements carry
+// no "memory" clobber (it would stop the compiler from reading the row table with scalar
+// loads); they are volatile, so they keep their order relative to each other and to the
+// workgroup barrier, which is what separates a stage's DMA writes from its LDS reads.
+//
+// LDS layout of one stage:
+//   [0, 64*BN*2)                gathered B rows, row pitch BN*2 bytes (a DMA instruction writes
+//                               1 KiB contiguous, so rows cannot be padded); bank conflicts of
+//                               the transposing reads are avoided by XOR-ing the 16-byte chunk
+//                               index of row rho with 2*(rho % 8) on the GLOBAL side of the copy
+//   [.., + WM*APACK_BLOCK)      per 64-row wave tile: 4 KiB A operands + 512 B index words
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void dma_b128(const void* gptr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "m0");
+}
+__device__ __forceinline__ void dma_b32(const void* gptr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(gptr) : "m0");
+}
+template <int N_>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N_ >= 0 && N_ < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_));
+}
+template <int L, int MAXK>
+__device__ __forceinline__ void wait_stages(int k) {
+    // wait until at most k stages (k * L loads) of this wave are still in flight
+    if constexpr (MAXK == 0) {
+        wait_vmcnt<0>();
+    } else {
+        if (k >= MAXK) wait_vmcnt<MAXK * L>();
+        else wait_stages<L, MAXK - 1>(k);
+    }
+}
+
+template <int WM, int WN, int NS, int OUT_LAYOUT>
+__global__ __launch_bounds__(WM* WN * 64) void spmm_pipe_kernel(SpmmParams p) {
+    constexpr int NW = WM * WN;
+    constexpr int BM = WM * 64, BN = WN * 64;
+    constexpr int ROW_BYTES = BN * 2;
+    constexpr int B_BYTES = 64 * ROW_BYTES;
+    constexpr int STAGE_BYTES = B_BYTES + WM * APACK_BLOCK;
+    constexpr int CHUNKS = BN / 8;                   // 16-byte chunks per row
+    constexpr int ROWS_PER_INST = 1024 / ROW_BYTES;  // rows one DMA instruction covers (4 or 2)
+    constexpr int NB_LOADS = 64 / ROWS_PER_INST / NW;  // B DMA instructions per wave per stage
+    constexpr int NA_X4 = 4 / WN > 0 ? 4 / WN : 1;   // A-operand DMA instructions per wave per stage
+    constexpr int LOADS_PER_STAGE = NB_LOADS + NA_X4 + 1;
+    constexpr int PA = NS - 1;                       // prefetch distance in k-steps
+    constexpr int PITCH_C = 144;
+    static_assert(WN == 1 || WN == 2 || WN == 4, "A operand split");
+    static_assert(64 % (ROWS_PER_INST * NW) == 0, "rows per step must split over the waves");
+    static_assert((NS - 2) * LOADS_PER_STAGE < 64, "vmcnt range");
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    uint32_t* lds_rt = (uint32_t*)(smem + NS * STAGE_BYTES);      // row table of this V block: S*64 words
+
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int chunk = (tiles + 7) >> 3;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int tile = xcd * chunk + local;
+    if (local >= chunk || tile >= tiles) return;
+    const int tile_n = tile / p.tiles_m, tile_m = tile - tile_n * p.tiles_m;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave - wm * WN;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int S = p.S, N = p.N;
+
+    const char* a_src = (const char*)p.apack + ((int64_t)(m0 / 64 + wm) * S) * APACK_BLOCK;
+    const uint32_t* rt = p.rowtab + (int64_t)(m0 / p.v) * S * 64;
+
+    // ---- B loader: this lane's slot in each of the wave's NB_LOADS instructions
+    const int slot_row = lane / CHUNKS;
+    const int slot_chunk = lane % CHUNKS;
+    int64_t b_col_off[NB_LOADS];                     // byte offset of the source chunk inside a B row, or -1
+    const char* zero_src = (const char*)p.zeros + lane * 16;
+#pragma unroll
+    for (int j = 0; j < NB_LOADS; j++) {
+        const int rho = (wave * NB_LOADS + j) * ROWS_PER_INST + slot_row;
+        const int src_chunk = slot_chunk ^ ((rho & 7) << 1);
+        const int col = n0 + src_chunk * 8;
+        b_col_off[j] = (col < N) ? (int64_t)col * 2 : -1;
+    }
+    auto issue_stage = [&](int s) {
+        const uint32_t stage = smem_base + (s % NS) * STAGE_BYTES;
+        uint32_t rows[NB_LOADS];
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) rows[j] = lds_rt[s * 64 + (wave * NB_LOADS + j) * ROWS_PER_INST + slot_row];
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) {
+            const int inst = wave * NB_LOADS + j;
+            const bool ok = (rows[j] != 0xffffffffu) && (b_col_off[j] >= 0) && !(p.debug & 1);
+            const char* src = (const char*)p.B + (int64_t)rows[j] * N * 2 + b_col_off[j];
+            src = ok ? src : zero_src;
+            dma_b128(src, stage + inst * 1024);
+        }
+        // A operands of wave tile wm: the WN waves of the row split the 4 operand blocks; the
+        // two index blocks go to waves with even / odd wn (duplicates write identical bytes)
+        const char* ab = a_src + (int64_t)s * APACK_BLOCK;
+        const uint32_t a_lds = stage + B_BYTES + wm * APACK_BLOCK;
+#pragma unroll
+        for (int k = 0; k < NA_X4; k++) {
+            const int mb = (WN >= 4) ? wn : wn * NA_X4 + k;
+            dma_b128(ab + mb * 1024 + lane * 16, a_lds + mb * 1024);
+        }
+        const int d = wn & 1;
+        dma_b32(ab + 4096 + d * 256 + lane * 4, a_lds + 4096 + d * 256);
+        if (WN == 1) dma_b32(ab + 4096 + 256 + lane * 4, a_lds + 4096 + 256);
+    };
+    constexpr int L = LOADS_PER_STAGE + (WN == 1 ? 1 : 0);
+
+    float4_t acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+    // transposing-read offsets: row fb*16 + kb*4 + i/4; 16-byte chunk (wn*8 + nb*2 + (i%4)/2) ^ swizzle
+    const int li = lane & 15, kb = lane >> 4;
+    const int rrow = kb * 4 + (li >> 2);
+    const int sw = rrow & 7;
+    int tr_off[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int ch = (wn * 8 + nb * 2 + ((li & 3) >> 1)) ^ (sw << 1);
+        tr_off[nb] = rrow * ROW_BYTES + ch * 16 + (li & 1) * 8;
+    }
+    const int a_off = B_BYTES + wm * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + wm * APACK_BLOCK + 4096 + lane * 4;
+
+    // ---- the V-block's row table goes to LDS once (ordinary loads, before any DMA is in flight:
+    //      a vector load inside the loop would make the compiler drain the DMA queue)
+    for (int i = tid; i < S * 64; i += NW * 64) lds_rt[i] = rt[i];
+    __syncthreads();
+
+    // ---- prologue: NS-1 stages in flight
+#pragma unroll
+    for (int t = 0; t < PA; t++)
+        if (t < S) issue_stage(t);
+
+    for (int s = 0; s < S; s++) {
+        // stages after s that this wave has already issued may stay in flight
+        const int later = (S - 1 - s) < (NS - 2) ? (S - 1 - s) : (NS - 2);
+        wait_stages<L, NS - 2>(later);
+        __syncthreads();          // stage s is complete for every wave; stage s-1 is no longer read
+        mma_stage<ROW_BYTES>(smem + (s % NS) * STAGE_BYTES, a_off, i_off, tr_off, acc, [&]() {
+            if (s + PA < S) issue_stage(s + PA);
+        });
+    }
+
+    // ------------------------------------------------------------------ epilogue
+    const int j = lane & 15, ib = lane >> 4;
+    if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+        const int64_t row0 = (int64_t)m0 + wm * 64 + ib * 16;
+        half8_t bias_lo, bias_hi;
+        if (p.bias) {
+            bias_lo = *(const half8_t*)(p.bias + row0);
+            bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+        }
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+            const int col = n0 + wn * 64 + nb * 16 + j;
+            half8_t lo, hi;
+#pragma unroll
+            for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
+                    hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
+                }
+            if (p.bias) {
+                lo = lo + bias_lo;
+                hi = hi + bias_hi;
+            }
+            if (col < N) {
+                uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
+                *(half8_t*)dst = lo;
+                *(half8_t*)(dst + 8) = hi;
+            }
+        }
+    } else if (!(p.debug & 4)) {
+        __syncthreads();                 // every wave is done reading the stages
+        char* stg = smem + wave * (64 * PITCH_C);
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int Lr = (4 * mb + r) * 4 + ib;
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++)
+                    *(_Float16*)(stg + Lr * PITCH_C + (nb * 16 + j) * 2) = (_Float16)acc[mb][nb][r];
+            }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+            const int Lr = it * 8 + (lane >> 3), ch = lane & 7;
+            const int row = 16 * (Lr & 3) + (Lr >> 2);
+            const int col = n0 + wn * 64 + ch * 8;
+            u32x4 v = *(const u32x4*)(stg + Lr * PITCH_C + ch * 16);
+            if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)m0 + wm * 64 + row) * N + col) = v;
+        }
+    }
+}
+
+template <int WM, int WN, int NS, int OUT_LAYOUT>
+static hipError_t launch_pipe(const SpmmParams& p, hipStream_t stream) {
+    constexpr int BN = WN * 64;
+    constexpr int stage_bytes = NS * (64 * BN * 2 + WM * APACK_BLOCK);
+    static_assert(stage_bytes >= WM * WN * 64 * 144, "the epilogue staging reuses the stage buffers");
+    const int lds = stage_bytes + p.S * 256;
+    if (lds > 160 * 1024) return hipErrorInvalidValue;     // callers check with spmm_variant_fits first
+    static bool attr_set = false;
+    auto kern = spmm_pipe_kernel<WM, WN, NS, OUT_LAYOUT>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int chunk = (tiles + 7) / 8;
+    hipLaunchKernelGGL(kern, dim3(chunk * 8), dim3(WM * WN * 64), lds, stream, p);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Persistent pipelined SpMM kernel.
+//
+// One workgroup per CU slot walks a list of C tiles; the k-steps of all its tiles form one
+// flat sequence, and the DMA pipeline (NS LDS stages, NS-1 steps ahead) runs across tile
+// boundaries, so the load latency at the start of a tile and the store latency at its end
+// are hidden behind the neighbouring tiles' work.
+//
+// All loads inside the loop are buffer loads with the LDS modifier (buffer_load_dword[x4] ...
+// offen lds) issued from inline assembly (see the note on spmm_pipe_kernel).  A buffer
+// descriptor's bounds check returns zero for an out-of-range offset; zero rows of B (padding
+// groups, columns beyond K, columns beyond N) are therefore requested at offset 0xF0000000.
+//
+// Per k-step each wave issues one batch, always in this order and always complete:
+//   NB_LOADS x  b128   gathered B rows of stage f = q + NS-1      -> stage f % NS
+//   NA_X4    x  b128   A operands of stage f                       -> stage f % NS
+//   1        x  b32    index words of stage f                      -> stage f % NS
+//   1        x  b32    row table of stage f + NS-1 (this wave's private ring)
+// and waits with s_waitcnt vmcnt(k * LOADS) for the batch issued NS-1 steps earlier.
+// ---------------------------------------------------------------------------
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ i32x4 make_buffer(const void* base, uint32_t bytes) {
+    const uint64_t a = (uint64_t)(uintptr_t)base;
+    i32x4 r;
+    r.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+    r.y = __builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu));   // stride 0: raw buffer
+    r.z = __builtin_amdgcn_readfirstlane((int)bytes);
+    r.w = 0x00020000;
+    return r;
+}
+__device__ __forceinline__ void bdma_b128(uint32_t voff, i32x4 rsrc, uint32_t soff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc),
+                 "s"(soff)
+                 : "m0");
+}
+__device__ __forceinline__ void bdma_b32(uint32_t voff, i32x4 rsrc, uint32_t soff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc),
+                 "s"(soff)
+                 : "m0");
+}
+
+template <int WM, int WN, int NS>
+struct PersistCfg {
+    static constexpr int NW = WM * WN;
+    static constexpr int BM = WM * 64, BN = WN * 64;
+    static constexpr int ROW_BYTES = BN * 2;
+    static constexpr int B_BYTES = 64 * ROW_BYTES;
+    static constexpr int STAGE_BYTES = B_BYTES + WM * APACK_BLOCK;
+    static constexpr int PA = NS - 1;
+    static constexpr int EPI_PITCH = 144;
+    static constexpr int EPI_BYTES = NW * 16 * EPI_PITCH;          // one 16-row slab per wave at a time
+    static constexpr int RT_BYTES = NW * (PA + 1) * 256;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES + EPI_BYTES + RT_BYTES;
+};
+
+template <int WM, int WN, int NS, int OUT_LAYOUT>
+__global__ __launch_bounds__(WM* WN * 64) void spmm_persist_kernel(SpmmParams p) {
+    using Cfg = PersistCfg<WM, WN, NS>;
+    constexpr int NW = Cfg::NW, BM = Cfg::BM, BN = Cfg::BN;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int CHUNKS = BN / 8;
+    constexpr int RPI = 1024 / ROW_BYTES;            // rows one DMA instruction covers (4 or 2)
+    constexpr int NB_LOADS = 64 / RPI / NW;
+    constexpr int NA_X4 = 4 / WN > 0 ? 4 / WN : 1;
+    constexpr int LOADS = NB_LOADS + NA_X4 + 2;
+    constexpr int PA = Cfg::PA;
+    constexpr int EPI_PITCH = Cfg::EPI_PITCH;
+    static_assert(WN == 2 || WN == 4, "A operand split");
+    static_assert(64 % (RPI * NW) == 0, "rows per step must split over the waves");
+    static_assert((PA - 1) * LOADS < 64, "vmcnt range");
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave - wm * WN;
+    const int S = p.S, N = p.N;
+
+    // ---- this workgroup's tile list: XCD x (= id % 8) owns a contiguous range of tile ids
+    //      (id -> n-tile major, m-tile minor); its workgroups take them round robin.  Tile
+    //      coordinates advance by a fixed (dm, dn) with carry: no division per tile.
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int chunk = (tiles + 7) >> 3;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+    const int first = xcd * chunk;
+    const int last = (first + chunk) < tiles ? (first + chunk) : tiles;      // exclusive
+    int my_tiles = 0;
+    if (first + slot < last) my_tiles = (last - first - slot + slots - 1) / slots;
+    if (my_tiles == 0) return;
+    const int Q = my_tiles * S;
+    const int step_dn = slots / p.tiles_m, step_dm = slots - step_dn * p.tiles_m;
+    const int tn0 = (first + slot) / p.tiles_m, tm0 = (first + slot) - tn0 * p.tiles_m;
+    auto next_tile = [&](int& tm, int& tn) {
+        tm += step_dm;
+        tn += step_dn;
+        if (tm >= p.tiles_m) { tm -= p.tiles_m; tn += 1; }
+    };
+    const int tiles_per_vblock = p.v / BM;           // V % BM == 0 is checked on the host
+
+    const i32x4 rsrc_b = make_buffer(p.B, p.b_bytes);
+    const i32x4 rsrc_a = make_buffer(p.apack, p.apack_bytes);
+    const i32x4 rsrc_rt = make_buffer(p.rowtab, p.rowtab_bytes);
+    const uint32_t row_bytes_b = (uint32_t)N * 2u;
+
+    // ---- LDS regions
+    constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
+    const uint32_t rt_base = EPI_BASE + Cfg::EPI_BYTES + wave * ((PA + 1) * 256);
+
+    // ---- B loader slots of this lane
+    const int slot_row = lane / CHUNKS;
+    const int slot_chunk = lane % CHUNKS;
+    int src_chunk[NB_LOADS];
+#pragma unroll
+    for (int j = 0; j < NB_LOADS; j++) {
+        const int rho = (wave * NB_LOADS + j) * RPI + slot_row;
+        src_chunk[j] = slot_chunk ^ ((rho & 7) << 1);
+    }
+    const uint32_t lane16 = lane * 16, lane4 = lane * 4;
+    const uint32_t rt_lane_off = (uint32_t)((wave * NB_LOADS) * RPI + slot_row) * 4;   // + j*RPI*4
+
+    // ---- issue state (all scalar except coloff): stage f = next batch to issue
+    int is_tm = tm0, is_tn = tn0, is_step = 0;
+    uint32_t is_stage = 0;                                   // byte offset of the LDS stage for f
+    uint32_t a_soff = (uint32_t)((is_tm * (BM / 64) + wm) * S) * (uint32_t)APACK_BLOCK;
+    int issue_left = Q;                                      // batches not yet issued
+    uint32_t rt_read = 0;                                    // ring slot (bytes) holding the rows of stage f
+    // row-table state: stage f + PA (clamped to the last stage)
+    int rt_tm = tm0, rt_tn = tn0, rt_step = 0, rt_left = Q - 1;   // advances still allowed
+    uint32_t rt_soff = (uint32_t)((rt_tm / tiles_per_vblock) * S) * 256u;
+    uint32_t coloff[NB_LOADS];
+    auto set_coloff = [&]() {
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) {
+            const int col = is_tn * BN + src_chunk[j] * 8;
+            coloff[j] = (col < N && !(p.debug & 1)) ? (uint32_t)col * 2u : 0xF0000000u;
+        }
+    };
+    set_coloff();
+    auto rt_advance = [&]() {
+        if (rt_left > 0) {
+            --rt_left;
+            rt_soff += 256u;
+            if (++rt_step == S) {
+                rt_step = 0;
+                next_tile(rt_tm, rt_tn);
+                rt_soff = (uint32_t)((rt_tm / tiles_per_vblock) * S) * 256u;
+            }
+        }
+    };
+
+    // issues the batch of stage f with the given rows and moves the issue state to f + 1
+    auto issue_batch = [&](const uint32_t (&rows)[NB_LOADS]) {
+        const uint32_t stage = smem_base + is_stage;
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) {
+            const uint32_t voff = (rows[j] == 0xffffffffu) ? 0xF0000000u : rows[j] * row_bytes_b + coloff[j];
+            bdma_b128(voff, rsrc_b, 0, stage + (wave * NB_LOADS + j) * 1024);
+        }
+        const uint32_t a_lds = stage + B_BYTES + wm * APACK_BLOCK;
+#pragma unroll
+        for (int k = 0; k < NA_X4; k++) {
+            const int mb = (WN >= 4) ? wn : wn * NA_X4 + k;
+            bdma_b128(lane16, rsrc_a, a_soff + mb * 1024, a_lds + mb * 1024);
+        }
+        const int d = wn & 1;
+        bdma_b32(lane4, rsrc_a, a_soff + 4096 + d * 256, a_lds + 4096 + d * 256);
+        // row table of stage f + PA goes to the ring slot just before the one read now
+        const uint32_t rt_write = (rt_read == 0) ? (uint32_t)PA * 256u : rt_read - 256u;
+        bdma_b32(lane4, rsrc_rt, rt_soff, smem_base + rt_base + rt_write);
+        rt_advance();
+        // advance to stage f + 1
+        --issue_left;
+        is_stage = (is_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : is_stage + STAGE_BYTES;
+        rt_read = (rt_read == (uint32_t)PA * 256u) ? 0u : rt_read + 256u;
+        a_soff += (uint32_t)APACK_BLOCK;
+        if (++is_step == S) {
+            is_step = 0;
+            next_tile(is_tm, is_tn);
+            a_soff = (uint32_t)((is_tm * (BM / 64) + wm) * S) * (uint32_t)APACK_BLOCK;
+            set_coloff();
+        }
+    };
+
+    float4_t acc[4][4];
+
+    const int li = lane & 15, kb = lane >> 4;
+    const int rrow = kb * 4 + (li >> 2);
+    const int sw = rrow & 7;
+    int tr_off[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int ch = (wn * 8 + nb * 2 + ((li & 3) >> 1)) ^ (sw << 1);
+        tr_off[nb] = rrow * ROW_BYTES + ch * 16 + (li & 1) * 8;
+    }
+    const int a_off = B_BYTES + wm * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + wm * APACK_BLOCK + 4096 + lane * 4;
+
+    // ---- prologue: the first PA batches take their rows through ordinary loads (nothing is in
+    //      flight yet); the row-table cursor starts PA stages ahead of the issue cursor.
+    {
+        uint32_t rows0[PA][NB_LOADS];
+        int st_tm = tm0, st_tn = tn0, st_step = 0;
+#pragma unroll
+        for (int t = 0; t < PA; t++) {
+            const int64_t base = ((int64_t)(st_tm / tiles_per_vblock) * S + st_step) * 64;
+#pragma unroll
+            for (int j = 0; j < NB_LOADS; j++)
+                rows0[t][j] = (t < Q) ? p.rowtab[base + (wave * NB_LOADS + j) * RPI + slot_row] : 0xffffffffu;
+            if (++st_step == S) { st_step = 0; next_tile(st_tm, st_tn); }
+        }
+#pragma unroll
+        for (int t = 0; t < PA; t++) rt_advance();
+#pragma unroll
+        for (int t = 0; t < PA; t++)
+            if (t < Q) issue_batch(rows0[t]);
+    }
+
+    const int j16 = lane & 15, ib = lane >> 4;
+    int c_tm = tm0, c_tn = tn0;
+    int q_left = Q;                 // steps not yet multiplied
+    uint32_t c_stage = 0;           // byte offset of the stage multiplied next
+    for (int c_tile = 0; c_tile < my_tiles; c_tile++) {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            // batches issued after the one needed now may stay in flight
+            if (q_left > PA - 1) wait_vmcnt<(PA - 1) * LOADS>();
+            else wait_stages<LOADS, PA - 1>(q_left - 1);
+            --q_left;
+            __syncthreads();
+            mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {
+                if (issue_left > 0) {
+                    uint32_t rows[NB_LOADS];
+                    const char* rr = smem + rt_base + rt_read + rt_lane_off;
+#pragma unroll
+                    for (int j = 0; j < NB_LOADS; j++) rows[j] = *(const uint32_t*)(rr + j * (RPI * 4));
+                    issue_batch(rows);
+                }
+            });
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+        }
+        // ------------------------------------------------ tile finished: write it out
+        const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+            const int64_t row0 = (int64_t)cm0 + wm * 64 + ib * 16;
+            half8_t bias_lo, bias_hi;
+            if (p.bias) {
+                bias_lo = *(const half8_t*)(p.bias + row0);
+                bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+            }
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++) {
+                const int col = cn0 + wn * 64 + nb * 16 + j16;
+                half8_t lo, hi;
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
+                        hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
+                    }
+                if (p.bias) {
+                    lo = lo + bias_lo;
+                    hi = hi + bias_hi;
+                }
+                if (col < N && !(p.debug & 2)) {
+                    uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
+                    *(half8_t*)dst = lo;
+                    *(half8_t*)(dst + 8) = hi;
+                }
+            }
+        } else if (!(p.debug & 4)) {
+            // 16-row slabs through a wave-private LDS buffer -> 128-byte row segments
+            char* stg = smem + EPI_BASE + wave * (16 * EPI_PITCH);
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int nb = 0; nb < 4; nb++)
+                        *(_Float16*)(stg + (r * 4 + ib) * EPI_PITCH + (nb * 16 + j16) * 2) = (_Float16)acc[mb][nb][r];
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int it = 0; it < 2; it++) {
+                    const int Lr = it * 8 + (lane >> 3), ch = lane & 7;
+                    const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
+                    const int col = cn0 + wn * 64 + ch * 8;
+                    u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
+                    if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col) = v;
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+        next_tile(c_tm, c_tn);
+    }
+}
+
+template <int WM, int WN, int NS, int OUT_LAYOUT>
+static hipError_t launch_persist(const SpmmParams& p, hipStream_t stream) {
+    using Cfg = PersistCfg<WM, WN, NS>;
+    constexpr int lds = Cfg::LDS_BYTES;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static bool attr_set = false;
+    static int cus = 0;
+    auto kern = spmm_persist_kernel<WM, WN, NS, OUT_LAYOUT>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        int dev = 0;
+        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int per_cu = (160 * 1024) / lds;
+    const int tiles = p.tiles_m * p.tiles_n;
+    int grid = cus * per_cu;
+    grid = (grid / 8) * 8;
+    const int need = ((tiles + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    if (grid < 8) grid = 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(WM * WN * 64), lds, stream, p);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Warp-specialised persistent SpMM kernel.
+//
+// The workgroup has NC = WM*WN consumer waves and NP producer waves.  Consumers do nothing
+// but read operands from LDS and issue sparse matrix instructions (and write finished tiles);
+// producers do nothing but address arithmetic and DMA issue for the stages NS-1 k-steps
+// ahead.  A wave can issue roughly one instruction every few cycles, so keeping the
+// bookkeeping out of the consumers' instruction stream is what lets their matrix pipe stay
+// busy.  One workgroup barrier per k-step joins the two roles:
+//   producer: wait own DMA of stage q | barrier | issue stage q + NS-1
+//   consumer:                           barrier | multiply stage q
+// Producer pr stands in for the wave (wm = pr / 2, wn = pr % 2) of the 2 x 2 arrangement when
+// it comes to which DMA instructions of a stage it issues.
+// ---------------------------------------------------------------------------
+template <int WM, int WN, int NS, int NP>
+struct WsCfg {
+    static constexpr int NC = WM * WN;
+    static constexpr int BM = WM * 64, BN = WN * 64;
+    static constexpr int ROW_BYTES = BN * 2;
+    static constexpr int B_BYTES = 64 * ROW_BYTES;
+    static constexpr int STAGE_BYTES = B_BYTES + WM * APACK_BLOCK;
+    static constexpr int PA = NS - 1;
+    static constexpr int EPI_PITCH = 144;
+    static constexpr int EPI_BYTES = NC * 16 * EPI_PITCH;
+    static constexpr int RT_BYTES = NP * (PA + 1) * 256;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES + EPI_BYTES + RT_BYTES;
+    static constexpr int THREADS = (NC + NP) * 64;
+    static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
+    static constexpr uint32_t RT_BASE = EPI_BASE + EPI_BYTES;
+};
+
+// Tile walk shared by both roles: XCD x (= workgroup id % 8) owns a contiguous range of tile
+// ids (id -> n-tile major, m-tile minor) and its workgroups take them round robin; the
+// coordinates advance by a fixed (dm, dn) with carry, so no division per tile.
+struct TileWalk {
+    int my_tiles, tm0, tn0, step_dm, step_dn, tiles_m;
+    __device__ __forceinline__ void init(int tiles_m_, int tiles_n_) {
+        tiles_m = tiles_m_;
+        const int tiles = tiles_m_ * tiles_n_;
+        const int chunk = (tiles + 7) >> 3;
+        const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+        const int first = xcd * chunk;
+        const int last = (first + chunk) < tiles ? (first + chunk) : tiles;
+        my_tiles = 0;
+        if (first + slot < last) my_tiles = (last - first - slot + slots - 1) / slots;
+        step_dn = slots / tiles_m;
+        step_dm = slots - step_dn * tiles_m;
+        tn0 = (first + slot) / tiles_m;
+        tm0 = (first + slot) - tn0 * tiles_m;
+    }
+    __device__ __forceinline__ void next(int& tm, int& tn) const {
+        tm += step_dm;
+        tn += step_dn;
+        if (tm >= tiles_m) { tm -= tiles_m; tn += 1; }
+    }
+};
+
+template <class Cfg, int NP, int PR>
+__device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk& walk, char* smem, uint32_t smem_base,
+                                            int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1, PA = Cfg::PA;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int WM = BM / 64;
+    constexpr int CHUNKS = BN / 8;
+    constexpr int RPI = 1024 / ROW_BYTES;
+    constexpr int NB_LOADS = 64 / RPI / NP;          // B DMA instructions per producer per stage
+    constexpr int A_INSTR = WM * 6;                  // per wave-tile row: 4 operand blocks + 2 index blocks
+    constexpr int NA_LOADS = A_INSTR / NP;
+    constexpr int LOADS = NB_LOADS + NA_LOADS + 1;
+    static_assert(64 % (RPI * NP) == 0 && A_INSTR % NP == 0, "DMA work must split evenly over the producers");
+    static_assert((PA - 1) * LOADS < 64, "vmcnt range");
+
+    const int S = p.S, N = p.N;
+    const int Q = walk.my_tiles * S;
+    const int tiles_per_vblock = p.v / BM;
+    const i32x4 rsrc_b = make_buffer(p.B, p.b_bytes);
+    const i32x4 rsrc_a = make_buffer(p.apack, p.apack_bytes);
+    const i32x4 rsrc_rt = make_buffer(p.rowtab, p.rowtab_bytes);
+    const uint32_t row_bytes_b = (uint32_t)N * 2u;
+    constexpr uint32_t rt_base = Cfg::RT_BASE + PR * ((PA + 1) * 256);
+    const int slot_row = lane / CHUNKS, slot_chunk = lane % CHUNKS;
+    int src_chunk[NB_LOADS];
+#pragma unroll
+    for (int j = 0; j < NB_LOADS; j++) {
+        const int rho = (PR * NB_LOADS + j) * RPI + slot_row;
+        src_chunk[j] = slot_chunk ^ ((rho & 7) << 1);
+    }
+    const uint32_t lane16 = lane * 16, lane4 = lane * 4;
+    const uint32_t rt_lane_off = (uint32_t)((PR * NB_LOADS) * RPI + slot_row) * 4;
+
+    int is_tm = walk.tm0, is_tn = walk.tn0, is_step = 0;
+    uint32_t is_stage = 0;
+    uint32_t rt_read = 0;
+    int rt_tm = walk.tm0, rt_tn = walk.tn0, rt_step = 0, rt_left = Q - 1;
+    uint32_t rt_soff = (uint32_t)((rt_tm / tiles_per_vblock) * S) * 256u;
+    uint32_t a_soff = (uint32_t)((is_tm * WM) * S) * (uint32_t)APACK_BLOCK;    // wave-tile row 0 of the tile
+    uint32_t coloff[NB_LOADS];
+    auto set_coloff = [&]() {
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) {
+            const int col = is_tn * BN + src_chunk[j] * 8;
+            coloff[j] = (col < N && !(p.debug & 1)) ? (uint32_t)col * 2u : 0xF0000000u;
+        }
+    };
+    set_coloff();
+    auto rt_advance = [&]() {
+        if (rt_left > 0) {
+            --rt_left;
+            rt_soff += 256u;
+            if (++rt_step == S) {
+                rt_step = 0;
+                walk.next(rt_tm, rt_tn);
+                rt_soff = (uint32_t)((rt_tm / tiles_per_vblock) * S) * 256u;
+            }
+        }
+    };
+    auto issue_batch = [&](const uint32_t (&rows)[NB_LOADS]) {
+        const uint32_t stage = smem_base + is_stage;
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) {
+            const uint32_t voff = (rows[j] == 0xffffffffu) ? 0xF0000000u : rows[j] * row_bytes_b + coloff[j];
+            bdma_b128(voff, rsrc_b, 0, stage + (PR * NB_LOADS + j) * 1024);
+        }
+        // the A_INSTR operand / index blocks of the stage, NA_LOADS consecutive ones per producer:
+        // instruction a = wm*6 + k; k < 4: operand block k (1 KiB); k >= 4: index block k-4 (256 B)
+#pragma unroll
+        for (int k = 0; k < NA_LOADS; k++) {
+            constexpr int dummy = 0;
+            (void)dummy;
+            const int a = PR * NA_LOADS + k;
+            const int awm = a / 6, ak = a - awm * 6;
+            const uint32_t soff = a_soff + (uint32_t)(awm * S) * (uint32_t)APACK_BLOCK;
+            const uint32_t dst = stage + B_BYTES + awm * APACK_BLOCK;
+            if (ak < 4) bdma_b128(lane16, rsrc_a, soff + ak * 1024, dst + ak * 1024);
+            else bdma_b32(lane4, rsrc_a, soff + 4096 + (ak - 4) * 256, dst + 4096 + (ak - 4) * 256);
+        }
+        const uint32_t rt_write = (rt_read == 0) ? (uint32_t)PA * 256u : rt_read - 256u;
+        bdma_b32(lane4, rsrc_rt, rt_soff, smem_base + rt_base + rt_write);
+        rt_advance();
+        is_stage = (is_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : is_stage + STAGE_BYTES;
+        rt_read = (rt_read == (uint32_t)PA * 256u) ? 0u : rt_read + 256u;
+        a_soff += (uint32_t)APACK_BLOCK;
+        if (++is_step == S) {
+            is_step = 0;
+            walk.next(is_tm, is_tn);
+            a_soff = (uint32_t)((is_tm * WM) * S) * (uint32_t)APACK_BLOCK;
+            set_coloff();
+        }
+    };
+    // prologue: rows of the first PA stages through ordinary loads (nothing is in flight yet)
+    {
+        uint32_t rows0[PA][NB_LOADS];
+        int st_tm = walk.tm0, st_tn = walk.tn0, st_step = 0;
+#pragma unroll
+        for (int t = 0; t < PA; t++) {
+            const int64_t base = ((int64_t)(st_tm / tiles_per_vblock) * S + st_step) * 64;
+#pragma unroll
+            for (int j = 0; j < NB_LOADS; j++)
+                rows0[t][j] = (t < Q) ? p.rowtab[base + (PR * NB_LOADS + j) * RPI + slot_row] : 0xffffffffu;
+            if (++st_step == S) { st_step = 0; walk.next(st_tm, st_tn); }
+        }
+#pragma unroll
+        for (int t = 0; t < PA; t++) rt_advance();
+#pragma unroll
+        for (int t = 0; t < PA; t++)
+            if (t < Q) issue_batch(rows0[t]);
+    }
+    auto issue_from_ring = [&]() {
+        uint32_t rows[NB_LOADS];
+        const char* rr = smem + rt_base + rt_read + rt_lane_off;
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) rows[j] = *(const uint32_t*)(rr + j * (RPI * 4));
+        issue_batch(rows);
+    };
+    // steady state: PA-1 younger batches stay in flight behind the one being waited for
+    const int q_main = Q - PA > 0 ? Q - PA : 0;       // steps that still issue a batch
+    for (int q = 0; q < q_main; q++) {
+        wait_vmcnt<(PA - 1) * LOADS>();
+        __syncthreads();
+        if (!(p.debug & 8)) issue_from_ring();
+    }
+    // drain: nothing left to issue
+    for (int q = q_main; q < Q; q++) {
+        wait_stages<LOADS, PA - 1>(Q - 1 - q);
+        __syncthreads();
+    }
+}
+
+template <class Cfg, int WN, int OUT_LAYOUT>
+__device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int EPI_PITCH = Cfg::EPI_PITCH;
+    const int S = p.S, N = p.N;
+    const int wm = wave / WN, wn = wave - wm * WN;
+    float4_t acc[4][4];
+    const int li = lane & 15, kb = lane >> 4;
+    const int rrow = kb * 4 + (li >> 2);
+    const int sw = rrow & 7;
+    int tr_off[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int ch = (wn * 8 + nb * 2 + ((li & 3) >> 1)) ^ (sw << 1);
+        tr_off[nb] = rrow * ROW_BYTES + ch * 16 + (li & 1) * 8;
+    }
+    const int a_off = B_BYTES + wm * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + wm * APACK_BLOCK + 4096 + lane * 4;
+    const int j16 = lane & 15, ib = lane >> 4;
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    uint32_t c_stage = 0;
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            __syncthreads();
+            if (!(p.debug & 16)) mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {});
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+        }
+        const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+            // the lane owns 16 consecutive matrix rows of one output column: 32 contiguous bytes
+            const int64_t row0 = (int64_t)cm0 + wm * 64 + ib * 16;
+            half8_t bias_lo, bias_hi;
+            if (p.bias) {
+                bias_lo = *(const half8_t*)(p.bias + row0);
+                bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+            }
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++) {
+                const int col = cn0 + wn * 64 + nb * 16 + j16;
+                half8_t lo, hi;
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
+                        hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
+                    }
+                if (p.bias) {
+                    lo = lo + bias_lo;
+                    hi = hi + bias_hi;
+                }
+                if (col < N && !(p.debug & 2)) {
+                    uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
+                    *(half8_t*)dst = lo;
+                    *(half8_t*)(dst + 8) = hi;
+                }
+            }
+        } else if (!(p.debug & 4)) {
+            // 16-row slabs through a wave-private LDS buffer -> 128-byte row segments
+            char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int nb = 0; nb < 4; nb++)
+                        *(_Float16*)(stg + (r * 4 + ib) * EPI_PITCH + (nb * 16 + j16) * 2) = (_Float16)acc[mb][nb][r];
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int it = 0; it < 2; it++) {
+                    const int Lr = it * 8 + (lane >> 3), ch = lane & 7;
+                    const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
+                    const int col = cn0 + wn * 64 + ch * 8;
+                    u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
+                    if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col) = v;
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+        walk.next(c_tm, c_tn);
+    }
+}
+
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT>
+__global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams p) {
+    using Cfg = WsCfg<WM, WN, NS, NP>;
+    static_assert(NP == 2 || NP == 4, "producer count");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TileWalk walk;
+    walk.init(p.tiles_m, p.tiles_n);
+    if (walk.my_tiles == 0) return;
+    if (wave < Cfg::NC) {
+        ws_consumer<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
+    } else {
+        // the producer index is a template argument: which DMA instructions a producer issues
+        // is then fixed at compile time (no branches in its loop)
+        const int pr = wave - Cfg::NC;
+        if (pr == 0) ws_producer<Cfg, NP, 0>(p, walk, smem, smem_base, lane);
+        else if (pr == 1) ws_producer<Cfg, NP, 1>(p, walk, smem, smem_base, lane);
+        else if (NP > 2 && pr == 2) ws_producer<Cfg, NP, (NP > 2 ? 2 : 0)>(p, walk, smem, smem_base, lane);
+        else if (NP > 2) ws_producer<Cfg, NP, (NP > 2 ? 3 : 0)>(p, walk, smem, smem_base, lane);
+    }
+}
+
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT>
+static hipError_t launch_ws(const SpmmParams& p, hipStream_t stream) {
+    using Cfg = WsCfg<WM, WN, NS, NP>;
+    constexpr int lds = Cfg::LDS_BYTES;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static bool attr_set = false;
+    static int cus = 0;
+    auto kern = spmm_ws_kernel<WM, WN, NS, NP, OUT_LAYOUT>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        int dev = 0;
+        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int per_cu = (160 * 1024) / lds;
+    const int tiles = p.tiles_m * p.tiles_n;
+    int grid = cus * per_cu;
+    grid = (grid / 8) * 8;
+    const int need = ((tiles + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    if (grid < 8) grid = 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::THREADS), lds, stream, p);
+    return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------
@@ -330,12 +1277,60 @@ const char* spmm_variant_name(int variant) {
     switch (variant) {
         case SPMM_VARIANT_128x128: return "smfmac16x16x64_wg256_tile128x128";
         case SPMM_VARIANT_64x256: return "smfmac16x16x64_wg256_tile64x256";
+        case SPMM_VARIANT_P128x128_S4: return "smfmac16x16x64_ldsdirect_tile128x128_4stage";
+        case SPMM_VARIANT_P128x128_S3: return "smfmac16x16x64_ldsdirect_tile128x128_3stage";
+        case SPMM_VARIANT_P64x256_S2: return "smfmac16x16x64_ldsdirect_tile64x256_2stage";
+        case SPMM_VARIANT_P64x256_S3: return "smfmac16x16x64_ldsdirect_tile64x256_3stage";
+        case SPMM_VARIANT_P128x128_S6: return "smfmac16x16x64_ldsdirect_tile128x128_6stage";
+        case SPMM_VARIANT_P64x256_S4: return "smfmac16x16x64_ldsdirect_tile64x256_4stage";
+        case SPMM_VARIANT_R128x128_S4: return "smfmac16x16x64_persistent_tile128x128_4stage";
+        case SPMM_VARIANT_R128x128_S5: return "smfmac16x16x64_persistent_tile128x128_5stage";
+        case SPMM_VARIANT_R128x128_S2: return "smfmac16x16x64_persistent_tile128x128_2stage";
+        case SPMM_VARIANT_R64x256_S3: return "smfmac16x16x64_persistent_tile64x256_3stage";
+        case SPMM_VARIANT_R64x256_S4: return "smfmac16x16x64_persistent_tile64x256_4stage";
+        case SPMM_VARIANT_W128x128_S5: return "smfmac16x16x64_warpspec_tile128x128_5stage";
+        case SPMM_VARIANT_W128x128_S3: return "smfmac16x16x64_warpspec_tile128x128_3stage";
+        case SPMM_VARIANT_W128x128_S2: return "smfmac16x16x64_warpspec_tile128x128_2stage";
+        case SPMM_VARIANT_W128x256_S3: return "smfmac16x16x64_warpspec_tile128x256_3stage";
+        case SPMM_VARIANT_W64x256_S2: return "smfmac16x16x64_warpspec_tile64x256_2stage";
+        case SPMM_VARIANT_W64x256_S3: return "smfmac16x16x64_warpspec_tile64x256_3stage";
         default: return nullptr;
     }
 }
 
-int spmm_variant_bm(int variant) { return variant == SPMM_VARIANT_128x128 ? 128 : variant == SPMM_VARIANT_64x256 ? 64 : 0; }
-int spmm_variant_bn(int variant) { return variant == SPMM_VARIANT_128x128 ? 128 : variant == SPMM_VARIANT_64x256 ? 256 : 0; }
+// LDS bytes the variant needs for S k-steps (pipelined variants keep the row table in LDS)
+int spmm_variant_lds(int variant, int S) {
+    switch (variant) {
+        case SPMM_VARIANT_P128x128_S4: return 4 * (64 * 128 * 2 + 2 * APACK_BLOCK) + S * 256;
+        case SPMM_VARIANT_P128x128_S3: return 3 * (64 * 128 * 2 + 2 * APACK_BLOCK) + S * 256;
+        case SPMM_VARIANT_P128x128_S6: return 6 * (64 * 128 * 2 + 2 * APACK_BLOCK) + S * 256;
+        case SPMM_VARIANT_P64x256_S2: return 2 * (64 * 256 * 2 + APACK_BLOCK) + S * 256;
+        case SPMM_VARIANT_P64x256_S3: return 3 * (64 * 256 * 2 + APACK_BLOCK) + S * 256;
+        case SPMM_VARIANT_P64x256_S4: return 4 * (64 * 256 * 2 + APACK_BLOCK) + S * 256;
+        default: return 0;
+    }
+}
+
+int spmm_variant_bm(int variant) {
+    switch (variant) {
+        case SPMM_VARIANT_128x128: case SPMM_VARIANT_P128x128_S4: case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P128x128_S6:
+        case SPMM_VARIANT_R128x128_S4: case SPMM_VARIANT_R128x128_S5: case SPMM_VARIANT_R128x128_S2:
+        case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2: case SPMM_VARIANT_W128x256_S3: return 128;
+        case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3:
+        case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 64;
+        default: return 0;
+    }
+}
+int spmm_variant_bn(int variant) {
+    switch (variant) {
+        case SPMM_VARIANT_128x128: case SPMM_VARIANT_P128x128_S4: case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P128x128_S6:
+        case SPMM_VARIANT_R128x128_S4: case SPMM_VARIANT_R128x128_S5: case SPMM_VARIANT_R128x128_S2:
+        case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2: return 128;
+        case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_W128x256_S3:
+        case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 256;
+        default: return 0;
+    }
+}
 
 hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStream_t stream) {
     if (variant == SPMM_VARIANT_128x128) {
@@ -346,16 +1341,47 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_variant<1, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
                                                    : launch_variant<1, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
     }
+#define SPATHA_PIPE_CASE(ID, WM_, WN_, NS_)                                                             \
+    if (variant == ID)                                                                                  \
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_pipe<WM_, WN_, NS_, SPATHA_OUT_TRANSPOSED>(p, stream) \
+                                                   : launch_pipe<WM_, WN_, NS_, SPATHA_OUT_ROW_MAJOR>(p, stream);
+    SPATHA_PIPE_CASE(SPMM_VARIANT_P128x128_S4, 2, 2, 4)
+    SPATHA_PIPE_CASE(SPMM_VARIANT_P128x128_S3, 2, 2, 3)
+    SPATHA_PIPE_CASE(SPMM_VARIANT_P64x256_S2, 1, 4, 2)
+    SPATHA_PIPE_CASE(SPMM_VARIANT_P64x256_S3, 1, 4, 3)
+    SPATHA_PIPE_CASE(SPMM_VARIANT_P128x128_S6, 2, 2, 6)
+    SPATHA_PIPE_CASE(SPMM_VARIANT_P64x256_S4, 1, 4, 4)
+#undef SPATHA_PIPE_CASE
+#define SPATHA_PERSIST_CASE(ID, WM_, WN_, NS_)                                                          \
+    if (variant == ID)                                                                                  \
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_persist<WM_, WN_, NS_, SPATHA_OUT_TRANSPOSED>(p, stream) \
+                                                   : launch_persist<WM_, WN_, NS_, SPATHA_OUT_ROW_MAJOR>(p, stream);
+    SPATHA_PERSIST_CASE(SPMM_VARIANT_R128x128_S4, 2, 2, 4)
+    SPATHA_PERSIST_CASE(SPMM_VARIANT_R128x128_S5, 2, 2, 5)
+    SPATHA_PERSIST_CASE(SPMM_VARIANT_R128x128_S2, 2, 2, 2)
+    SPATHA_PERSIST_CASE(SPMM_VARIANT_R64x256_S3, 1, 4, 3)
+    SPATHA_PERSIST_CASE(SPMM_VARIANT_R64x256_S4, 1, 4, 4)
+#undef SPATHA_PERSIST_CASE
+#define SPATHA_WS_CASE(ID, WM_, WN_, NS_, NP_)                                                          \
+    if (variant == ID)                                                                                  \
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ws<WM_, WN_, NS_, NP_, SPATHA_OUT_TRANSPOSED>(p, stream) \
+                                                   : launch_ws<WM_, WN_, NS_, NP_, SPATHA_OUT_ROW_MAJOR>(p, stream);
+    SPATHA_WS_CASE(SPMM_VARIANT_W128x128_S5, 2, 2, 5, 4)
+    SPATHA_WS_CASE(SPMM_VARIANT_W128x128_S3, 2, 2, 3, 4)
+    SPATHA_WS_CASE(SPMM_VARIANT_W128x128_S2, 2, 2, 2, 4)
+    SPATHA_WS_CASE(SPMM_VARIANT_W128x256_S3, 2, 4, 3, 4)
+    SPATHA_WS_CASE(SPMM_VARIANT_W64x256_S2, 1, 4, 2, 2)
+    SPATHA_WS_CASE(SPMM_VARIANT_W64x256_S3, 1, 4, 3, 2)
+#undef SPATHA_WS_CASE
     return hipErrorInvalidValue;
 }
 
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
-                       int m, int v, int ksp, int S, uint16_t* apack, uint32_t* ipack, uint32_t* rowtab,
-                       hipStream_t stream) {
+                       int m, int v, int ksp, int S, uint16_t* apack, uint32_t* rowtab, hipStream_t stream) {
     int64_t total_a = (int64_t)(rows / 64) * S * 256;
     int blocks_a = (int)((total_a + 255) / 256);
     if (blocks_a > 65535 * 8) blocks_a = 65535 * 8;
-    hipLaunchKernelGGL(pack_a_kernel, dim3(blocks_a), dim3(256), 0, stream, values, metadata, rows, ksp, S, apack, ipack);
+    hipLaunchKernelGGL(pack_a_kernel, dim3(blocks_a), dim3(256), 0, stream, values, metadata, rows, ksp, S, apack);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     int64_t total_r = (int64_t)(rows / v) * S * 64;

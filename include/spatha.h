@@ -144,6 +144,9 @@ int spatha_spmm_plan_destroy(spatha_spmm_plan* plan);
 int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
                     uint16_t* out_dev, int out_layout, int variant, void* stream);
 
+/* Kernel variants are numbered 1 .. spatha_spmm_num_variants() - 1; 0 selects automatically. */
+int spatha_spmm_num_variants(void);
+
 /* Name / tile shape of the kernel `variant` (or of the automatic choice for N
  * when variant == 0) would use, for logs; returns NULL if unsupported. */
 const char* spatha_spmm_kernel_name(const spatha_spmm_plan* plan, int N, int out_layout, int variant);

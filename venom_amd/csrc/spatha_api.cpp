@@ -31,19 +31,45 @@ inline int hip_fail(hipError_t e) {
     return SPATHA_ERR_HIP;
 }
 
+bool variant_ok(const spatha_spmm_plan* plan, int N, int variant) {
+    using namespace spatha;
+    if (variant <= 0 || variant >= SPMM_VARIANT_COUNT) return false;
+    const int bm = spmm_variant_bm(variant);
+    if (bm == 0 || plan->geo.v % bm != 0) return false;
+    if (spmm_variant_lds(variant, plan->S) > 160 * 1024) return false;      // row table kept in LDS
+    if (variant >= SPMM_VARIANT_R128x128_S4) {
+        // buffer-descriptor kernels address B, the packed operands and the row table with 32-bit offsets
+        const uint64_t bb = (uint64_t)plan->geo.cols * (uint64_t)N * 2u;
+        if (bb >= 0xE0000000ull || plan->apack_bytes >= 0xE0000000ull || plan->rowtab_bytes >= 0xE0000000ull) return false;
+    }
+    return true;
+}
+
+// Kernel choice.  V a multiple of 128: producer/consumer kernel on 128-row tiles, 256 columns
+// wide when that still gives every CU at least two tiles, else 128 wide.  Otherwise (V a
+// multiple of 64 only) the 64 x 256 tile whose B rows are gathered per 64-row block.
 int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
     using namespace spatha;
-    (void)N;
+    if (variant != SPMM_VARIANT_AUTO) return variant_ok(plan, N, variant) ? variant : -1;
     const int v = plan->geo.v;
-    if (variant == SPMM_VARIANT_AUTO) {
-        if (v % 128 == 0) return SPMM_VARIANT_128x128;
-        if (v % 64 == 0) return SPMM_VARIANT_64x256;
+    int order[4] = {0, 0, 0, 0};
+    if (v % 128 == 0) {
+        const int64_t wide_tiles = (int64_t)(plan->geo.rows / 128) * ((N + 255) / 256);
+        order[0] = wide_tiles >= 512 ? SPMM_VARIANT_W128x256_S3 : SPMM_VARIANT_W128x128_S3;
+        order[1] = SPMM_VARIANT_W128x128_S3;
+        order[2] = SPMM_VARIANT_P128x128_S3;
+        order[3] = SPMM_VARIANT_128x128;
+    } else if (v % 64 == 0) {
+        order[0] = SPMM_VARIANT_P64x256_S2;
+        order[1] = SPMM_VARIANT_W64x256_S3;
+        order[2] = SPMM_VARIANT_64x256;
+        order[3] = SPMM_VARIANT_64x256;
+    } else {
         return -1;
     }
-    if (variant < 0 || variant >= SPMM_VARIANT_COUNT) return -1;
-    if (v % spmm_variant_bm(variant) != 0) return -1;
-    if (spmm_variant_lds(variant, plan->S) > 160 * 1024) return -1;
-    return variant;
+    for (int i = 0; i < 4; i++)
+        if (variant_ok(plan, N, order[i])) return order[i];
+    return -1;
 }
 }  // namespace
 
@@ -171,16 +197,15 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
     const int bm = spatha::spmm_variant_bm(var), bn = spatha::spmm_variant_bn(var);
     p.tiles_m = plan->geo.rows / bm;
     p.tiles_n = (N + bn - 1) / bn;
-    {
-        const uint64_t bb = (uint64_t)plan->geo.cols * (uint64_t)N * 2u;
-        const bool fits32 = bb < 0xE0000000ull && plan->apack_bytes < 0xE0000000ull && plan->rowtab_bytes < 0xE0000000ull;
-        if (!fits32 && var >= spatha::SPMM_VARIANT_R128x128_S4) return SPATHA_ERR_UNSUPPORTED;
-        p.b_bytes = (uint32_t)bb; p.apack_bytes = (uint32_t)plan->apack_bytes; p.rowtab_bytes = (uint32_t)plan->rowtab_bytes;
-    }
+    p.b_bytes = (uint32_t)((uint64_t)plan->geo.cols * (uint64_t)N * 2u);     // only read by variants that passed variant_ok
+    p.apack_bytes = (uint32_t)plan->apack_bytes;
+    p.rowtab_bytes = (uint32_t)plan->rowtab_bytes;
     { const char* d = std::getenv("SPATHA_DEBUG_KNOBS"); p.debug = d ? std::atoi(d) : 0; }
     hipError_t e = spatha::launch_spmm(var, out_layout, p, (hipStream_t)stream);
     return e == hipSuccess ? SPATHA_OK : hip_fail(e);
 }
+
+int spatha_spmm_num_variants(void) { return spatha::SPMM_VARIANT_COUNT; }
 
 const char* spatha_spmm_kernel_name(const spatha_spmm_plan* plan, int N, int out_layout, int variant) {
     (void)out_layout;

@@ -1307,6 +1307,18 @@ int spmm_variant_lds(int variant, int S) {
         case SPMM_VARIANT_P64x256_S2: return 2 * (64 * 256 * 2 + APACK_BLOCK) + S * 256;
         case SPMM_VARIANT_P64x256_S3: return 3 * (64 * 256 * 2 + APACK_BLOCK) + S * 256;
         case SPMM_VARIANT_P64x256_S4: return 4 * (64 * 256 * 2 + APACK_BLOCK) + S * 256;
+        case SPMM_VARIANT_R128x128_S4: return PersistCfg<2, 2, 4>::LDS_BYTES;
+        case SPMM_VARIANT_R128x128_S5: return PersistCfg<2, 2, 5>::LDS_BYTES;
+        case SPMM_VARIANT_R128x128_S2: return PersistCfg<2, 2, 2>::LDS_BYTES;
+        case SPMM_VARIANT_R64x256_S3: return PersistCfg<1, 4, 3>::LDS_BYTES;
+        case SPMM_VARIANT_R64x256_S4: return PersistCfg<1, 4, 4>::LDS_BYTES;
+        case SPMM_VARIANT_W128x128_S5: return WsCfg<2, 2, 5, 4>::LDS_BYTES;
+        case SPMM_VARIANT_W128x128_S3: return WsCfg<2, 2, 3, 4>::LDS_BYTES;
+        case SPMM_VARIANT_W128x128_S2: return WsCfg<2, 2, 2, 4>::LDS_BYTES;
+        case SPMM_VARIANT_W128x256_S3: return WsCfg<2, 4, 3, 4>::LDS_BYTES;
+        case SPMM_VARIANT_W64x256_S2: return WsCfg<1, 4, 2, 2>::LDS_BYTES;
+        case SPMM_VARIANT_W64x256_S3: return WsCfg<1, 4, 3, 2>::LDS_BYTES;
+        case SPMM_VARIANT_128x128: case SPMM_VARIANT_64x256: return 1;
         default: return 0;
     }
 }

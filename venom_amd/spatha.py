@@ -14,6 +14,11 @@ OUT_ROW_MAJOR = 0
 OUT_TRANSPOSED = 1
 
 
+def num_variants():
+    """Kernel variants are numbered 1 .. num_variants() - 1; 0 selects automatically."""
+    return int(_lib.lib().spatha_spmm_num_variants())
+
+
 def _stream_ptr(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 

@@ -142,27 +142,38 @@ def main():
         import oracle
 
         threads = min(oracle.num_threads(), os.cpu_count() or 1)
-        n_sample = min(N, 1024)
-        Bs = w["B"][:, :n_sample].contiguous().cpu().numpy()
+        # whole workload, all cores: the oracle's compressed-form SpMM (fp32 accumulate, fp16 out)
+        Bh = w["B"].cpu().numpy()
+        reps = 0
         t0 = time.perf_counter()
-        ref = oracle.spmm(w["vals"], w["meta"], w["columns"], rows, cols, 2, m, v, Bs, threads=threads)
-        t_spmm = time.perf_counter() - t0
+        while True:
+            ref = oracle.spmm(w["vals"], w["meta"], w["columns"], rows, cols, 2, m, v, Bh, threads=threads)
+            reps += 1
+            if time.perf_counter() - t0 > 4.0 or reps >= 20:
+                break
+        t_spmm = (time.perf_counter() - t0) / reps
+        # one thread on an eighth of the columns
+        n1 = max(8, (N // 8) // 8 * 8)
+        t0 = time.perf_counter()
+        oracle.spmm(w["vals"], w["meta"], w["columns"], rows, cols, 2, m, v, np.ascontiguousarray(Bh[:, :n1]), threads=1)
+        t_one = (time.perf_counter() - t0) * (N / n1)
         # host format conversion of the same matrix, the reference's single-threaded way: decode + encode
         t0 = time.perf_counter()
         dense = oracle.decode(w["vals"], w["meta"], w["columns"], rows, cols, 2, m, v)
         oracle.encode(dense, w["columns"], 2, m, v)
         t_fmt = time.perf_counter() - t0
-        got = w["C"][:, :n_sample].cpu().numpy()
+        got = w["C"].cpu().numpy()
         err = float(np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64)) /
                            np.maximum(np.abs(ref.astype(np.float64)), 1.0)))
         out["cpu_baseline"] = {
-            "value": round(2.0 * rows * cols * n_sample / t_spmm / 1e12, 5),
+            "value": round(flops_dense / t_spmm / 1e12, 5),
             "unit": "TFLOPS (dense-equivalent)",
             "cores": threads,
             "kind": "port",
-            "sample": "oracle SpMM (compressed form, fp32 accumulate, OpenMP) on the first %d of %d columns of B: %.2f s; "
-                      "host format decode+encode of A, 1 thread: %.3f s; max rel err GPU vs oracle on the sample %.2e"
-                      % (n_sample, N, t_spmm, t_fmt, err),
+            "sample": "oracle SpMM (compressed form, fp32 accumulate, OpenMP, %d threads) on the whole workload, mean of %d runs: "
+                      "%.3f s per SpMM; 1 thread (timed on %d of %d columns, scaled): %.2f s; host format decode+encode of A, "
+                      "1 thread: %.3f s; max rel err GPU vs oracle over all of C: %.2e"
+                      % (threads, reps, t_spmm, n1, N, t_one, t_fmt, err),
         }
     print(json.dumps(out))
 

@@ -1,0 +1,77 @@
+"""End-to-end Python side: sparsifier, SrNMTensor, the Linear replacement."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from venom_amd.grouped_nmv_tensor import SrNMTensor, nm_vector_mask_sparsify
+
+
+def test_sparsify_and_tensor_on_cpu():
+    torch.manual_seed(0)
+    rows, cols, n, m, v = 128, 96, 2, 8, 64
+    w = torch.randn(rows, cols)
+    masks, columns = nm_vector_mask_sparsify(w, n, m, v)
+    omasks, ocols = oracle.select_columns(np.abs(w.numpy()), n, m, v)
+    assert np.array_equal(masks.numpy(), omasks) and np.array_equal(columns.numpy(), ocols)
+    t = SrNMTensor(n, m, v, w * masks, masks, columns, "cpu")
+    assert t.values.dtype == torch.float16 and t.metadata.dtype == torch.int32 and t.columns.dtype == torch.int32
+    assert (t.nrows, t.ncols, t.nnz) == (rows, cols, rows * 32)      # Ksp = ROUND_UP(12 * 2, 16) = 32
+    ovals, ometa = oracle.encode((w * masks).numpy(), ocols.astype(np.uint32), n, m, v, mask=omasks)
+    assert np.array_equal(t.values.numpy(), ovals.astype(np.float16))
+    assert np.array_equal(t.metadata.numpy().view(np.uint32), ometa)
+    assert torch.equal(t.to_dense(), (w * masks).half())
+
+
+def test_fixed_pattern_sparsifier_shapes():
+    from venom_amd.bert import NMVectorSparsifier
+
+    w = torch.randn(128, 64)
+    t = NMVectorSparsifier(2, 8, 64)(w).wrapped_tensor
+    kept = torch.zeros(8)
+    kept[0] = kept[2] = 1
+    want = (w.reshape(128, 8, 8) * kept).reshape(128, 64).half()
+    assert torch.equal(t.to_dense(), want)
+
+
+@pytest.mark.gpu
+def test_srnm_linear_matches_masked_dense_linear(gpu):
+    from venom_amd.bert import SrnmSpmm
+
+    torch.manual_seed(1)
+    lin = torch.nn.Linear(256, 128).to(gpu).half()
+    x = torch.randn(4, 24, 256, device=gpu).half()
+    for magnitude in (False, True):
+        sp = SrnmSpmm(lin, 2, 8, 64, magnitude=magnitude)
+        y = sp(x)
+        assert y.shape == (4, 24, 128)
+        wd = SrNMTensor.to_dense(type("T", (), dict(values=sp.values, metadata=sp.metadata, columns=sp.columns, nrows=128,
+                                                      ncols=256, n=2, m=8, tileM=64, device=gpu))())
+        ref = x.float().reshape(-1, 256) @ wd.float().T
+        ref = ref.half().float() + lin.bias.float()
+        err = (y.float().reshape(-1, 128) - ref).abs() / ref.abs().clamp(min=1.0)
+        assert err.max().item() <= 1e-2
+
+
+@pytest.mark.gpu
+def test_bert_encoder_swap_runs_and_tracks_masked_dense(gpu):
+    from venom_amd.bert import build_bert_large, linear_to_spmm, SrnmSpmm
+
+    torch.set_grad_enabled(False)
+    model = build_bert_large(layers=2).to(gpu).half()
+    ids = torch.randint(0, 30522, (2, 64), device=gpu)
+    sparse = linear_to_spmm(build_bert_large(layers=2).to(gpu).half(), 2, 8, 64)
+    swapped = [n for n, mod in sparse.named_modules() if isinstance(mod, SrnmSpmm)]
+    assert len(swapped) == 2 * 6 and all("encoder.layer" in n for n in swapped)
+    assert isinstance(sparse.pooler.dense, torch.nn.Linear)
+    # a dense model whose encoder weights carry the same mask must give the same activations
+    for name, mod in model.named_modules():
+        if isinstance(mod, torch.nn.Linear) and "encoder.layer" in name:
+            w = mod.weight
+            kept = torch.zeros(8, device=gpu, dtype=w.dtype)
+            kept[0] = kept[2] = 1
+            mod.weight.copy_((w.reshape(w.shape[0], -1, 8) * kept).reshape(w.shape))
+    a = sparse(ids).last_hidden_state.float()
+    b = model(ids).last_hidden_state.float()
+    assert torch.isfinite(a).all()
+    assert (a - b).abs().max().item() <= 5e-2

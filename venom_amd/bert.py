@@ -1,0 +1,138 @@
+"""BERT-large inference with every encoder Linear stored in V:N:M and run through `spatha.spmm`.
+
+Counterpart of the reference harness end2end/bert_pytorch.py (`NMVectorSparsifier` :56-83,
+`SrnmSpmm` :109-136, `linear_to_spmm` :155-167, timing :169-219).  Differences, on purpose:
+the model is built from a local `BertConfig` with random weights (no hub download), only
+`encoder.layer.*` Linears are swapped (the reference also swaps `pooler.dense`, whose 32-token
+input is narrower than its kernel's tile), and the STEN wrapper is replaced by a two-method
+stand-in because only `wrapped_from_dense(...)` / `.wrapped_tensor` are used.
+
+    python -m venom_amd.bert -m 8 -n 2 -v 64 [--layers 24] [--magnitude] [--repeats 30]
+prints `algo,n,m,v,mean_ms,median_ms,std_ms,len` rows for the dense and the V:N:M model."""
+import argparse
+import statistics
+import timeit
+
+import torch
+
+from . import spatha
+from .grouped_nmv_tensor import SrNMTensor, nm_vector_mask_sparsify
+
+
+class SparseTensorWrapper:
+    """The part of sten.SparseTensorWrapper the harness uses."""
+
+    def __init__(self, wrapped_tensor, dense, grad_fmt=None):
+        self.wrapped_tensor = wrapped_tensor
+        self.dense_shape = tuple(dense.shape)
+        self.grad_fmt = grad_fmt
+
+    @staticmethod
+    def wrapped_from_dense(wrapped_tensor, dense, grad_fmt=None):
+        return SparseTensorWrapper(wrapped_tensor, dense, grad_fmt)
+
+
+class NMVectorSparsifier:
+    """magnitude=False: the reference harness's pattern (column-loc {0,1,2,3} in every group,
+    mask [1,0,1,0,0,...]); magnitude=True: `nm_vector_mask_sparsify`."""
+
+    def __init__(self, n, m, tileM, magnitude=False):
+        self.n, self.m, self.tileM, self.magnitude = n, m, tileM, magnitude
+
+    def __call__(self, tensor, grad_fmt=None):
+        nrows, ncols = tensor.shape
+        if self.magnitude:
+            mask, columns = nm_vector_mask_sparsify(tensor, self.n, self.m, self.tileM)
+        else:
+            columns = torch.arange(4, dtype=torch.int32).repeat(nrows // self.tileM, ncols // self.m)
+            pat = torch.zeros(self.m, dtype=torch.int32)
+            pat[0] = 1
+            pat[2] = 1
+            mask = pat.repeat(nrows, ncols // self.m)
+        return SparseTensorWrapper.wrapped_from_dense(
+            SrNMTensor(self.n, self.m, self.tileM, tensor, mask, columns, tensor.device), tensor, grad_fmt)
+
+
+class SrnmSpmm(torch.nn.Module):
+    """Drop-in for nn.Linear: y = x W^T + b with W in V:N:M."""
+
+    def __init__(self, original, n, m, v, magnitude=False):
+        super().__init__()
+        self.n, self.m, self.v = n, m, v
+        self.bias = original.bias
+        w = NMVectorSparsifier(n, m, v, magnitude)(original.weight).wrapped_tensor
+        self.values = torch.nn.Parameter(w.values, requires_grad=False)
+        self.columns = w.columns
+        self.metadata = w.metadata
+        self.nrows_sp, self.ncols_sp, self.nnz = w.nrows, w.ncols, w.nnz
+
+    def forward(self, input):
+        flat = torch.flatten(input, start_dim=0, end_dim=-2)          # [tokens, in]
+        rhs = flat.T.contiguous()                                     # [in, tokens], as the operator expects
+        bias = self.bias if self.bias is not None else torch.zeros(self.nrows_sp, dtype=rhs.dtype, device=rhs.device)
+        out = spatha.spmm(self.metadata, self.columns, self.values, rhs, bias, self.nrows_sp, self.ncols_sp,
+                          rhs.shape[1], self.v, self.n, self.m, self.nnz, 0, 32, 4)   # [tokens, out]
+        return out.reshape(*input.shape[:-1], -1)
+
+
+def linear_to_spmm(mod, n, m, v, magnitude=False, prefix="", only=("encoder.layer",)):
+    """Replaces, in place, every nn.Linear whose qualified name contains one of `only`."""
+    for name, child in list(mod.named_children()):
+        full = prefix + "." + name if prefix else name
+        if isinstance(child, torch.nn.Linear) and any(tag in full for tag in only):
+            setattr(mod, name, SrnmSpmm(child, n, m, v, magnitude))
+        elif not isinstance(child, SrnmSpmm):
+            linear_to_spmm(child, n, m, v, magnitude, full, only)
+    return mod
+
+
+def report_time(name, data, number, n, m, v):
+    ds = [d / number * 1000 for d in data]
+    cfg = "%d,%d," % (n, m) if name == "n:m" else "0,0,"
+    std = statistics.stdev(ds) if len(ds) > 1 else 0.0
+    print("0," + cfg + "%d,%s,%s,%s,%d" % (v, statistics.mean(ds), statistics.median(ds), std, len(ds)), flush=True)
+    return statistics.mean(ds)
+
+
+def build_bert_large(layers=24, seed=0):
+    from transformers import BertConfig, BertModel
+
+    torch.manual_seed(seed)
+    cfg = BertConfig(hidden_size=1024, num_hidden_layers=layers, num_attention_heads=16, intermediate_size=4096,
+                     vocab_size=30522, max_position_embeddings=512)
+    return BertModel(cfg).eval()
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("-m", type=int, default=8)
+    ap.add_argument("-n", type=int, default=2)
+    ap.add_argument("-v", type=int, default=64)
+    ap.add_argument("--layers", type=int, default=24)
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--seq", type=int, default=512)
+    ap.add_argument("--repeats", type=int, default=30)
+    ap.add_argument("--magnitude", action="store_true", help="magnitude column selection instead of the fixed pattern")
+    args = ap.parse_args(argv)
+    torch.set_grad_enabled(False)
+    dev = torch.device("cuda:0")
+    dense_model = build_bert_large(args.layers).to(dev).half()
+    sparse_model = build_bert_large(args.layers)
+    sparse_model = linear_to_spmm(sparse_model.to(dev).half(), args.n, args.m, args.v, args.magnitude)
+    ids = torch.randint(0, 30522, (args.batch, args.seq), device=dev)
+
+    def run(model):
+        out = model(ids).last_hidden_state
+        torch.cuda.synchronize()
+        return out
+
+    run(sparse_model)
+    timeit.repeat(lambda: run(dense_model), repeat=5, number=1)
+    t_dense = report_time("dense", timeit.repeat(lambda: run(dense_model), repeat=args.repeats, number=1), 1, args.n, args.m, args.v)
+    timeit.repeat(lambda: run(sparse_model), repeat=5, number=1)
+    t_sparse = report_time("n:m", timeit.repeat(lambda: run(sparse_model), repeat=args.repeats, number=1), 1, args.n, args.m, args.v)
+    print("# dense %.2f ms, %d:%d:%d %.2f ms, speed-up %.2fx" % (t_dense, args.v, args.n, args.m, t_sparse, t_dense / t_sparse))
+
+
+if __name__ == "__main__":
+    main()

@@ -201,6 +201,7 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
     p.apack_bytes = (uint32_t)plan->apack_bytes;
     p.rowtab_bytes = (uint32_t)plan->rowtab_bytes;
     { const char* d = std::getenv("SPATHA_DEBUG_KNOBS"); p.debug = d ? std::atoi(d) : 0; }
+    { const char* d = std::getenv("SPATHA_SKEW"); p.skew = d ? std::atoi(d) : 0; }
     hipError_t e = spatha::launch_spmm(var, out_layout, p, (hipStream_t)stream);
     return e == hipSuccess ? SPATHA_OK : hip_fail(e);
 }

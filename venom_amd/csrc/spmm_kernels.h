@@ -20,6 +20,7 @@ struct SpmmParams {
     int rows, cols, N, S, v;
     uint32_t b_bytes, apack_bytes, rowtab_bytes;   // sizes for buffer descriptors (persistent kernels)
     int tiles_m, tiles_n;
+    int skew;                 // start-up skew between workgroups, in units of 1024 clocks (0 = none)
     int debug;                // development knobs (0 in production): 1 = skip B loads, 2 = skip C stores
 };
 
@@ -44,7 +45,11 @@ enum {
     SPMM_VARIANT_W128x256_S3 = 17,
     SPMM_VARIANT_W64x256_S2 = 18,
     SPMM_VARIANT_W64x256_S3 = 19,
-    SPMM_VARIANT_COUNT = 20
+    SPMM_VARIANT_D128x256_S3 = 20,  // wave-specialised + write-out deferred into the next tile
+    SPMM_VARIANT_D128x128_S3 = 21,
+    SPMM_VARIANT_D128x128_S5 = 22,
+    SPMM_VARIANT_D64x256_S3 = 23,
+    SPMM_VARIANT_COUNT = 24
 };
 
 const char* spmm_variant_name(int variant);

@@ -1200,7 +1200,145 @@ __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk&
     }
 }
 
-template <int WM, int WN, int NS, int NP, int OUT_LAYOUT>
+// ---- deferred write-out -------------------------------------------------------------------
+// A finished 64 x 64 wave tile is rounded to fp16 pairs (32 registers) and written one quarter
+// per k-step of the NEXT tile: the stores of a tile are then spread over the following tile's
+// matrix work instead of stalling every consumer on a burst that all CUs issue together.
+__device__ __forceinline__ uint32_t pack_half2(float a, float b) {
+    half2_t h = {(_Float16)a, (_Float16)b};
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// rows 4*MB..4*MB+3 (+16*ib) of the pending wave tile -> row-major C through the wave's LDS slab
+template <int MB, int EPI_PITCH>
+__device__ __forceinline__ void store_slab_row_major(const uint32_t (&pend)[4][4][2], char* stg, uint16_t* C, int64_t row_base,
+                                                     int col_base, int N, int lane, bool enable) {
+    const int j16 = lane & 15, ib = lane >> 4;
+#pragma unroll
+    for (int rp = 0; rp < 2; rp++)
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+            uint32_t w = pend[MB][nb][rp];
+            asm volatile("" : "+v"(w));      // keeps the >> 16 below from being hoisted out of the k-loop (32 registers)
+            *(uint16_t*)(stg + ((2 * rp) * 4 + ib) * EPI_PITCH + (nb * 16 + j16) * 2) = (uint16_t)w;
+            *(uint16_t*)(stg + ((2 * rp + 1) * 4 + ib) * EPI_PITCH + (nb * 16 + j16) * 2) = (uint16_t)(w >> 16);
+        }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < 2; it++) {
+        const int Lr = it * 8 + (lane >> 3), ch = lane & 7;
+        const int row = 16 * (Lr & 3) + 4 * MB + (Lr >> 2);
+        const int col = col_base + ch * 8;
+        u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
+        if (col < N && enable) *(u32x4*)(C + (row_base + row) * N + col) = v;
+    }
+    __builtin_amdgcn_wave_barrier();
+}
+
+// column block NB of the pending wave tile -> transposed output (32 contiguous bytes per lane)
+template <int NB>
+__device__ __forceinline__ void store_block_transposed(const uint32_t (&pend)[4][4][2], uint16_t* C, int64_t row0, int col,
+                                                       int rows_total, int N, bool enable) {
+    u32x4 lo = {pend[0][NB][0], pend[0][NB][1], pend[1][NB][0], pend[1][NB][1]};
+    u32x4 hi = {pend[2][NB][0], pend[2][NB][1], pend[3][NB][0], pend[3][NB][1]};
+    if (col < N && enable) {
+        uint16_t* dst = C + (int64_t)col * rows_total + row0;
+        *(u32x4*)dst = lo;
+        *(u32x4*)(dst + 8) = hi;
+    }
+}
+
+template <class Cfg, int WN, int OUT_LAYOUT>
+__device__ __forceinline__ void ws_consumer_deferred(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int EPI_PITCH = Cfg::EPI_PITCH;
+    const int S = p.S, N = p.N;
+    const int wm = wave / WN, wn = wave - wm * WN;
+    float4_t acc[4][4];
+    uint32_t pend[4][4][2];         // previous tile: [mb][nb][r / 2] = fp16 pair (r even | r odd << 16)
+    const int li = lane & 15, kb = lane >> 4;
+    const int rrow = kb * 4 + (li >> 2);
+    const int sw = rrow & 7;
+    int tr_off[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int ch = (wn * 8 + nb * 2 + ((li & 3) >> 1)) ^ (sw << 1);
+        tr_off[nb] = rrow * ROW_BYTES + ch * 16 + (li & 1) * 8;
+    }
+    const int a_off = B_BYTES + wm * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + wm * APACK_BLOCK + 4096 + lane * 4;
+    const int j16 = lane & 15, ib = lane >> 4;
+    char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
+    const bool stores_on = !(p.debug & 2);
+
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    int pm0 = 0, pn0 = 0;           // origin of the tile held in pend
+    bool have_pend = false;
+    uint32_t c_stage = 0;
+    auto flush_part = [&](int part) {
+        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+            const int64_t row0 = (int64_t)pm0 + wm * 64 + ib * 16;
+            const int colb = pn0 + wn * 64 + j16;
+            if (part == 0) store_block_transposed<0>(pend, p.C, row0, colb, p.rows, N, stores_on);
+            else if (part == 1) store_block_transposed<1>(pend, p.C, row0, colb + 16, p.rows, N, stores_on);
+            else if (part == 2) store_block_transposed<2>(pend, p.C, row0, colb + 32, p.rows, N, stores_on);
+            else store_block_transposed<3>(pend, p.C, row0, colb + 48, p.rows, N, stores_on);
+        } else {
+            const int64_t rb = (int64_t)pm0 + wm * 64;
+            const int cb = pn0 + wn * 64;
+            if (part == 0) store_slab_row_major<0, EPI_PITCH>(pend, stg, p.C, rb, cb, N, lane, stores_on);
+            else if (part == 1) store_slab_row_major<1, EPI_PITCH>(pend, stg, p.C, rb, cb, N, lane, stores_on);
+            else if (part == 2) store_slab_row_major<2, EPI_PITCH>(pend, stg, p.C, rb, cb, N, lane, stores_on);
+            else store_slab_row_major<3, EPI_PITCH>(pend, stg, p.C, rb, cb, N, lane, stores_on);
+        }
+    };
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            __syncthreads();
+            if (!(p.debug & 16)) mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {});
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+            if (have_pend && c_step < 4 && !(p.debug & 4)) flush_part(c_step);
+        }
+        // a k-loop shorter than four steps leaves parts of the previous tile unwritten
+        if (have_pend && !(p.debug & 4))
+            for (int part = S; part < 4; part++) flush_part(part);
+        const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+        const bool with_bias = (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) && p.bias;
+        u32x4 bias_lo = {0, 0, 0, 0}, bias_hi = {0, 0, 0, 0};
+        if (with_bias) {
+            const int64_t row0 = (int64_t)cm0 + wm * 64 + ib * 16;
+            bias_lo = *(const u32x4*)(p.bias + row0);
+            bias_hi = *(const u32x4*)(p.bias + row0 + 8);
+        }
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++)
+#pragma unroll
+                for (int rp = 0; rp < 2; rp++) {
+                    uint32_t w = pack_half2(acc[mb][nb][2 * rp], acc[mb][nb][2 * rp + 1]);
+                    if (with_bias) {
+                        const uint32_t bw = (mb < 2) ? bias_lo[mb * 2 + rp] : bias_hi[(mb - 2) * 2 + rp];
+                        const half2_t sum = __builtin_bit_cast(half2_t, w) + __builtin_bit_cast(half2_t, bw);
+                        w = __builtin_bit_cast(uint32_t, sum);
+                    }
+                    pend[mb][nb][rp] = w;
+                }
+        pm0 = cm0;
+        pn0 = cn0;
+        have_pend = true;
+        walk.next(c_tm, c_tn);
+    }
+    if (have_pend && !(p.debug & 4))
+        for (int part = 0; part < 4; part++) flush_part(part);
+}
+
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false>
 __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams p) {
     using Cfg = WsCfg<WM, WN, NS, NP>;
     static_assert(NP == 2 || NP == 4, "producer count");
@@ -1211,8 +1349,15 @@ __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams
     TileWalk walk;
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
+    // Workgroups of one XCD start up to 7 * skew apart, so that tiles do not all finish (and
+    // hit HBM with their stores) at the same moment on every CU.
+    if (p.skew > 0) {
+        const int units = ((blockIdx.x >> 3) & 7) * p.skew;
+        for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);      // 16 * 64 clocks
+    }
     if (wave < Cfg::NC) {
-        ws_consumer<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
+        if (DEFER) ws_consumer_deferred<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
+        else ws_consumer<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
     } else {
         // the producer index is a template argument: which DMA instructions a producer issues
         // is then fixed at compile time (no branches in its loop)
@@ -1224,14 +1369,14 @@ __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams
     }
 }
 
-template <int WM, int WN, int NS, int NP, int OUT_LAYOUT>
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false>
 static hipError_t launch_ws(const SpmmParams& p, hipStream_t stream) {
     using Cfg = WsCfg<WM, WN, NS, NP>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static bool attr_set = false;
     static int cus = 0;
-    auto kern = spmm_ws_kernel<WM, WN, NS, NP, OUT_LAYOUT>;
+    auto kern = spmm_ws_kernel<WM, WN, NS, NP, OUT_LAYOUT, DEFER>;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
@@ -1294,6 +1439,10 @@ const char* spmm_variant_name(int variant) {
         case SPMM_VARIANT_W128x256_S3: return "smfmac16x16x64_warpspec_tile128x256_3stage";
         case SPMM_VARIANT_W64x256_S2: return "smfmac16x16x64_warpspec_tile64x256_2stage";
         case SPMM_VARIANT_W64x256_S3: return "smfmac16x16x64_warpspec_tile64x256_3stage";
+        case SPMM_VARIANT_D128x256_S3: return "smfmac16x16x64_warpspec_deferred_tile128x256_3stage";
+        case SPMM_VARIANT_D128x128_S3: return "smfmac16x16x64_warpspec_deferred_tile128x128_3stage";
+        case SPMM_VARIANT_D128x128_S5: return "smfmac16x16x64_warpspec_deferred_tile128x128_5stage";
+        case SPMM_VARIANT_D64x256_S3: return "smfmac16x16x64_warpspec_deferred_tile64x256_3stage";
         default: return nullptr;
     }
 }
@@ -1318,6 +1467,10 @@ int spmm_variant_lds(int variant, int S) {
         case SPMM_VARIANT_W128x256_S3: return WsCfg<2, 4, 3, 4>::LDS_BYTES;
         case SPMM_VARIANT_W64x256_S2: return WsCfg<1, 4, 2, 2>::LDS_BYTES;
         case SPMM_VARIANT_W64x256_S3: return WsCfg<1, 4, 3, 2>::LDS_BYTES;
+        case SPMM_VARIANT_D128x256_S3: return WsCfg<2, 4, 3, 4>::LDS_BYTES;
+        case SPMM_VARIANT_D128x128_S3: return WsCfg<2, 2, 3, 4>::LDS_BYTES;
+        case SPMM_VARIANT_D128x128_S5: return WsCfg<2, 2, 5, 4>::LDS_BYTES;
+        case SPMM_VARIANT_D64x256_S3: return WsCfg<1, 4, 3, 2>::LDS_BYTES;
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_64x256: return 1;
         default: return 0;
     }
@@ -1327,8 +1480,9 @@ int spmm_variant_bm(int variant) {
     switch (variant) {
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_P128x128_S4: case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P128x128_S6:
         case SPMM_VARIANT_R128x128_S4: case SPMM_VARIANT_R128x128_S5: case SPMM_VARIANT_R128x128_S2:
-        case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2: case SPMM_VARIANT_W128x256_S3: return 128;
-        case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3:
+        case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2: case SPMM_VARIANT_W128x256_S3:
+        case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: return 128;
+        case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_D64x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 64;
         default: return 0;
     }
@@ -1337,7 +1491,9 @@ int spmm_variant_bn(int variant) {
     switch (variant) {
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_P128x128_S4: case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P128x128_S6:
         case SPMM_VARIANT_R128x128_S4: case SPMM_VARIANT_R128x128_S5: case SPMM_VARIANT_R128x128_S2:
-        case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2: return 128;
+        case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2:
+        case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: return 128;
+        case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D64x256_S3:
         case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_W128x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 256;
         default: return 0;
@@ -1385,6 +1541,15 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
     SPATHA_WS_CASE(SPMM_VARIANT_W64x256_S2, 1, 4, 2, 2)
     SPATHA_WS_CASE(SPMM_VARIANT_W64x256_S3, 1, 4, 3, 2)
 #undef SPATHA_WS_CASE
+#define SPATHA_WSD_CASE(ID, WM_, WN_, NS_, NP_)                                                         \
+    if (variant == ID)                                                                                  \
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ws<WM_, WN_, NS_, NP_, SPATHA_OUT_TRANSPOSED, true>(p, stream) \
+                                                   : launch_ws<WM_, WN_, NS_, NP_, SPATHA_OUT_ROW_MAJOR, true>(p, stream);
+    SPATHA_WSD_CASE(SPMM_VARIANT_D128x256_S3, 2, 4, 3, 4)
+    SPATHA_WSD_CASE(SPMM_VARIANT_D128x128_S3, 2, 2, 3, 4)
+    SPATHA_WSD_CASE(SPMM_VARIANT_D128x128_S5, 2, 2, 5, 4)
+    SPATHA_WSD_CASE(SPMM_VARIANT_D64x256_S3, 1, 4, 3, 2)
+#undef SPATHA_WSD_CASE
     return hipErrorInvalidValue;
 }
 

@@ -32,7 +32,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=500, help="untimed launches (the GPU needs ~50 ms of work to settle its clocks)")
     ap.add_argument("--rows", type=int, default=4096)
     ap.add_argument("--cols", type=int, default=1024)
     ap.add_argument("--n", type=int, default=16384, help="columns of B (tokens)")
@@ -129,7 +129,7 @@ def main():
                                      (1024, 4096, 4096, 8, 128), (4096, 1024, 16384, 4, 128),
                                      (4096, 1024, 16384, 16, 64), (4096, 1024, 16384, 32, 64)]:
             w2 = prepare(r2, c2, n2, m2, v2)
-            _, k2 = timed(w2, 50, 10)
+            _, k2 = timed(w2, 100, 200)
             by = algorithmic_bytes(r2, c2, n2, m2, v2, w2["geo"].ksp)
             extra.append({"shape": "%dx%dx%d %d:2:%d" % (r2, c2, n2, v2, m2), "us": round(k2 * 1e3, 2),
                           "dense_equiv_tflops": round(2.0 * r2 * c2 * n2 / (k2 * 1e-3) / 1e12, 1),

@@ -45,8 +45,8 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant) {
     return true;
 }
 
-// Kernel choice.  V a multiple of 128: producer/consumer kernel on 128-row tiles, 256 columns
-// wide when that still gives every CU at least two tiles, else 128 wide.  Otherwise (V a
+// Kernel choice.  V a multiple of 128: producer/consumer kernel on 128-row tiles; 256 columns wide
+// with 128 x 64 consumer waves when that still gives every CU at least two tiles, else 128 wide.  Otherwise (V a
 // multiple of 64 only) the 64 x 256 tile whose B rows are gathered per 64-row block.
 int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
     using namespace spatha;
@@ -55,7 +55,7 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
     int order[4] = {0, 0, 0, 0};
     if (v % 128 == 0) {
         const int64_t wide_tiles = (int64_t)(plan->geo.rows / 128) * ((N + 255) / 256);
-        order[0] = wide_tiles >= 512 ? SPMM_VARIANT_W128x256_S3 : SPMM_VARIANT_W128x128_S3;
+        order[0] = wide_tiles >= 512 ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x128_S3;
         order[1] = SPMM_VARIANT_W128x128_S3;
         order[2] = SPMM_VARIANT_P128x128_S3;
         order[3] = SPMM_VARIANT_128x128;

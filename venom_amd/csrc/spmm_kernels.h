@@ -49,7 +49,10 @@ enum {
     SPMM_VARIANT_D128x128_S3 = 21,
     SPMM_VARIANT_D128x128_S5 = 22,
     SPMM_VARIANT_D64x256_S3 = 23,
-    SPMM_VARIANT_COUNT = 24
+    SPMM_VARIANT_T128x256_S3 = 24,  // wave-specialised, each consumer wave owns 128 x 64
+    SPMM_VARIANT_T128x128_S4 = 25,
+    SPMM_VARIANT_T128x128_S5 = 26,
+    SPMM_VARIANT_COUNT = 27
 };
 
 const char* spmm_variant_name(int variant);

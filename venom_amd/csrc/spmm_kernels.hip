@@ -1338,6 +1338,188 @@ __device__ __forceinline__ void ws_consumer_deferred(const SpmmParams& p, const 
         for (int part = 0; part < 4; part++) flush_part(part);
 }
 
+// ---- tall consumer: one wave owns a 128 x 64 tile (two stacked 64-row halves sharing the B
+// fragments): 32 matrix instructions per k-step for the same 16 transposing reads, so the
+// LDS and issue cost per matrix instruction drops by a third and one consumer per SIMD is enough.
+#define SPATHA_MMA8(NB, BF)                                                                                     \
+    _Pragma("unroll") for (int h_ = 0; h_ < 2; h_++) {                                                          \
+        acc[h_][0][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[h_][0], BF, acc[h_][0][NB], (int)ix[h_][0], 0, 0); \
+        acc[h_][1][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[h_][1], BF, acc[h_][1][NB], (int)ix[h_][0], 0, 1); \
+        acc[h_][2][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[h_][2], BF, acc[h_][2][NB], (int)ix[h_][1], 0, 0); \
+        acc[h_][3][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[h_][3], BF, acc[h_][3][NB], (int)ix[h_][1], 0, 1); \
+    }
+
+template <int ROW_BYTES>
+__device__ __forceinline__ void mma_stage_tall(const char* st, int a_off, int i_off, const int (&tr_off)[4],
+                                               float4_t (&acc)[2][4][4]) {
+    half8_t a_cur[2][4];
+    uint32_t ix[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) a_cur[h][mb] = *(const half8_t*)(st + a_off + h * APACK_BLOCK + mb * 1024);
+        ix[h][0] = *(const uint32_t*)(st + i_off + h * APACK_BLOCK);
+        ix[h][1] = *(const uint32_t*)(st + i_off + h * APACK_BLOCK + 256);
+    }
+    half16_t bf0 = read_b_fragment<ROW_BYTES>(st, tr_off[0]);
+    half16_t bf1 = read_b_fragment<ROW_BYTES>(st, tr_off[1]);
+    __builtin_amdgcn_sched_barrier(0);
+    SPATHA_MMA8(0, bf0)
+    __builtin_amdgcn_sched_barrier(0);
+    bf0 = read_b_fragment<ROW_BYTES>(st, tr_off[2]);
+    __builtin_amdgcn_sched_barrier(0);
+    SPATHA_MMA8(1, bf1)
+    __builtin_amdgcn_sched_barrier(0);
+    bf1 = read_b_fragment<ROW_BYTES>(st, tr_off[3]);
+    __builtin_amdgcn_sched_barrier(0);
+    SPATHA_MMA8(2, bf0)
+    SPATHA_MMA8(3, bf1)
+}
+
+template <class Cfg, int WN, int OUT_LAYOUT>
+__device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int EPI_PITCH = Cfg::EPI_PITCH;
+    static_assert(BM == 128, "two stacked 64-row halves");
+    const int S = p.S, N = p.N;
+    const int wn = wave;
+    float4_t acc[2][4][4];
+    const int li = lane & 15, kb = lane >> 4;
+    const int rrow = kb * 4 + (li >> 2);
+    const int sw = rrow & 7;
+    int tr_off[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int ch = (wn * 8 + nb * 2 + ((li & 3) >> 1)) ^ (sw << 1);
+        tr_off[nb] = rrow * ROW_BYTES + ch * 16 + (li & 1) * 8;
+    }
+    const int a_off = B_BYTES + lane * 16;
+    const int i_off = B_BYTES + 4096 + lane * 4;
+    const int j16 = lane & 15, ib = lane >> 4;
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    uint32_t c_stage = 0;
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int a = 0; a < 4; a++)
+#pragma unroll
+                for (int b = 0; b < 4; b++) acc[h][a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            __syncthreads();
+            if (!(p.debug & 16)) mma_stage_tall<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc);
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+        }
+        const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+                const int64_t row0 = (int64_t)cm0 + h * 64 + ib * 16;
+                half8_t bias_lo, bias_hi;
+                if (p.bias) {
+                    bias_lo = *(const half8_t*)(p.bias + row0);
+                    bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+                }
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++) {
+                    const int col = cn0 + wn * 64 + nb * 16 + j16;
+                    half8_t lo, hi;
+#pragma unroll
+                    for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            lo[mb * 4 + r] = (_Float16)acc[h][mb][nb][r];
+                            hi[mb * 4 + r] = (_Float16)acc[h][mb + 2][nb][r];
+                        }
+                    if (p.bias) {
+                        lo = lo + bias_lo;
+                        hi = hi + bias_hi;
+                    }
+                    if (col < N && !(p.debug & 2)) {
+                        uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
+                        *(half8_t*)dst = lo;
+                        *(half8_t*)(dst + 8) = hi;
+                    }
+                }
+            } else if (!(p.debug & 4)) {
+                char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
+#pragma unroll
+                for (int mb = 0; mb < 4; mb++) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+#pragma unroll
+                        for (int nb = 0; nb < 4; nb++)
+                            *(_Float16*)(stg + (r * 4 + ib) * EPI_PITCH + (nb * 16 + j16) * 2) = (_Float16)acc[h][mb][nb][r];
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int it = 0; it < 2; it++) {
+                        const int Lr = it * 8 + (lane >> 3), ch = lane & 7;
+                        const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
+                        const int col = cn0 + wn * 64 + ch * 8;
+                        u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
+                        if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)cm0 + h * 64 + row) * N + col) = v;
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+        }
+        walk.next(c_tm, c_tn);
+    }
+}
+
+// Tile 128 x (64 * WN): WN tall consumers + NP producers.
+template <int WN, int NS, int NP, int OUT_LAYOUT>
+__global__ __launch_bounds__((WN + NP) * 64) void spmm_wst_kernel(SpmmParams p) {
+    using Cfg = WsCfg<2, WN, NS, NP>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TileWalk walk;
+    walk.init(p.tiles_m, p.tiles_n);
+    if (walk.my_tiles == 0) return;
+    if (p.skew > 0) {
+        const int units = ((blockIdx.x >> 3) & 7) * p.skew;
+        for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);
+    }
+    if (wave < WN) {
+        ws_consumer_tall<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
+    } else {
+        const int pr = wave - WN;
+        if (pr == 0) ws_producer<Cfg, NP, 0>(p, walk, smem, smem_base, lane);
+        else if (pr == 1) ws_producer<Cfg, NP, 1>(p, walk, smem, smem_base, lane);
+        else if (NP > 2 && pr == 2) ws_producer<Cfg, NP, (NP > 2 ? 2 : 0)>(p, walk, smem, smem_base, lane);
+        else if (NP > 2) ws_producer<Cfg, NP, (NP > 2 ? 3 : 0)>(p, walk, smem, smem_base, lane);
+    }
+}
+
+template <int WN, int NS, int NP, int OUT_LAYOUT>
+static hipError_t launch_wst(const SpmmParams& p, hipStream_t stream) {
+    using Cfg = WsCfg<2, WN, NS, NP>;
+    constexpr int lds = Cfg::LDS_BYTES;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static bool attr_set = false;
+    static int cus = 0;
+    auto kern = spmm_wst_kernel<WN, NS, NP, OUT_LAYOUT>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        int dev = 0;
+        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int per_cu = (160 * 1024) / lds;
+    const int tiles = p.tiles_m * p.tiles_n;
+    int grid = ((cus * per_cu) / 8) * 8;
+    const int need = ((tiles + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    if (grid < 8) grid = 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3((WN + NP) * 64), lds, stream, p);
+    return hipGetLastError();
+}
+
 template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false>
 __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams p) {
     using Cfg = WsCfg<WM, WN, NS, NP>;
@@ -1443,6 +1625,9 @@ const char* spmm_variant_name(int variant) {
         case SPMM_VARIANT_D128x128_S3: return "smfmac16x16x64_warpspec_deferred_tile128x128_3stage";
         case SPMM_VARIANT_D128x128_S5: return "smfmac16x16x64_warpspec_deferred_tile128x128_5stage";
         case SPMM_VARIANT_D64x256_S3: return "smfmac16x16x64_warpspec_deferred_tile64x256_3stage";
+        case SPMM_VARIANT_T128x256_S3: return "smfmac16x16x64_warpspec_tall_tile128x256_3stage";
+        case SPMM_VARIANT_T128x128_S4: return "smfmac16x16x64_warpspec_tall_tile128x128_4stage";
+        case SPMM_VARIANT_T128x128_S5: return "smfmac16x16x64_warpspec_tall_tile128x128_5stage";
         default: return nullptr;
     }
 }
@@ -1471,6 +1656,9 @@ int spmm_variant_lds(int variant, int S) {
         case SPMM_VARIANT_D128x128_S3: return WsCfg<2, 2, 3, 4>::LDS_BYTES;
         case SPMM_VARIANT_D128x128_S5: return WsCfg<2, 2, 5, 4>::LDS_BYTES;
         case SPMM_VARIANT_D64x256_S3: return WsCfg<1, 4, 3, 2>::LDS_BYTES;
+        case SPMM_VARIANT_T128x256_S3: return WsCfg<2, 4, 3, 4>::LDS_BYTES;
+        case SPMM_VARIANT_T128x128_S4: return WsCfg<2, 2, 4, 2>::LDS_BYTES;
+        case SPMM_VARIANT_T128x128_S5: return WsCfg<2, 2, 5, 4>::LDS_BYTES;
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_64x256: return 1;
         default: return 0;
     }
@@ -1481,7 +1669,8 @@ int spmm_variant_bm(int variant) {
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_P128x128_S4: case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P128x128_S6:
         case SPMM_VARIANT_R128x128_S4: case SPMM_VARIANT_R128x128_S5: case SPMM_VARIANT_R128x128_S2:
         case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2: case SPMM_VARIANT_W128x256_S3:
-        case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: return 128;
+        case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5:
+        case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5: return 128;
         case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_D64x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 64;
         default: return 0;
@@ -1492,8 +1681,8 @@ int spmm_variant_bn(int variant) {
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_P128x128_S4: case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P128x128_S6:
         case SPMM_VARIANT_R128x128_S4: case SPMM_VARIANT_R128x128_S5: case SPMM_VARIANT_R128x128_S2:
         case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2:
-        case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: return 128;
-        case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D64x256_S3:
+        case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5: return 128;
+        case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D64x256_S3: case SPMM_VARIANT_T128x256_S3:
         case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_W128x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 256;
         default: return 0;
@@ -1550,6 +1739,14 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
     SPATHA_WSD_CASE(SPMM_VARIANT_D128x128_S5, 2, 2, 5, 4)
     SPATHA_WSD_CASE(SPMM_VARIANT_D64x256_S3, 1, 4, 3, 2)
 #undef SPATHA_WSD_CASE
+#define SPATHA_WST_CASE(ID, WN_, NS_, NP_)                                                              \
+    if (variant == ID)                                                                                  \
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_wst<WN_, NS_, NP_, SPATHA_OUT_TRANSPOSED>(p, stream) \
+                                                   : launch_wst<WN_, NS_, NP_, SPATHA_OUT_ROW_MAJOR>(p, stream);
+    SPATHA_WST_CASE(SPMM_VARIANT_T128x256_S3, 4, 3, 4)
+    SPATHA_WST_CASE(SPMM_VARIANT_T128x128_S4, 2, 4, 2)
+    SPATHA_WST_CASE(SPMM_VARIANT_T128x128_S5, 2, 5, 4)
+#undef SPATHA_WST_CASE
     return hipErrorInvalidValue;
 }
 

@@ -40,6 +40,11 @@ CASES = [
     (256, 512, 16, 32, 128),      # m = 32, skinny N
     (512, 640, 136, 20, 128),     # m not a power of two
     (384, 416, 520, 8, 192),      # V = 192 (multiple of 64 only)
+    (256, 100, 72, 8, 64),        # 256-row tiles (dense-staged kernels), cols % m != 0
+    (512, 1000, 392, 8, 64),
+    (256, 64, 8, 4, 64),          # dense-staged, plain 2:4
+    (512, 325, 136, 5, 128),      # dense-staged, m = 5, V = 128, cols % m == 0 but Ksp padded
+    (768, 450, 264, 7, 192),      # dense-staged, m = 7, V = 192, two-column tail
 ]
 
 
@@ -64,6 +69,18 @@ def test_integer_operands_bit_exact(gpu, rows, cols, N, m, v, transposed):
         torch.cuda.synchronize()
         assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16)), (variant,)
     assert ran >= 4
+
+
+def test_dense_staged_kernel_is_selected_for_v64(gpu):
+    rows, cols, N, m, v = 512, 256, 256, 8, 64
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=2, integer_values=True)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    assert "densestage" in plan.kernel_name(N, 0, 0)
+    # m = 16 does not fit a stage, 128-row matrices do not fill a 256-row tile
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, 16, v, seed=2, integer_values=True)
+    assert "densestage" not in _plan(vals, meta, columns, rows, cols, 16, v, gpu).kernel_name(N, 0, 0)
+    vals, meta, columns = F.synthetic_vnm(128, cols, 2, m, v, seed=2, integer_values=True)
+    assert "densestage" not in _plan(vals, meta, columns, 128, cols, m, v, gpu).kernel_name(N, 0, 0)
 
 
 @pytest.mark.parametrize("path", [p for p in golden_cases() if "_v64" in p or "_v128" in p],

@@ -20,6 +20,7 @@ struct spatha_spmm_plan {
     uint16_t* apack;
     uint32_t* rowtab;
     void* zeros;           // 1 KiB of zeros on the device
+    uint16_t* gtab;        // gather table of the dense-staged kernels (V = 64, m <= 8), or null
     size_t apack_bytes, rowtab_bytes;
 };
 
@@ -35,7 +36,13 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant) {
     using namespace spatha;
     if (variant <= 0 || variant >= SPMM_VARIANT_COUNT) return false;
     const int bm = spmm_variant_bm(variant);
-    if (bm == 0 || plan->geo.v % bm != 0) return false;
+    if (bm == 0) return false;
+    if (variant == SPMM_VARIANT_DS256x128_S3 || variant == SPMM_VARIANT_DS256x128_S2) {
+        // four 64-row blocks per tile; all 16*m dense rows of a k-step must fit one stage
+        if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 256 != 0 || !plan->gtab) return false;
+    } else if (plan->geo.v % bm != 0) {
+        return false;
+    }
     if (spmm_variant_lds(variant, plan->S) > 160 * 1024) return false;      // row table kept in LDS
     if (variant >= SPMM_VARIANT_R128x128_S4) {
         // buffer-descriptor kernels address B, the packed operands and the row table with 32-bit offsets
@@ -60,9 +67,10 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
         order[2] = SPMM_VARIANT_P128x128_S3;
         order[3] = SPMM_VARIANT_128x128;
     } else if (v % 64 == 0) {
-        order[0] = SPMM_VARIANT_P64x256_S2;
-        order[1] = SPMM_VARIANT_W64x256_S3;
-        order[2] = SPMM_VARIANT_64x256;
+        // m <= 8: staging the dense B rows once for four 64-row blocks halves the L2 -> LDS traffic
+        order[0] = SPMM_VARIANT_DS256x128_S3;
+        order[1] = SPMM_VARIANT_P64x256_S2;
+        order[2] = SPMM_VARIANT_W64x256_S3;
         order[3] = SPMM_VARIANT_64x256;
     } else {
         return -1;
@@ -151,7 +159,7 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     if (!plan) return SPATHA_ERR_BAD_ARGUMENT;
     plan->geo = geo;
     plan->S = (geo.ksp + 31) / 32;
-    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr;
+    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr;
     e = hipGetDevice(&plan->device);
     if (e != hipSuccess) { delete plan; return hip_fail(e); }
     const size_t a_bytes = (size_t)(rows / 64) * plan->S * spatha::APACK_BLOCK;
@@ -167,6 +175,14 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     e = spatha::launch_pack(values_dev, metadata_dev, columns_dev, rows, cols, m, v, geo.ksp, plan->S, plan->apack,
                             plan->rowtab, (hipStream_t)stream);
     if (e != hipSuccess) { spatha_spmm_plan_destroy(plan); return hip_fail(e); }
+    if (v % 64 == 0 && m <= 8 && rows % 256 == 0) {
+        const size_t g_bytes = (size_t)(rows / 64) * plan->S * 64 * 2;
+        if ((e = hipMalloc((void**)&plan->gtab, g_bytes)) != hipSuccess ||
+            (e = spatha::launch_pack_gtab(columns_dev, rows, m, v, geo.ksp, plan->S, plan->gtab, (hipStream_t)stream)) != hipSuccess) {
+            spatha_spmm_plan_destroy(plan);
+            return hip_fail(e);
+        }
+    }
     *out = plan;
     return SPATHA_OK;
 }
@@ -177,6 +193,7 @@ int spatha_spmm_plan_destroy(spatha_spmm_plan* plan) {
     if (plan->apack && (e = hipFree(plan->apack)) != hipSuccess && first == hipSuccess) first = e;
     if (plan->rowtab && (e = hipFree(plan->rowtab)) != hipSuccess && first == hipSuccess) first = e;
     if (plan->zeros && (e = hipFree(plan->zeros)) != hipSuccess && first == hipSuccess) first = e;
+    if (plan->gtab && (e = hipFree(plan->gtab)) != hipSuccess && first == hipSuccess) first = e;
     delete plan;
     return first == hipSuccess ? SPATHA_OK : hip_fail(first);
 }
@@ -192,8 +209,8 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
     if (var < 0) return SPATHA_ERR_UNSUPPORTED;
     spatha::SpmmParams p;
     p.apack = plan->apack; p.rowtab = plan->rowtab;
-    p.B = B_dev; p.bias = bias_dev; p.C = out_dev; p.zeros = plan->zeros;
-    p.rows = plan->geo.rows; p.cols = plan->geo.cols; p.N = N; p.S = plan->S; p.v = plan->geo.v;
+    p.B = B_dev; p.bias = bias_dev; p.C = out_dev; p.zeros = plan->zeros; p.gtab = plan->gtab;
+    p.rows = plan->geo.rows; p.cols = plan->geo.cols; p.N = N; p.S = plan->S; p.v = plan->geo.v; p.m = plan->geo.m;
     const int bm = spatha::spmm_variant_bm(var), bn = spatha::spmm_variant_bn(var);
     p.tiles_m = plan->geo.rows / bm;
     p.tiles_n = (N + bn - 1) / bn;

@@ -13,11 +13,13 @@ enum { APACK_BLOCK = 4096 + 512 };
 struct SpmmParams {
     const uint16_t* apack;    // packed A operands + sparse-index words, APACK_BLOCK bytes per (64 rows, k-step)
     const uint32_t* rowtab;   // gathered B row per LDS row
+    const uint16_t* gtab;     // dense-staged kernels: LDS offset per (64-row block, step, lane class, fragment), or null
     const uint16_t* B;        // cols x N, row-major
     const uint16_t* bias;     // rows, or null
     const void* zeros;        // >= 1 KiB of zero bytes (source of zero-filled B rows)
     uint16_t* C;              // rows x N, or N x rows when transposed
     int rows, cols, N, S, v;
+    int m;                    // dense columns per group (dense-staged kernels)
     uint32_t b_bytes, apack_bytes, rowtab_bytes;   // sizes for buffer descriptors (persistent kernels)
     int tiles_m, tiles_n;
     int skew;                 // start-up skew between workgroups, in units of 1024 clocks (0 = none)
@@ -52,7 +54,9 @@ enum {
     SPMM_VARIANT_T128x256_S3 = 24,  // wave-specialised, each consumer wave owns 128 x 64
     SPMM_VARIANT_T128x128_S4 = 25,
     SPMM_VARIANT_T128x128_S5 = 26,
-    SPMM_VARIANT_COUNT = 27
+    SPMM_VARIANT_DS256x128_S3 = 27,  // m <= 8: all 16*m dense B rows of a k-step staged once for four 64-row blocks
+    SPMM_VARIANT_DS256x128_S2 = 28,
+    SPMM_VARIANT_COUNT = 29
 };
 
 const char* spmm_variant_name(int variant);
@@ -64,6 +68,9 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
 
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
                        int m, int v, int ksp, int S, uint16_t* apack, uint32_t* rowtab, hipStream_t stream);
+
+hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, uint16_t* gtab,
+                            hipStream_t stream);
 
 hipError_t launch_dense_gemm(const uint16_t* A, const uint16_t* B, int rows, int cols, int N, uint16_t* C,
                              hipStream_t stream);

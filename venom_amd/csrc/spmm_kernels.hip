@@ -1520,6 +1520,338 @@ static hipError_t launch_wst(const SpmmParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// Dense-staged kernel for m <= 8 (tile 256 x 128 = four 64-row blocks; pays off most at V = 64).
+//
+// With 64-row blocks a gathered B stage serves only 64 rows of C, and the L2 -> LDS traffic
+// per output element doubles.  Here the producers stage ALL 16*m dense B rows of a k-step
+// (m <= 8: at most 128 rows x 256 B) once for the four V blocks of the tile, and each
+// consumer picks its V block's 4-of-m rows through the ADDRESSES of its transposing reads:
+// gtab holds, per (64-row block, k-step, lane class), the LDS byte offset of the row a lane has to
+// read for each of its four fragments (row * 256 + swizzle), built once per matrix.
+// Rows beyond K come back as zeros from the buffer bounds check, so padding groups (whose
+// column offsets are 0) and tail groups need no special case.
+// Consumer w owns rows 128*(w/2) .. +127 (two V blocks, one per 64-row half) x columns
+// 64*(w%2) .. +63.  Producers need no row table: B rows are consecutive.
+// ---------------------------------------------------------------------------
+template <int M, int NS, int NP>
+struct DsCfg {
+    static constexpr int NC = 4;
+    static constexpr int BM = 256, BN = 128;
+    static constexpr int ROW_BYTES = BN * 2;
+    static constexpr int DENSE_ROWS = 16 * M;
+    static constexpr int B_BYTES = DENSE_ROWS * ROW_BYTES;
+    static constexpr int STAGE_BYTES = B_BYTES + 4 * APACK_BLOCK;
+    static constexpr int PA = NS - 1;
+    static constexpr int EPI_PITCH = 144;
+    static constexpr int EPI_BYTES = NC * 16 * EPI_PITCH;
+    static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES + EPI_BYTES;
+    static constexpr int THREADS = (NC + NP) * 64;
+};
+
+template <class Cfg, int M, int NP, int PR>
+__device__ __forceinline__ void ds_producer(const SpmmParams& p, const TileWalk& walk, uint32_t smem_base, int lane) {
+    constexpr int BN = Cfg::BN, NS = Cfg::PA + 1, PA = Cfg::PA;
+    constexpr int B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int NB_LOADS = (4 * M) / NP;           // 4 rows per DMA instruction
+    constexpr int NA_LOADS = 24 / NP;                // 4 wave-tile rows x (4 operand + 2 index blocks)
+    constexpr int LOADS = NB_LOADS + NA_LOADS;
+    static_assert((4 * M) % NP == 0 && 24 % NP == 0, "DMA work must split evenly over the producers");
+    static_assert((PA - 1) * LOADS < 64, "vmcnt range");
+    const int S = p.S, N = p.N;
+    const int Q = walk.my_tiles * S;
+    const i32x4 rsrc_b = make_buffer(p.B, p.b_bytes);
+    const i32x4 rsrc_a = make_buffer(p.apack, p.apack_bytes);
+    const uint32_t row_bytes_b = (uint32_t)N * 2u;
+    const int dense_rows = 16 * p.m;                 // rows of B one k-step spans (<= 16 * M)
+    const uint32_t step_bytes_b = (uint32_t)dense_rows * row_bytes_b;
+    const int slot_row = lane >> 4, slot_chunk = lane & 15;
+    const uint32_t lane16 = lane * 16, lane4 = lane * 4;
+
+    int is_tm = walk.tm0, is_tn = walk.tn0, is_step = 0;
+    uint32_t is_stage = 0, b_soff = 0;
+    uint32_t a_soff = (uint32_t)((is_tm * 4) * S) * (uint32_t)APACK_BLOCK;
+    int issue_left = Q;
+    uint32_t voff[NB_LOADS];
+    auto set_voff = [&]() {
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) {
+            const int row = (PR * NB_LOADS + j) * 4 + slot_row;             // dense row inside the stage
+            const int col = is_tn * BN + (slot_chunk ^ ((row & 7) << 1)) * 8;
+            voff[j] = (col < N && row < dense_rows && !(p.debug & 1)) ? (uint32_t)row * row_bytes_b + (uint32_t)col * 2u
+                                                                       : 0xF0000000u;
+        }
+    };
+    set_voff();
+    auto issue_batch = [&]() {
+        const uint32_t stage = smem_base + is_stage;
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) bdma_b128(voff[j], rsrc_b, b_soff, stage + (PR * NB_LOADS + j) * 1024);
+#pragma unroll
+        for (int k = 0; k < NA_LOADS; k++) {
+            const int a = PR * NA_LOADS + k;
+            const int awm = a / 6, ak = a - awm * 6;
+            const uint32_t soff = a_soff + (uint32_t)(awm * S) * (uint32_t)APACK_BLOCK;
+            const uint32_t dst = stage + B_BYTES + awm * APACK_BLOCK;
+            if (ak < 4) bdma_b128(lane16, rsrc_a, soff + ak * 1024, dst + ak * 1024);
+            else bdma_b32(lane4, rsrc_a, soff + 4096 + (ak - 4) * 256, dst + 4096 + (ak - 4) * 256);
+        }
+        --issue_left;
+        is_stage = (is_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : is_stage + STAGE_BYTES;
+        a_soff += (uint32_t)APACK_BLOCK;
+        b_soff += step_bytes_b;
+        if (++is_step == S) {
+            is_step = 0;
+            b_soff = 0;
+            walk.next(is_tm, is_tn);
+            a_soff = (uint32_t)((is_tm * 4) * S) * (uint32_t)APACK_BLOCK;
+            set_voff();
+        }
+    };
+#pragma unroll
+    for (int t = 0; t < PA; t++)
+        if (t < Q) issue_batch();
+    const int q_main = Q - PA > 0 ? Q - PA : 0;
+    for (int q = 0; q < q_main; q++) {
+        wait_vmcnt<(PA - 1) * LOADS>();
+        __syncthreads();
+        if (!(p.debug & 8)) issue_batch();
+    }
+    for (int q = q_main; q < Q; q++) {
+        wait_stages<LOADS, PA - 1>(Q - 1 - q);
+        __syncthreads();
+    }
+}
+
+template <class Cfg, int OUT_LAYOUT>
+__device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
+    constexpr int B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int EPI_PITCH = Cfg::EPI_PITCH;
+    const int S = p.S, N = p.N;
+    const int wm2 = wave >> 1, wn = wave & 1;
+    float4_t acc[2][4][4];
+    const int li = lane & 15, kb = lane >> 4;
+    // fixed part of a transposing-read address: column chunk (wn*8 + (li%4)/2) and the 8-byte half
+    const uint32_t col_xor = (uint32_t)((wn * 8 + ((li & 3) >> 1)) << 4);
+    const uint32_t col_or = (uint32_t)(li & 1) * 8u;
+    const int a_off = B_BYTES + (wm2 * 2) * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + (wm2 * 2) * APACK_BLOCK + 4096 + lane * 4;
+    const int j16 = lane & 15, ib = lane >> 4;
+    // gather table: [64-row block][step][kb][c = (li/4)][fb] u16 -> this lane's 8 bytes per (block, step)
+    const int lane_class = kb * 4 + (li >> 2);
+    auto gtab_ptr = [&](int tm, int h, int step) {
+        const int64_t vb = (int64_t)tm * 4 + wm2 * 2 + h;
+        return (const u32x2*)(p.gtab + ((vb * S + step) * 16 + lane_class) * 4);
+    };
+
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    int n_tm = c_tm, n_tn = c_tn;       // tile of the NEXT step's table entries
+    uint32_t c_stage = 0;
+    u32x2 g_cur[2], g_next[2];
+    g_cur[0] = *gtab_ptr(c_tm, 0, 0);
+    g_cur[1] = *gtab_ptr(c_tm, 1, 0);
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int a = 0; a < 4; a++)
+#pragma unroll
+                for (int b = 0; b < 4; b++) acc[h][a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            // table entries of the next step (next tile after the last step; clamped at the very end)
+            int ns = c_step + 1;
+            if (ns == S) {
+                ns = 0;
+                if (c_tile + 1 < walk.my_tiles) walk.next(n_tm, n_tn);
+            }
+            g_next[0] = *gtab_ptr(n_tm, 0, ns);
+            g_next[1] = *gtab_ptr(n_tm, 1, ns);
+            __syncthreads();
+            if (!(p.debug & 16)) {
+                const char* st = smem + c_stage;
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    half8_t a_cur[4];
+#pragma unroll
+                    for (int mb = 0; mb < 4; mb++) a_cur[mb] = *(const half8_t*)(st + a_off + h * APACK_BLOCK + mb * 1024);
+                    const uint32_t i0 = *(const uint32_t*)(st + i_off + h * APACK_BLOCK);
+                    const uint32_t i1 = *(const uint32_t*)(st + i_off + h * APACK_BLOCK + 256);
+                    uint32_t base[4];
+                    base[0] = ((g_cur[h].x & 0xffffu) ^ col_xor) | col_or;
+                    base[1] = ((g_cur[h].x >> 16) ^ col_xor) | col_or;
+                    base[2] = ((g_cur[h].y & 0xffffu) ^ col_xor) | col_or;
+                    base[3] = ((g_cur[h].y >> 16) ^ col_xor) | col_or;
+                    auto read_frag = [&](int nb) {
+                        half16_t bf;
+#pragma unroll
+                        for (int fb = 0; fb < 4; fb++) {
+                            short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, st + (base[fb] ^ (uint32_t)(nb << 5))));
+                            half4_t h4 = __builtin_bit_cast(half4_t, t4);
+                            bf[fb * 4 + 0] = h4[0];
+                            bf[fb * 4 + 1] = h4[1];
+                            bf[fb * 4 + 2] = h4[2];
+                            bf[fb * 4 + 3] = h4[3];
+                        }
+                        return bf;
+                    };
+                    half16_t bf0 = read_frag(0);
+                    half16_t bf1 = read_frag(1);
+                    __builtin_amdgcn_sched_barrier(0);
+#define SPATHA_MMA4H(NB, BF)                                                                                          \
+    acc[h][0][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[0], BF, acc[h][0][NB], (int)i0, 0, 0);             \
+    acc[h][1][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], BF, acc[h][1][NB], (int)i0, 0, 1);             \
+    acc[h][2][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], BF, acc[h][2][NB], (int)i1, 0, 0);             \
+    acc[h][3][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], BF, acc[h][3][NB], (int)i1, 0, 1);
+                    SPATHA_MMA4H(0, bf0)
+                    __builtin_amdgcn_sched_barrier(0);
+                    bf0 = read_frag(2);
+                    __builtin_amdgcn_sched_barrier(0);
+                    SPATHA_MMA4H(1, bf1)
+                    __builtin_amdgcn_sched_barrier(0);
+                    bf1 = read_frag(3);
+                    __builtin_amdgcn_sched_barrier(0);
+                    SPATHA_MMA4H(2, bf0)
+                    SPATHA_MMA4H(3, bf1)
+#undef SPATHA_MMA4H
+                }
+            }
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+            g_cur[0] = g_next[0];
+            g_cur[1] = g_next[1];
+        }
+        const int cm0 = c_tm * BM + wm2 * 128, cn0 = c_tn * BN;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+                const int64_t row0 = (int64_t)cm0 + h * 64 + ib * 16;
+                half8_t bias_lo, bias_hi;
+                if (p.bias) {
+                    bias_lo = *(const half8_t*)(p.bias + row0);
+                    bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+                }
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++) {
+                    const int col = cn0 + wn * 64 + nb * 16 + j16;
+                    half8_t lo, hi;
+#pragma unroll
+                    for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            lo[mb * 4 + r] = (_Float16)acc[h][mb][nb][r];
+                            hi[mb * 4 + r] = (_Float16)acc[h][mb + 2][nb][r];
+                        }
+                    if (p.bias) {
+                        lo = lo + bias_lo;
+                        hi = hi + bias_hi;
+                    }
+                    if (col < N && !(p.debug & 2)) {
+                        uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
+                        *(half8_t*)dst = lo;
+                        *(half8_t*)(dst + 8) = hi;
+                    }
+                }
+            } else if (!(p.debug & 4)) {
+                char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
+#pragma unroll
+                for (int mb = 0; mb < 4; mb++) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+#pragma unroll
+                        for (int nb = 0; nb < 4; nb++)
+                            *(_Float16*)(stg + (r * 4 + ib) * EPI_PITCH + (nb * 16 + j16) * 2) = (_Float16)acc[h][mb][nb][r];
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int it = 0; it < 2; it++) {
+                        const int Lr = it * 8 + (lane >> 3), ch = lane & 7;
+                        const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
+                        const int col = cn0 + wn * 64 + ch * 8;
+                        u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
+                        if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)cm0 + h * 64 + row) * N + col) = v;
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+        }
+        walk.next(c_tm, c_tn);
+    }
+}
+
+template <int M, int NS, int NP, int OUT_LAYOUT>
+__global__ __launch_bounds__((4 + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
+    using Cfg = DsCfg<M, NS, NP>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TileWalk walk;
+    walk.init(p.tiles_m, p.tiles_n);
+    if (walk.my_tiles == 0) return;
+    if (wave < 4) {
+        ds_consumer<Cfg, OUT_LAYOUT>(p, walk, smem, wave, lane);
+    } else {
+        const int pr = wave - 4;
+        if (pr == 0) ds_producer<Cfg, M, NP, 0>(p, walk, smem_base, lane);
+        else if (pr == 1) ds_producer<Cfg, M, NP, 1>(p, walk, smem_base, lane);
+        else if (pr == 2) ds_producer<Cfg, M, NP, 2>(p, walk, smem_base, lane);
+        else ds_producer<Cfg, M, NP, 3>(p, walk, smem_base, lane);
+    }
+}
+
+template <int M, int NS, int NP, int OUT_LAYOUT>
+static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
+    using Cfg = DsCfg<M, NS, NP>;
+    constexpr int lds = Cfg::LDS_BYTES;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static bool attr_set = false;
+    static int cus = 0;
+    auto kern = spmm_ds_kernel<M, NS, NP, OUT_LAYOUT>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        int dev = 0;
+        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int tiles = p.tiles_m * p.tiles_n;
+    int grid = (cus / 8) * 8;
+    const int need = ((tiles + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    if (grid < 8) grid = 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::THREADS), lds, stream, p);
+    return hipGetLastError();
+}
+
+// gather table of the dense-staged kernel: [64-row block][step][kb][c][fb] u16 = LDS byte offset of dense
+// row d = gamma*m + column-loc (gamma = 4*fb + kb): d*256 + (d % 8)*32 (the swizzle of that row)
+__global__ void pack_gtab_kernel(const uint32_t* __restrict__ columns, int rows, int m, int v, int ksp, int S,
+                                 uint16_t* __restrict__ gtab) {
+    const int ngroups = ksp / 2;
+    const int64_t total = (int64_t)(rows / 64) * S * 64;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        const int fb = (int)(t & 3), c = (int)((t >> 2) & 3), kb = (int)((t >> 4) & 3);
+        const int64_t bs = t >> 6;
+        const int s = (int)(bs % S);
+        const int64_t b = (bs / S) * 64 / v;
+        const int gamma = fb * 4 + kb;
+        const int g = s * 16 + gamma;
+        uint32_t d = (uint32_t)gamma * m;
+        if (g < ngroups) d += columns[b * ngroups * 4 + (int64_t)g * 4 + c];
+        gtab[t] = (uint16_t)(d * 256u + (d & 7u) * 32u);
+    }
+}
+
+hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, uint16_t* gtab,
+                            hipStream_t stream) {
+    int64_t total = (int64_t)(rows / 64) * S * 64;
+    int blocks = (int)((total + 255) / 256);
+    if (blocks > 65535 * 8) blocks = 65535 * 8;
+    hipLaunchKernelGGL(pack_gtab_kernel, dim3(blocks), dim3(256), 0, stream, columns, rows, m, v, ksp, S, gtab);
+    return hipGetLastError();
+}
+
 template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false>
 __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams p) {
     using Cfg = WsCfg<WM, WN, NS, NP>;
@@ -1628,6 +1960,8 @@ const char* spmm_variant_name(int variant) {
         case SPMM_VARIANT_T128x256_S3: return "smfmac16x16x64_warpspec_tall_tile128x256_3stage";
         case SPMM_VARIANT_T128x128_S4: return "smfmac16x16x64_warpspec_tall_tile128x128_4stage";
         case SPMM_VARIANT_T128x128_S5: return "smfmac16x16x64_warpspec_tall_tile128x128_5stage";
+        case SPMM_VARIANT_DS256x128_S3: return "smfmac16x16x64_warpspec_densestage_tile256x128_3stage";
+        case SPMM_VARIANT_DS256x128_S2: return "smfmac16x16x64_warpspec_densestage_tile256x128_2stage";
         default: return nullptr;
     }
 }
@@ -1659,6 +1993,8 @@ int spmm_variant_lds(int variant, int S) {
         case SPMM_VARIANT_T128x256_S3: return WsCfg<2, 4, 3, 4>::LDS_BYTES;
         case SPMM_VARIANT_T128x128_S4: return WsCfg<2, 2, 4, 2>::LDS_BYTES;
         case SPMM_VARIANT_T128x128_S5: return WsCfg<2, 2, 5, 4>::LDS_BYTES;
+        case SPMM_VARIANT_DS256x128_S3: return DsCfg<8, 3, 4>::LDS_BYTES;
+        case SPMM_VARIANT_DS256x128_S2: return DsCfg<8, 2, 4>::LDS_BYTES;
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_64x256: return 1;
         default: return 0;
     }
@@ -1673,6 +2009,7 @@ int spmm_variant_bm(int variant) {
         case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5: return 128;
         case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_D64x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 64;
+        case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: return 256;
         default: return 0;
     }
 }
@@ -1681,7 +2018,8 @@ int spmm_variant_bn(int variant) {
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_P128x128_S4: case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P128x128_S6:
         case SPMM_VARIANT_R128x128_S4: case SPMM_VARIANT_R128x128_S5: case SPMM_VARIANT_R128x128_S2:
         case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2:
-        case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5: return 128;
+        case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5:
+        case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: return 128;
         case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D64x256_S3: case SPMM_VARIANT_T128x256_S3:
         case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_W128x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 256;
@@ -1747,6 +2085,12 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
     SPATHA_WST_CASE(SPMM_VARIANT_T128x128_S4, 2, 4, 2)
     SPATHA_WST_CASE(SPMM_VARIANT_T128x128_S5, 2, 5, 4)
 #undef SPATHA_WST_CASE
+    if (variant == SPMM_VARIANT_DS256x128_S3)
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ds<8, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
+                                                   : launch_ds<8, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
+    if (variant == SPMM_VARIANT_DS256x128_S2)
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ds<8, 2, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
+                                                   : launch_ds<8, 2, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
     return hipErrorInvalidValue;
 }
 

@@ -20,7 +20,9 @@ struct spatha_spmm_plan {
     uint16_t* apack;
     uint32_t* rowtab;
     void* zeros;           // 1 KiB of zeros on the device
-    uint16_t* gtab;        // gather table of the dense-staged kernels (V = 64, m <= 8), or null
+    uint16_t* gtab;        // gather table of the dense-staged kernels (m <= 8, rows % 256 == 0), or null
+    uint16_t* gtab_tiles;  // tile-major copy for the flag-synchronised kernel
+    size_t gtab_tiles_bytes;
     size_t apack_bytes, rowtab_bytes;
 };
 
@@ -37,7 +39,9 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant) {
     if (variant <= 0 || variant >= SPMM_VARIANT_COUNT) return false;
     const int bm = spmm_variant_bm(variant);
     if (bm == 0) return false;
-    if (variant == SPMM_VARIANT_DS256x128_S3 || variant == SPMM_VARIANT_DS256x128_S2) {
+    if (variant == SPMM_VARIANT_DS256x128_S3 || variant == SPMM_VARIANT_DS256x128_S2 ||
+        variant == SPMM_VARIANT_DS256x128_S3_C8 || variant == SPMM_VARIANT_DS256x128_S3_PP ||
+        variant == SPMM_VARIANT_DSF256x128_S3) {
         // four 64-row blocks per tile; all 16*m dense rows of a k-step must fit one stage
         if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 256 != 0 || !plan->gtab) return false;
     } else if (plan->geo.v % bm != 0) {
@@ -68,7 +72,7 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
         order[3] = SPMM_VARIANT_128x128;
     } else if (v % 64 == 0) {
         // m <= 8: staging the dense B rows once for four 64-row blocks halves the L2 -> LDS traffic
-        order[0] = SPMM_VARIANT_DS256x128_S3;
+        order[0] = SPMM_VARIANT_DS256x128_S3_C8;
         order[1] = SPMM_VARIANT_P64x256_S2;
         order[2] = SPMM_VARIANT_W64x256_S3;
         order[3] = SPMM_VARIANT_64x256;
@@ -159,7 +163,7 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     if (!plan) return SPATHA_ERR_BAD_ARGUMENT;
     plan->geo = geo;
     plan->S = (geo.ksp + 31) / 32;
-    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr;
+    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr; plan->gtab_tiles = nullptr; plan->gtab_tiles_bytes = 0;
     e = hipGetDevice(&plan->device);
     if (e != hipSuccess) { delete plan; return hip_fail(e); }
     const size_t a_bytes = (size_t)(rows / 64) * plan->S * spatha::APACK_BLOCK;
@@ -182,6 +186,13 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
             spatha_spmm_plan_destroy(plan);
             return hip_fail(e);
         }
+        plan->gtab_tiles_bytes = (size_t)(rows / 256) * plan->S * 512;
+        if ((e = hipMalloc((void**)&plan->gtab_tiles, plan->gtab_tiles_bytes)) != hipSuccess ||
+            (e = spatha::launch_pack_gtab_tiles(columns_dev, rows, m, v, geo.ksp, plan->S, plan->gtab_tiles,
+                                                (hipStream_t)stream)) != hipSuccess) {
+            spatha_spmm_plan_destroy(plan);
+            return hip_fail(e);
+        }
     }
     *out = plan;
     return SPATHA_OK;
@@ -194,6 +205,7 @@ int spatha_spmm_plan_destroy(spatha_spmm_plan* plan) {
     if (plan->rowtab && (e = hipFree(plan->rowtab)) != hipSuccess && first == hipSuccess) first = e;
     if (plan->zeros && (e = hipFree(plan->zeros)) != hipSuccess && first == hipSuccess) first = e;
     if (plan->gtab && (e = hipFree(plan->gtab)) != hipSuccess && first == hipSuccess) first = e;
+    if (plan->gtab_tiles && (e = hipFree(plan->gtab_tiles)) != hipSuccess && first == hipSuccess) first = e;
     delete plan;
     return first == hipSuccess ? SPATHA_OK : hip_fail(first);
 }
@@ -210,6 +222,7 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
     spatha::SpmmParams p;
     p.apack = plan->apack; p.rowtab = plan->rowtab;
     p.B = B_dev; p.bias = bias_dev; p.C = out_dev; p.zeros = plan->zeros; p.gtab = plan->gtab;
+    p.gtab_tiles = plan->gtab_tiles; p.gtab_tiles_bytes = (uint32_t)plan->gtab_tiles_bytes;
     p.rows = plan->geo.rows; p.cols = plan->geo.cols; p.N = N; p.S = plan->S; p.v = plan->geo.v; p.m = plan->geo.m;
     const int bm = spatha::spmm_variant_bm(var), bn = spatha::spmm_variant_bn(var);
     p.tiles_m = plan->geo.rows / bm;
@@ -219,6 +232,10 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
     p.rowtab_bytes = (uint32_t)plan->rowtab_bytes;
     { const char* d = std::getenv("SPATHA_DEBUG_KNOBS"); p.debug = d ? std::atoi(d) : 0; }
     { const char* d = std::getenv("SPATHA_SKEW"); p.skew = d ? std::atoi(d) : 0; }
+    p.prof = nullptr;
+#ifdef SPATHA_DEV_PROFILE
+    { const char* d = std::getenv("SPATHA_PROF_PTR"); if (d) p.prof = (long long*)std::strtoull(d, nullptr, 0); }
+#endif
     hipError_t e = spatha::launch_spmm(var, out_layout, p, (hipStream_t)stream);
     return e == hipSuccess ? SPATHA_OK : hip_fail(e);
 }

@@ -14,6 +14,8 @@ struct SpmmParams {
     const uint16_t* apack;    // packed A operands + sparse-index words, APACK_BLOCK bytes per (64 rows, k-step)
     const uint32_t* rowtab;   // gathered B row per LDS row
     const uint16_t* gtab;     // dense-staged kernels: LDS offset per (64-row block, step, lane class, fragment), or null
+    const uint16_t* gtab_tiles;  // the same table, tile-major (512 B per 256-row tile and step), or null
+    uint32_t gtab_tiles_bytes;
     const uint16_t* B;        // cols x N, row-major
     const uint16_t* bias;     // rows, or null
     const void* zeros;        // >= 1 KiB of zero bytes (source of zero-filled B rows)
@@ -23,6 +25,7 @@ struct SpmmParams {
     uint32_t b_bytes, apack_bytes, rowtab_bytes;   // sizes for buffer descriptors (persistent kernels)
     int tiles_m, tiles_n;
     int skew;                 // start-up skew between workgroups, in units of 1024 clocks (0 = none)
+    long long* prof;          // development cycle-accounting buffer (SPATHA_DEV_PROFILE builds), else null
     int debug;                // development knobs (0 in production): 1 = skip B loads, 2 = skip C stores
 };
 
@@ -56,7 +59,10 @@ enum {
     SPMM_VARIANT_T128x128_S5 = 26,
     SPMM_VARIANT_DS256x128_S3 = 27,  // m <= 8: all 16*m dense B rows of a k-step staged once for four 64-row blocks
     SPMM_VARIANT_DS256x128_S2 = 28,
-    SPMM_VARIANT_COUNT = 29
+    SPMM_VARIANT_DS256x128_S3_C8 = 29,  // eight 64 x 64 consumer waves (two per SIMD)
+    SPMM_VARIANT_DS256x128_S3_PP = 30,  // eight consumers in two phase groups (ping-pong)
+    SPMM_VARIANT_DSF256x128_S3 = 31,    // dense-staged, LDS flag counters instead of workgroup barriers
+    SPMM_VARIANT_COUNT = 32
 };
 
 const char* spmm_variant_name(int variant);
@@ -71,6 +77,9 @@ hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const u
 
 hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, uint16_t* gtab,
                             hipStream_t stream);
+
+hipError_t launch_pack_gtab_tiles(const uint32_t* columns, int rows, int m, int v, int ksp, int S, uint16_t* gtab,
+                                  hipStream_t stream);
 
 hipError_t launch_dense_gemm(const uint16_t* A, const uint16_t* B, int rows, int cols, int N, uint16_t* C,
                              hipStream_t stream);

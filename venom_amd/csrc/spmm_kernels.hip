@@ -1520,6 +1520,91 @@ static hipError_t launch_wst(const SpmmParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// Row-major write-out of one wave's 64 x 64 block through a column-major LDS slab.
+// A lane holds, per (mb, nb), rows 16*ib + 4*mb + r (r = 0..3) of column nb*16 + j16: four
+// consecutive slab rows q = 4*ib + r of one column, i.e. ONE 8-byte LDS write into slab[col][q]
+// (TR_PITCH bytes per column).  The transposing read gives result lanes 4k..4k+3 of a 16-lane
+// block the four halfs of the 8-byte chunks that lanes k, 4+k, 8+k, 12+k address, so the chunk
+// addresses are chosen per lane such that result lane (kb, 4k+x) ends up with slab row
+// 8*s + 4*(k%2) + x and columns 8*(2*kb + k/2) .. +3 (+4 for the second read): one global store
+// instruction then covers 8 rows x 128 contiguous bytes.
+// Development-only cycle accounting (compiled in with -DSPATHA_DEV_PROFILE): each consumer wave sums the
+// s_memtime ticks it spends (0) computing, (1) waiting at the step barrier, (2) in the write-out, and
+// lane 0 writes the three sums to prof[(block * 16 + wave) * 4 ..].
+#ifdef SPATHA_DEV_PROFILE
+#define SPATHA_PROF_DECL long long prof_t = __builtin_readcyclecounter(), prof_sum[3] = {0, 0, 0};
+#define SPATHA_PROF_MARK(SLOT)                                   \
+    {                                                            \
+        const long long now = __builtin_readcyclecounter();      \
+        prof_sum[SLOT] += now - prof_t;                          \
+        prof_t = now;                                            \
+    }
+#define SPATHA_PROF_FLUSH                                                                 \
+    if (p.prof && lane == 0) {                                                            \
+        long long* dst = p.prof + ((int64_t)blockIdx.x * 16 + wave) * 4;                  \
+        dst[0] = prof_sum[0];                                                             \
+        dst[1] = prof_sum[1];                                                             \
+        dst[2] = prof_sum[2];                                                             \
+    }
+#else
+#define SPATHA_PROF_DECL
+#define SPATHA_PROF_MARK(SLOT)
+#define SPATHA_PROF_FLUSH
+#endif
+
+constexpr int TR_PITCH = 40;                       // 16 rows x 2 B + 8 B pad
+constexpr int TR_SLAB_BYTES = 64 * TR_PITCH;       // per wave, all 16 slab rows at once
+constexpr int TR8_PITCH = 16;                      // 8 rows x 2 B
+constexpr int TR8_SLAB_BYTES = 64 * TR8_PITCH;     // per wave, 8 slab rows at a time (ROWS8: half the lanes write)
+template <bool ROWS8>
+__device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4][4], char* stg, uint16_t* C, int64_t row0,
+                                                         int col0, int N, int lane, bool stores_on) {
+    constexpr int PITCH = ROWS8 ? TR8_PITCH : TR_PITCH;
+    const int j16 = lane & 15, ib = lane >> 4;     // as accumulator lane: column j16, rows 4*ib + r
+    const int li = lane & 15, kb = lane >> 4;
+    // as chunk supplier: source row e = li/4, chunk k = li%4
+    const int rd_off = (8 * (2 * kb + ((li & 3) >> 1)) + (li >> 2)) * PITCH + (li & 1) * 8;
+    // as result lane: k = li/4, x = li%4
+    const int q_lo = 4 * ((li >> 2) & 1) + (li & 3);
+    const int out_col = col0 + 8 * (2 * kb + (li >> 3));
+#pragma unroll
+    for (int mb = 0; mb < 4; mb++) {
+        half4_t h4[4];
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) h4[nb][r] = (_Float16)acc[mb][nb][r];
+        if (!ROWS8) {
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++) *(half4_t*)(stg + (nb * 16 + j16) * PITCH + ib * 8) = h4[nb];
+            __builtin_amdgcn_wave_barrier();
+        }
+#pragma unroll
+        for (int sidx = 0; sidx < 2; sidx++) {
+            if (ROWS8) {
+                if ((ib >> 1) == sidx) {
+#pragma unroll
+                    for (int nb = 0; nb < 4; nb++) *(half4_t*)(stg + (nb * 16 + j16) * PITCH + (ib & 1) * 8) = h4[nb];
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+            const int roff = rd_off + (ROWS8 ? 0 : sidx * 16);
+            short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff));
+            short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff + 4 * PITCH));
+            u32x4 v;
+            v.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+            v.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+            v.z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+            v.w = (uint32_t)(uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+            const int q = 8 * sidx + q_lo;
+            const int row = 16 * (q >> 2) + 4 * mb + (q & 3);
+            if (out_col < N && stores_on) *(u32x4*)(C + (row0 + row) * N + out_col) = v;
+            if (ROWS8) __builtin_amdgcn_wave_barrier();
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Dense-staged kernel for m <= 8 (tile 256 x 128 = four 64-row blocks; pays off most at V = 64).
 //
@@ -1531,20 +1616,23 @@ static hipError_t launch_wst(const SpmmParams& p, hipStream_t stream) {
 // read for each of its four fragments (row * 256 + swizzle), built once per matrix.
 // Rows beyond K come back as zeros from the buffer bounds check, so padding groups (whose
 // column offsets are 0) and tail groups need no special case.
-// Consumer w owns rows 128*(w/2) .. +127 (two V blocks, one per 64-row half) x columns
-// 64*(w%2) .. +63.  Producers need no row table: B rows are consecutive.
+// With four consumer waves, wave w owns rows 128*(w/2) .. +127 (two 64-row blocks) x columns
+// 64*(w%2) .. +63; with eight, rows 64*(w/2) .. +63 (two waves per SIMD hide each other's LDS
+// latency and barrier waits).  Producers need no row table: B rows are consecutive.
 // ---------------------------------------------------------------------------
-template <int M, int NS, int NP>
+template <int M, int NS, int NP, int NC_>
 struct DsCfg {
-    static constexpr int NC = 4;
+    static constexpr int NC = NC_;                 // consumer waves: 4 (128 x 64 each) or 8 (64 x 64 each)
+    static constexpr int H = 8 / NC;               // 64-row blocks per consumer wave
+    static_assert(NC == 4 || NC == 8, "consumer waves");
     static constexpr int BM = 256, BN = 128;
     static constexpr int ROW_BYTES = BN * 2;
     static constexpr int DENSE_ROWS = 16 * M;
     static constexpr int B_BYTES = DENSE_ROWS * ROW_BYTES;
     static constexpr int STAGE_BYTES = B_BYTES + 4 * APACK_BLOCK;
     static constexpr int PA = NS - 1;
-    static constexpr int EPI_PITCH = 144;
-    static constexpr int EPI_BYTES = NC * 16 * EPI_PITCH;
+    static constexpr int SLAB_BYTES = NC == 4 ? TR_SLAB_BYTES : TR8_SLAB_BYTES;
+    static constexpr int EPI_BYTES = NC * SLAB_BYTES;
     static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
     static constexpr int LDS_BYTES = NS * STAGE_BYTES + EPI_BYTES;
     static constexpr int THREADS = (NC + NP) * 64;
@@ -1628,33 +1716,34 @@ template <class Cfg, int OUT_LAYOUT>
 __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
     constexpr int B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
-    constexpr int EPI_PITCH = Cfg::EPI_PITCH;
     const int S = p.S, N = p.N;
-    const int wm2 = wave >> 1, wn = wave & 1;
-    float4_t acc[2][4][4];
+    constexpr int H = Cfg::H;
+    const int rb0 = (wave >> 1) * H, wn = wave & 1;      // first 64-row block of this wave, column half
+    float4_t acc[H][4][4];
     const int li = lane & 15, kb = lane >> 4;
     // fixed part of a transposing-read address: column chunk (wn*8 + (li%4)/2) and the 8-byte half
     const uint32_t col_xor = (uint32_t)((wn * 8 + ((li & 3) >> 1)) << 4);
     const uint32_t col_or = (uint32_t)(li & 1) * 8u;
-    const int a_off = B_BYTES + (wm2 * 2) * APACK_BLOCK + lane * 16;
-    const int i_off = B_BYTES + (wm2 * 2) * APACK_BLOCK + 4096 + lane * 4;
+    const int a_off = B_BYTES + rb0 * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + rb0 * APACK_BLOCK + 4096 + lane * 4;
     const int j16 = lane & 15, ib = lane >> 4;
     // gather table: [64-row block][step][kb][c = (li/4)][fb] u16 -> this lane's 8 bytes per (block, step)
     const int lane_class = kb * 4 + (li >> 2);
     auto gtab_ptr = [&](int tm, int h, int step) {
-        const int64_t vb = (int64_t)tm * 4 + wm2 * 2 + h;
+        const int64_t vb = (int64_t)tm * 4 + rb0 + h;
         return (const u32x2*)(p.gtab + ((vb * S + step) * 16 + lane_class) * 4);
     };
 
     int c_tm = walk.tm0, c_tn = walk.tn0;
     int n_tm = c_tm, n_tn = c_tn;       // tile of the NEXT step's table entries
+    SPATHA_PROF_DECL
     uint32_t c_stage = 0;
-    u32x2 g_cur[2], g_next[2];
-    g_cur[0] = *gtab_ptr(c_tm, 0, 0);
-    g_cur[1] = *gtab_ptr(c_tm, 1, 0);
+    u32x2 g_cur[H], g_next[H];
+#pragma unroll
+    for (int h = 0; h < H; h++) g_cur[h] = *gtab_ptr(c_tm, h, 0);
     for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
 #pragma unroll
-        for (int h = 0; h < 2; h++)
+        for (int h = 0; h < H; h++)
 #pragma unroll
             for (int a = 0; a < 4; a++)
 #pragma unroll
@@ -1666,13 +1755,15 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
                 ns = 0;
                 if (c_tile + 1 < walk.my_tiles) walk.next(n_tm, n_tn);
             }
-            g_next[0] = *gtab_ptr(n_tm, 0, ns);
-            g_next[1] = *gtab_ptr(n_tm, 1, ns);
+#pragma unroll
+            for (int h = 0; h < H; h++) g_next[h] = *gtab_ptr(n_tm, h, ns);
+            SPATHA_PROF_MARK(0)
             __syncthreads();
+            SPATHA_PROF_MARK(1)
             if (!(p.debug & 16)) {
                 const char* st = smem + c_stage;
 #pragma unroll
-                for (int h = 0; h < 2; h++) {
+                for (int h = 0; h < H; h++) {
                     half8_t a_cur[4];
 #pragma unroll
                     for (int mb = 0; mb < 4; mb++) a_cur[mb] = *(const half8_t*)(st + a_off + h * APACK_BLOCK + mb * 1024);
@@ -1718,12 +1809,13 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
                 }
             }
             c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
-            g_cur[0] = g_next[0];
-            g_cur[1] = g_next[1];
-        }
-        const int cm0 = c_tm * BM + wm2 * 128, cn0 = c_tn * BN;
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
+            for (int h = 0; h < H; h++) g_cur[h] = g_next[h];
+        }
+        const int cm0 = c_tm * BM + rb0 * 64, cn0 = c_tn * BN;
+        SPATHA_PROF_MARK(0)
+#pragma unroll
+        for (int h = 0; h < H; h++) {
             if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
                 const int64_t row0 = (int64_t)cm0 + h * 64 + ib * 16;
                 half8_t bias_lo, bias_hi;
@@ -1753,34 +1845,212 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
                     }
                 }
             } else if (!(p.debug & 4)) {
-                char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
-#pragma unroll
-                for (int mb = 0; mb < 4; mb++) {
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-#pragma unroll
-                        for (int nb = 0; nb < 4; nb++)
-                            *(_Float16*)(stg + (r * 4 + ib) * EPI_PITCH + (nb * 16 + j16) * 2) = (_Float16)acc[h][mb][nb][r];
-                    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-                    for (int it = 0; it < 2; it++) {
-                        const int Lr = it * 8 + (lane >> 3), ch = lane & 7;
-                        const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
-                        const int col = cn0 + wn * 64 + ch * 8;
-                        u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
-                        if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)cm0 + h * 64 + row) * N + col) = v;
-                    }
-                    __builtin_amdgcn_wave_barrier();
-                }
+                store_block_row_major_tr<Cfg::NC == 8>(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C,
+                                                        (int64_t)cm0 + h * 64, cn0 + wn * 64, N, lane, !(p.debug & 2));
             }
         }
+        SPATHA_PROF_MARK(2)
         walk.next(c_tm, c_tn);
     }
+    SPATHA_PROF_FLUSH
+}
+
+// Ping-pong consumer of the dense-staged kernel (eight 64 x 64 consumer waves, two per SIMD).
+// Waves 0-3 ("early") read a stage's operands right after its barrier and multiply as the
+// fragments arrive.  Waves 4-7 ("late") run one phase behind: after the barrier of step s they
+// first issue the 16 matrix instructions of step s-1 from registers, re-loading each fragment's
+// registers from stage s as soon as the instructions that read it are issued, and reach the
+// next barrier once stage s sits in registers.  On every SIMD one wave's LDS latency is thus
+// covered by the other wave's matrix work, with a single register set per wave.
+template <class Cfg, int OUT_LAYOUT, bool LATE>
+__device__ __forceinline__ void ds_consumer_pp(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+    static_assert(Cfg::NC == 8, "ping-pong needs two consumer waves per SIMD");
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
+    constexpr int B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    const int S = p.S, N = p.N;
+    const int rb0 = wave & 3, wn = (wave >> 2) & 1;      // 64-row block, column half (= phase group)
+    float4_t acc[4][4];
+    SPATHA_PROF_DECL
+    const int li = lane & 15, kb = lane >> 4;
+    const uint32_t col_xor = (uint32_t)((wn * 8 + ((li & 3) >> 1)) << 4);
+    const uint32_t col_or = (uint32_t)(li & 1) * 8u;
+    const int a_off = B_BYTES + rb0 * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + rb0 * APACK_BLOCK + 4096 + lane * 4;
+    const int j16 = lane & 15, ib = lane >> 4;
+    const int lane_class = kb * 4 + (li >> 2);
+    auto gtab_ptr = [&](int tm, int step) {
+        const int64_t vb = (int64_t)tm * 4 + rb0;
+        return (const u32x2*)(p.gtab + ((vb * S + step) * 16 + lane_class) * 4);
+    };
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    };
+    half8_t a_cur[4];
+    uint32_t i0 = 0, i1 = 0;
+    half16_t bf[4];
+    uint32_t base[4];
+    auto set_base = [&](u32x2 g) {
+        base[0] = ((g.x & 0xffffu) ^ col_xor) | col_or;
+        base[1] = ((g.x >> 16) ^ col_xor) | col_or;
+        base[2] = ((g.y & 0xffffu) ^ col_xor) | col_or;
+        base[3] = ((g.y >> 16) ^ col_xor) | col_or;
+    };
+    auto read_frag = [&](const char* st, int nb) {
+#pragma unroll
+        for (int fb = 0; fb < 4; fb++) {
+            short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, st + (base[fb] ^ (uint32_t)(nb << 5))));
+            half4_t h4 = __builtin_bit_cast(half4_t, t4);
+            bf[nb][fb * 4 + 0] = h4[0];
+            bf[nb][fb * 4 + 1] = h4[1];
+            bf[nb][fb * 4 + 2] = h4[2];
+            bf[nb][fb * 4 + 3] = h4[3];
+        }
+    };
+    auto read_a = [&](const char* st) {
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) a_cur[mb] = *(const half8_t*)(st + a_off + mb * 1024);
+        i0 = *(const uint32_t*)(st + i_off);
+        i1 = *(const uint32_t*)(st + i_off + 256);
+    };
+#define SPATHA_MMA4P(NB)                                                                                         \
+    acc[0][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[0], bf[NB], acc[0][NB], (int)i0, 0, 0);          \
+    acc[1][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], bf[NB], acc[1][NB], (int)i0, 0, 1);          \
+    acc[2][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], bf[NB], acc[2][NB], (int)i1, 0, 0);          \
+    acc[3][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], bf[NB], acc[3][NB], (int)i1, 0, 1);
+    auto write_out = [&](int tm, int tn) {
+        const int cm0 = tm * BM + rb0 * 64, cn0 = tn * BN;
+        SPATHA_PROF_MARK(0)
+        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+            const int64_t row0 = (int64_t)cm0 + ib * 16;
+            half8_t bias_lo, bias_hi;
+            if (p.bias) {
+                bias_lo = *(const half8_t*)(p.bias + row0);
+                bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+            }
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++) {
+                const int col = cn0 + wn * 64 + nb * 16 + j16;
+                half8_t lo, hi;
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
+                        hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
+                    }
+                if (p.bias) {
+                    lo = lo + bias_lo;
+                    hi = hi + bias_hi;
+                }
+                if (col < N && !(p.debug & 2)) {
+                    uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
+                    *(half8_t*)dst = lo;
+                    *(half8_t*)(dst + 8) = hi;
+                }
+            }
+        } else if (!(p.debug & 4)) {
+            store_block_row_major_tr<true>(acc, smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, (int64_t)cm0,
+                                           cn0 + wn * 64, N, lane, !(p.debug & 2));
+        }
+        SPATHA_PROF_MARK(2)
+    };
+
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    int n_tm = c_tm, n_tn = c_tn;       // tile of the NEXT step's table entries
+    int o_tm = c_tm, o_tn = c_tn;       // late waves: tile whose last step is still in registers
+    uint32_t c_stage = 0;
+    u32x2 g_next = *gtab_ptr(c_tm, 0);
+    set_base(g_next);
+    zero_acc();
+    if (LATE) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            a_cur[k] = (half8_t)(_Float16)0.f;
+            bf[k] = (half16_t)(_Float16)0.f;
+        }
+    }
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+        for (int c_step = 0; c_step < S; c_step++) {
+            int ns = c_step + 1;
+            if (ns == S) {
+                ns = 0;
+                if (c_tile + 1 < walk.my_tiles) walk.next(n_tm, n_tn);
+            }
+            g_next = *gtab_ptr(n_tm, ns);
+            SPATHA_PROF_MARK(0)
+            __syncthreads();
+            SPATHA_PROF_MARK(1)
+            const char* st = smem + c_stage;
+            if (!LATE) {
+                if (!(p.debug & 16)) {
+                    read_a(st);
+                    read_frag(st, 0);
+                    read_frag(st, 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    SPATHA_MMA4P(0)
+                    __builtin_amdgcn_sched_barrier(0);
+                    read_frag(st, 2);
+                    __builtin_amdgcn_sched_barrier(0);
+                    SPATHA_MMA4P(1)
+                    __builtin_amdgcn_sched_barrier(0);
+                    read_frag(st, 3);
+                    __builtin_amdgcn_sched_barrier(0);
+                    SPATHA_MMA4P(2)
+                    SPATHA_MMA4P(3)
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else if (!(p.debug & 16)) {
+                // registers hold the previous step (all zeros before the first one)
+                SPATHA_MMA4P(0)
+                __builtin_amdgcn_sched_barrier(0);
+                read_frag(st, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                SPATHA_MMA4P(1)
+                __builtin_amdgcn_sched_barrier(0);
+                read_frag(st, 1);
+                __builtin_amdgcn_sched_barrier(0);
+                SPATHA_MMA4P(2)
+                __builtin_amdgcn_sched_barrier(0);
+                read_frag(st, 2);
+                __builtin_amdgcn_sched_barrier(0);
+                SPATHA_MMA4P(3)
+                __builtin_amdgcn_sched_barrier(0);
+                read_frag(st, 3);
+                read_a(st);
+                __builtin_amdgcn_sched_barrier(0);
+                if (c_step == 0 && c_tile > 0) {
+                    // that was the last step of the previous tile
+                    write_out(o_tm, o_tn);
+                    zero_acc();
+                }
+                o_tm = c_tm;
+                o_tn = c_tn;
+            }
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+            set_base(g_next);
+        }
+        if (!LATE) write_out(c_tm, c_tn), zero_acc();
+        walk.next(c_tm, c_tn);
+    }
+    if (LATE) {
+        if (!(p.debug & 16)) {
+            SPATHA_MMA4P(0)
+            SPATHA_MMA4P(1)
+            SPATHA_MMA4P(2)
+            SPATHA_MMA4P(3)
+        }
+        write_out(o_tm, o_tn);
+    }
+#undef SPATHA_MMA4P
+    SPATHA_PROF_FLUSH
 }
 
 template <int M, int NS, int NP, int OUT_LAYOUT>
-__global__ __launch_bounds__((4 + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
-    using Cfg = DsCfg<M, NS, NP>;
+__global__ __launch_bounds__((8 + NP) * 64) void spmm_dspp_kernel(SpmmParams p) {
+    using Cfg = DsCfg<M, NS, NP, 8>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1789,9 +2059,11 @@ __global__ __launch_bounds__((4 + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
     if (wave < 4) {
-        ds_consumer<Cfg, OUT_LAYOUT>(p, walk, smem, wave, lane);
+        ds_consumer_pp<Cfg, OUT_LAYOUT, false>(p, walk, smem, wave, lane);
+    } else if (wave < 8) {
+        ds_consumer_pp<Cfg, OUT_LAYOUT, true>(p, walk, smem, wave, lane);
     } else {
-        const int pr = wave - 4;
+        const int pr = wave - 8;
         if (pr == 0) ds_producer<Cfg, M, NP, 0>(p, walk, smem_base, lane);
         else if (pr == 1) ds_producer<Cfg, M, NP, 1>(p, walk, smem_base, lane);
         else if (pr == 2) ds_producer<Cfg, M, NP, 2>(p, walk, smem_base, lane);
@@ -1799,14 +2071,38 @@ __global__ __launch_bounds__((4 + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
     }
 }
 
-template <int M, int NS, int NP, int OUT_LAYOUT>
+template <int M, int NS, int NP, int NC, int OUT_LAYOUT>
+__global__ __launch_bounds__((NC + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
+    using Cfg = DsCfg<M, NS, NP, NC>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TileWalk walk;
+    walk.init(p.tiles_m, p.tiles_n);
+    if (walk.my_tiles == 0) return;
+    if (wave < NC) {
+        ds_consumer<Cfg, OUT_LAYOUT>(p, walk, smem, wave, lane);
+    } else {
+        const int pr = wave - NC;
+        if (pr == 0) ds_producer<Cfg, M, NP, 0>(p, walk, smem_base, lane);
+        else if (pr == 1) ds_producer<Cfg, M, NP, 1>(p, walk, smem_base, lane);
+        else if (pr == 2) ds_producer<Cfg, M, NP, 2>(p, walk, smem_base, lane);
+        else ds_producer<Cfg, M, NP, 3>(p, walk, smem_base, lane);
+    }
+}
+
+template <int M, int NS, int NP, int NC, int OUT_LAYOUT, bool PINGPONG = false>
 static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
-    using Cfg = DsCfg<M, NS, NP>;
+    using Cfg = DsCfg<M, NS, NP, NC>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
+    static_assert(!PINGPONG || NC == 8, "ping-pong needs eight consumer waves");
     static bool attr_set = false;
     static int cus = 0;
-    auto kern = spmm_ds_kernel<M, NS, NP, OUT_LAYOUT>;
+    void (*kern)(SpmmParams);
+    if constexpr (PINGPONG) kern = spmm_dspp_kernel<M, NS, NP, OUT_LAYOUT>;
+    else kern = spmm_ds_kernel<M, NS, NP, NC, OUT_LAYOUT>;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
@@ -1821,6 +2117,321 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
     if (grid > need) grid = need;
     if (grid < 8) grid = 8;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::THREADS), lds, stream, p);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Dense-staged kernel without workgroup barriers in the main loop ("flag-synchronised").
+//
+// A step of the barrier-synchronised kernels above costs the matrix pipes several hundred idle
+// clocks: every wave has to issue its last instruction of the step before any wave may start the
+// next one.  Here each stage of the ring carries two monotonic counters in LDS instead:
+//   full[stage]  += 1 by every producer wave once its share of the stage has landed (vmcnt),
+//   empty[stage] += 1 by every consumer wave once it has read the stage into registers.
+// A consumer polls full >= NP * (use + 1) before reading, a producer polls empty >= NC * use
+// before overwriting, so waves only ever wait for data, never for each other.  Polls are
+// bounded (SPIN_LIMIT) so that a logic error ends in wrong results, not in a hang.
+// The gather table travels with the stage (512 B per k-step, tile-major copy of it), so consumer
+// waves issue no global loads at all and never wait for their own stores.
+// ---------------------------------------------------------------------------
+constexpr int SPIN_LIMIT = 1 << 20;
+
+__device__ __forceinline__ void flag_wait(uint32_t lds_addr, uint32_t target) {
+    for (int spin = 0; spin < SPIN_LIMIT; spin++) {
+        uint32_t v;
+        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_addr) : "memory");
+        if ((int)((uint32_t)__builtin_amdgcn_readfirstlane((int)v) - target) >= 0) break;
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
+// all LDS reads of this wave have landed -> bump the counter (one lane)
+__device__ __forceinline__ void flag_signal(uint32_t lds_addr, int lane) {
+    if (lane == 0) {
+        const uint32_t one = 1;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\tds_add_u32 %0, %1" ::"v"(lds_addr), "v"(one) : "memory");
+    }
+}
+
+template <int M, int NS, int NP>
+struct DsfCfg {
+    static constexpr int NC = 8;
+    static constexpr int BM = 256, BN = 128;
+    static constexpr int B_BYTES = 16 * M * BN * 2;
+    static constexpr int GT_OFF = B_BYTES + 4 * APACK_BLOCK;
+    static constexpr int GT_BYTES = 512;
+    static constexpr int STAGE_BYTES = GT_OFF + GT_BYTES;
+    static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
+    static constexpr int EPI_BYTES = NC * TR8_SLAB_BYTES;
+    static constexpr uint32_t FLAG_BASE = EPI_BASE + EPI_BYTES;     // full[NS], empty[NS]
+    static constexpr int LDS_BYTES = FLAG_BASE + 64;
+    static constexpr int THREADS = (NC + NP) * 64;
+};
+
+template <class Cfg, int M, int NS, int NP, int PR>
+__device__ __forceinline__ void dsf_producer(const SpmmParams& p, const TileWalk& walk, uint32_t smem_base, int lane) {
+    constexpr int BN = Cfg::BN;
+    constexpr int B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int NB_LOADS = (4 * M) / NP;
+    constexpr int NA_LOADS = 24 / NP;
+    constexpr int NG_LOADS = PR < 2 ? 1 : 0;         // the 512-byte gather table slice: two 256-byte pieces
+    constexpr int LOADS = NB_LOADS + NA_LOADS + NG_LOADS;
+    static_assert((4 * M) % NP == 0 && 24 % NP == 0 && NP >= 2, "DMA work must split evenly over the producers");
+    const int S = p.S, N = p.N;
+    const int Q = walk.my_tiles * S;
+    const i32x4 rsrc_b = make_buffer(p.B, p.b_bytes);
+    const i32x4 rsrc_a = make_buffer(p.apack, p.apack_bytes);
+    const i32x4 rsrc_g = make_buffer(p.gtab_tiles, p.gtab_tiles_bytes);
+    const uint32_t row_bytes_b = (uint32_t)N * 2u;
+    const int dense_rows = 16 * p.m;
+    const uint32_t step_bytes_b = (uint32_t)dense_rows * row_bytes_b;
+    const int slot_row = lane >> 4, slot_chunk = lane & 15;
+    const uint32_t lane16 = lane * 16, lane4 = lane * 4;
+    const uint32_t full_base = smem_base + Cfg::FLAG_BASE, empty_base = full_base + NS * 4;
+
+    int is_tm = walk.tm0, is_tn = walk.tn0, is_step = 0;
+    uint32_t b_soff = 0;
+    uint32_t a_soff = (uint32_t)((is_tm * 4) * S) * (uint32_t)APACK_BLOCK;
+    uint32_t g_soff = (uint32_t)(is_tm * S) * 512u + PR * 256u;
+    uint32_t voff[NB_LOADS];
+    auto set_voff = [&]() {
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) {
+            const int row = (PR * NB_LOADS + j) * 4 + slot_row;
+            const int col = is_tn * BN + (slot_chunk ^ ((row & 7) << 1)) * 8;
+            voff[j] = (col < N && row < dense_rows && !(p.debug & 1)) ? (uint32_t)row * row_bytes_b + (uint32_t)col * 2u
+                                                                       : 0xF0000000u;
+        }
+    };
+    set_voff();
+    int st = 0, prev_st = 0;            // ring slot of the batch being issued / of the one before it
+    uint32_t use = 0;                   // how often slot `st` has been filled before
+    for (int q = 0; q < Q; q++) {
+        if (use > 0) flag_wait(empty_base + st * 4, (uint32_t)Cfg::NC * use);
+        if (!(p.debug & 8)) {
+            const uint32_t stage = smem_base + st * STAGE_BYTES;
+#pragma unroll
+            for (int j = 0; j < NB_LOADS; j++) bdma_b128(voff[j], rsrc_b, b_soff, stage + (PR * NB_LOADS + j) * 1024);
+#pragma unroll
+            for (int k = 0; k < NA_LOADS; k++) {
+                const int a = PR * NA_LOADS + k;
+                const int awm = a / 6, ak = a - awm * 6;
+                const uint32_t soff = a_soff + (uint32_t)(awm * S) * (uint32_t)APACK_BLOCK;
+                const uint32_t dst = stage + B_BYTES + awm * APACK_BLOCK;
+                if (ak < 4) bdma_b128(lane16, rsrc_a, soff + ak * 1024, dst + ak * 1024);
+                else bdma_b32(lane4, rsrc_a, soff + 4096 + (ak - 4) * 256, dst + 4096 + (ak - 4) * 256);
+            }
+            if (NG_LOADS) bdma_b32(lane4, rsrc_g, g_soff, stage + Cfg::GT_OFF + PR * 256);
+        }
+        a_soff += (uint32_t)APACK_BLOCK;
+        b_soff += step_bytes_b;
+        g_soff += 512u;
+        if (++is_step == S) {
+            is_step = 0;
+            b_soff = 0;
+            walk.next(is_tm, is_tn);
+            a_soff = (uint32_t)((is_tm * 4) * S) * (uint32_t)APACK_BLOCK;
+            g_soff = (uint32_t)(is_tm * S) * 512u + PR * 256u;
+            set_voff();
+        }
+        if (q > 0) {
+            // everything but the batch just issued has landed: publish the previous batch
+            if (!(p.debug & 8)) wait_vmcnt<LOADS>();
+            flag_signal(full_base + prev_st * 4, lane);
+        }
+        prev_st = st;
+        if (++st == NS) {
+            st = 0;
+            ++use;
+        }
+    }
+    wait_vmcnt<0>();
+    if (Q > 0) flag_signal(full_base + prev_st * 4, lane);
+}
+
+template <class Cfg, int NS, int NP, int OUT_LAYOUT>
+__device__ __forceinline__ void dsf_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, uint32_t smem_base,
+                                             int wave, int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN;
+    constexpr int B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    const int S = p.S, N = p.N;
+    const int rb0 = wave & 3, wn = (wave >> 2) & 1;      // 64-row block, column half
+    float4_t acc[4][4];
+    SPATHA_PROF_DECL
+    const int li = lane & 15, kb = lane >> 4;
+    const uint32_t col_xor = (uint32_t)((wn * 8 + ((li & 3) >> 1)) << 4);
+    const uint32_t col_or = (uint32_t)(li & 1) * 8u;
+    const int a_off = B_BYTES + rb0 * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + rb0 * APACK_BLOCK + 4096 + lane * 4;
+    const int g_off = Cfg::GT_OFF + rb0 * 128 + (kb * 4 + (li >> 2)) * 8;
+    const int j16 = lane & 15, ib = lane >> 4;
+    const uint32_t full_base = smem_base + Cfg::FLAG_BASE, empty_base = full_base + NS * 4;
+
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    int st = 0;
+    uint32_t use = 0;
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            SPATHA_PROF_MARK(0)
+            flag_wait(full_base + st * 4, (uint32_t)NP * (use + 1));
+            SPATHA_PROF_MARK(1)
+            if (!(p.debug & 16)) {
+                const char* stg = smem + st * STAGE_BYTES;
+                const u32x2 g = *(const u32x2*)(stg + g_off);
+                half8_t a_cur[4];
+#pragma unroll
+                for (int mb = 0; mb < 4; mb++) a_cur[mb] = *(const half8_t*)(stg + a_off + mb * 1024);
+                const uint32_t i0 = *(const uint32_t*)(stg + i_off);
+                const uint32_t i1 = *(const uint32_t*)(stg + i_off + 256);
+                uint32_t base[4];
+                base[0] = ((g.x & 0xffffu) ^ col_xor) | col_or;
+                base[1] = ((g.x >> 16) ^ col_xor) | col_or;
+                base[2] = ((g.y & 0xffffu) ^ col_xor) | col_or;
+                base[3] = ((g.y >> 16) ^ col_xor) | col_or;
+                half16_t bf[4];
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++)
+#pragma unroll
+                    for (int fb = 0; fb < 4; fb++) {
+                        short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + (base[fb] ^ (uint32_t)(nb << 5))));
+                        half4_t h4 = __builtin_bit_cast(half4_t, t4);
+                        bf[nb][fb * 4 + 0] = h4[0];
+                        bf[nb][fb * 4 + 1] = h4[1];
+                        bf[nb][fb * 4 + 2] = h4[2];
+                        bf[nb][fb * 4 + 3] = h4[3];
+                    }
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++) {
+                    acc[0][nb] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[0], bf[nb], acc[0][nb], (int)i0, 0, 0);
+                    acc[1][nb] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], bf[nb], acc[1][nb], (int)i0, 0, 1);
+                    acc[2][nb] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], bf[nb], acc[2][nb], (int)i1, 0, 0);
+                    acc[3][nb] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], bf[nb], acc[3][nb], (int)i1, 0, 1);
+                }
+            }
+            flag_signal(empty_base + st * 4, lane);
+            if (++st == NS) {
+                st = 0;
+                ++use;
+            }
+        }
+        const int cm0 = c_tm * BM + rb0 * 64, cn0 = c_tn * BN;
+        SPATHA_PROF_MARK(0)
+        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+            const int64_t row0 = (int64_t)cm0 + ib * 16;
+            half8_t bias_lo, bias_hi;
+            if (p.bias) {
+                bias_lo = *(const half8_t*)(p.bias + row0);
+                bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+            }
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++) {
+                const int col = cn0 + wn * 64 + nb * 16 + j16;
+                half8_t lo, hi;
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
+                        hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
+                    }
+                if (p.bias) {
+                    lo = lo + bias_lo;
+                    hi = hi + bias_hi;
+                }
+                if (col < N && !(p.debug & 2)) {
+                    uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
+                    *(half8_t*)dst = lo;
+                    *(half8_t*)(dst + 8) = hi;
+                }
+            }
+        } else if (!(p.debug & 4)) {
+            store_block_row_major_tr<true>(acc, smem + Cfg::EPI_BASE + wave * TR8_SLAB_BYTES, p.C, (int64_t)cm0, cn0 + wn * 64,
+                                           N, lane, !(p.debug & 2));
+        }
+        SPATHA_PROF_MARK(2)
+        walk.next(c_tm, c_tn);
+    }
+    SPATHA_PROF_FLUSH
+}
+
+template <int M, int NS, int NP, int OUT_LAYOUT>
+__global__ __launch_bounds__((8 + NP) * 64) void spmm_dsf_kernel(SpmmParams p) {
+    using Cfg = DsfCfg<M, NS, NP>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TileWalk walk;
+    walk.init(p.tiles_m, p.tiles_n);
+    if (walk.my_tiles == 0) return;
+    if (tid < 16) *(uint32_t*)(smem + Cfg::FLAG_BASE + tid * 4) = 0u;
+    __syncthreads();
+    if (wave < 8) {
+        dsf_consumer<Cfg, NS, NP, OUT_LAYOUT>(p, walk, smem, smem_base, wave, lane);
+    } else {
+        const int pr = wave - 8;
+        if (pr == 0) dsf_producer<Cfg, M, NS, NP, 0>(p, walk, smem_base, lane);
+        else if (pr == 1) dsf_producer<Cfg, M, NS, NP, 1>(p, walk, smem_base, lane);
+        else if (pr == 2) dsf_producer<Cfg, M, NS, NP, 2>(p, walk, smem_base, lane);
+        else dsf_producer<Cfg, M, NS, NP, 3>(p, walk, smem_base, lane);
+    }
+}
+
+template <int M, int NS, int NP, int OUT_LAYOUT>
+static hipError_t launch_dsf(const SpmmParams& p, hipStream_t stream) {
+    using Cfg = DsfCfg<M, NS, NP>;
+    constexpr int lds = Cfg::LDS_BYTES;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static bool attr_set = false;
+    static int cus = 0;
+    auto kern = spmm_dsf_kernel<M, NS, NP, OUT_LAYOUT>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        int dev = 0;
+        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int tiles = p.tiles_m * p.tiles_n;
+    int grid = (cus / 8) * 8;
+    const int need = ((tiles + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    if (grid < 8) grid = 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::THREADS), lds, stream, p);
+    return hipGetLastError();
+}
+
+// tile-major copy of the gather table for the flag-synchronised kernel:
+// [256-row tile][step][64-row block in tile][kb][c][fb] u16, 512 contiguous bytes per (tile, step)
+__global__ void pack_gtab_tiles_kernel(const uint32_t* __restrict__ columns, int rows, int m, int v, int ksp, int S,
+                                       uint16_t* __restrict__ gtab) {
+    const int ngroups = ksp / 2;
+    const int64_t total = (int64_t)(rows / 256) * S * 256;
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
+        const int fb = (int)(t & 3), c = (int)((t >> 2) & 3), kb = (int)((t >> 4) & 3), rb = (int)((t >> 6) & 3);
+        const int64_t ts = t >> 8;
+        const int s = (int)(ts % S);
+        const int64_t tile = ts / S;
+        const int64_t b = (tile * 256 + rb * 64) / v;
+        const int gamma = fb * 4 + kb;
+        const int g = s * 16 + gamma;
+        uint32_t d = (uint32_t)gamma * m;
+        if (g < ngroups) d += columns[b * ngroups * 4 + (int64_t)g * 4 + c];
+        gtab[t] = (uint16_t)(d * 256u + (d & 7u) * 32u);
+    }
+}
+
+hipError_t launch_pack_gtab_tiles(const uint32_t* columns, int rows, int m, int v, int ksp, int S, uint16_t* gtab,
+                                  hipStream_t stream) {
+    int64_t total = (int64_t)(rows / 256) * S * 256;
+    int blocks = (int)((total + 255) / 256);
+    if (blocks > 65535 * 8) blocks = 65535 * 8;
+    hipLaunchKernelGGL(pack_gtab_tiles_kernel, dim3(blocks), dim3(256), 0, stream, columns, rows, m, v, ksp, S, gtab);
     return hipGetLastError();
 }
 
@@ -1962,6 +2573,9 @@ const char* spmm_variant_name(int variant) {
         case SPMM_VARIANT_T128x128_S5: return "smfmac16x16x64_warpspec_tall_tile128x128_5stage";
         case SPMM_VARIANT_DS256x128_S3: return "smfmac16x16x64_warpspec_densestage_tile256x128_3stage";
         case SPMM_VARIANT_DS256x128_S2: return "smfmac16x16x64_warpspec_densestage_tile256x128_2stage";
+        case SPMM_VARIANT_DS256x128_S3_C8: return "smfmac16x16x64_warpspec_densestage_tile256x128_3stage_8consumers";
+        case SPMM_VARIANT_DS256x128_S3_PP: return "smfmac16x16x64_warpspec_densestage_tile256x128_3stage_pingpong";
+        case SPMM_VARIANT_DSF256x128_S3: return "smfmac16x16x64_warpspec_densestage_flagsync_tile256x128_3stage";
         default: return nullptr;
     }
 }
@@ -1993,8 +2607,11 @@ int spmm_variant_lds(int variant, int S) {
         case SPMM_VARIANT_T128x256_S3: return WsCfg<2, 4, 3, 4>::LDS_BYTES;
         case SPMM_VARIANT_T128x128_S4: return WsCfg<2, 2, 4, 2>::LDS_BYTES;
         case SPMM_VARIANT_T128x128_S5: return WsCfg<2, 2, 5, 4>::LDS_BYTES;
-        case SPMM_VARIANT_DS256x128_S3: return DsCfg<8, 3, 4>::LDS_BYTES;
-        case SPMM_VARIANT_DS256x128_S2: return DsCfg<8, 2, 4>::LDS_BYTES;
+        case SPMM_VARIANT_DS256x128_S3: return DsCfg<8, 3, 4, 4>::LDS_BYTES;
+        case SPMM_VARIANT_DS256x128_S2: return DsCfg<8, 2, 4, 4>::LDS_BYTES;
+        case SPMM_VARIANT_DS256x128_S3_C8: return DsCfg<8, 3, 4, 8>::LDS_BYTES;
+        case SPMM_VARIANT_DS256x128_S3_PP: return DsCfg<8, 3, 4, 8>::LDS_BYTES;
+        case SPMM_VARIANT_DSF256x128_S3: return DsfCfg<8, 3, 4>::LDS_BYTES;
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_64x256: return 1;
         default: return 0;
     }
@@ -2009,7 +2626,7 @@ int spmm_variant_bm(int variant) {
         case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5: return 128;
         case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_D64x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 64;
-        case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: return 256;
+        case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3: return 256;
         default: return 0;
     }
 }
@@ -2019,7 +2636,7 @@ int spmm_variant_bn(int variant) {
         case SPMM_VARIANT_R128x128_S4: case SPMM_VARIANT_R128x128_S5: case SPMM_VARIANT_R128x128_S2:
         case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2:
         case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5:
-        case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: return 128;
+        case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3: return 128;
         case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D64x256_S3: case SPMM_VARIANT_T128x256_S3:
         case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_W128x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 256;
@@ -2085,12 +2702,20 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
     SPATHA_WST_CASE(SPMM_VARIANT_T128x128_S4, 2, 4, 2)
     SPATHA_WST_CASE(SPMM_VARIANT_T128x128_S5, 2, 5, 4)
 #undef SPATHA_WST_CASE
-    if (variant == SPMM_VARIANT_DS256x128_S3)
-        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ds<8, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
-                                                   : launch_ds<8, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
-    if (variant == SPMM_VARIANT_DS256x128_S2)
-        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ds<8, 2, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
-                                                   : launch_ds<8, 2, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
+#define SPATHA_DS_CASE(V, NS, NC)                                                                              \
+    if (variant == V)                                                                                          \
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ds<8, NS, 4, NC, SPATHA_OUT_TRANSPOSED>(p, stream) \
+                                                   : launch_ds<8, NS, 4, NC, SPATHA_OUT_ROW_MAJOR>(p, stream);
+    SPATHA_DS_CASE(SPMM_VARIANT_DS256x128_S3, 3, 4)
+    SPATHA_DS_CASE(SPMM_VARIANT_DS256x128_S2, 2, 4)
+    SPATHA_DS_CASE(SPMM_VARIANT_DS256x128_S3_C8, 3, 8)
+#undef SPATHA_DS_CASE
+    if (variant == SPMM_VARIANT_DSF256x128_S3)
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_dsf<8, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
+                                                   : launch_dsf<8, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
+    if (variant == SPMM_VARIANT_DS256x128_S3_PP)
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ds<8, 3, 4, 8, SPATHA_OUT_TRANSPOSED, true>(p, stream)
+                                                   : launch_ds<8, 3, 4, 8, SPATHA_OUT_ROW_MAJOR, true>(p, stream);
     return hipErrorInvalidValue;
 }
 

@@ -23,6 +23,13 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 SMFMAC_PEAK_TFLOPS = 5033.0    # fp16 MFMA with 2:4 structured sparsity (dense fp16 peak 2516.6 x 2)
 
 
+# HBM-side bytes per launch of the default workload's kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# scaled by a plain 256 MiB copy (summary under profiles/, named for the kernel); keyed by kernel name and shape.
+MEASURED_TRAFFIC_BYTES = {
+    ("smfmac16x16x64_warpspec_densestage_tile256x128_3stage_8consumers", 4096, 1024, 16384, 8, 64): 225_088_000,
+}
+
+
 def algorithmic_bytes(rows, cols, N, m, v, ksp):
     """values + metadata + column-loc (as stored) + B read once + C written once."""
     return 2 * rows * ksp + 4 * (rows // 2) * (ksp // 8) + 16 * (rows // v) * (ksp // 2) + 2 * cols * N + 2 * rows * N
@@ -41,6 +48,9 @@ def main():
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extra", action="store_true", help="also time the other BASELINE shapes (reported under 'extra')")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="before the benchmark, run 5 plain device copies of 256 MiB (a kernel of known HBM traffic, "
+                         "for scaling the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the SpMM path has no multi-GPU part); run with --gpus 1",
@@ -91,6 +101,14 @@ def main():
         t1 = time.perf_counter()
         return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
 
+    if args.copy_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     rows, cols, N, m, v = args.rows, args.cols, args.n, args.m, args.v
     w = prepare(rows, cols, N, m, v)
     ms_wall, ms_kernel = timed(w, args.steps, args.warmup, args.variant)
@@ -119,7 +137,8 @@ def main():
                    "kernel": w["plan"].kernel_name(N, 0, args.variant)},
         "pct_smfmac_peak": round(100.0 * flops_smfmac / (ms_kernel * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved_gbs / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((w["plan"].kernel_name(N, 0, args.variant), rows, cols, N, m, v)),
                      "algorithmic_bytes": nbytes, "kernel_us": round(ms_kernel * 1e3, 3)},
     }
 

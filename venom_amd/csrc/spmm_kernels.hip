@@ -2136,12 +2136,13 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
 // ---------------------------------------------------------------------------
 constexpr int SPIN_LIMIT = 1 << 20;
 
+template <int SLEEP = 1>
 __device__ __forceinline__ void flag_wait(uint32_t lds_addr, uint32_t target) {
     for (int spin = 0; spin < SPIN_LIMIT; spin++) {
         uint32_t v;
         asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_addr) : "memory");
         if ((int)((uint32_t)__builtin_amdgcn_readfirstlane((int)v) - target) >= 0) break;
-        __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_s_sleep(SLEEP);
     }
 }
 
@@ -2207,7 +2208,7 @@ __device__ __forceinline__ void dsf_producer(const SpmmParams& p, const TileWalk
     int st = 0, prev_st = 0;            // ring slot of the batch being issued / of the one before it
     uint32_t use = 0;                   // how often slot `st` has been filled before
     for (int q = 0; q < Q; q++) {
-        if (use > 0) flag_wait(empty_base + st * 4, (uint32_t)Cfg::NC * use);
+        if (use > 0) flag_wait<8>(empty_base + st * 4, (uint32_t)Cfg::NC * use);
         if (!(p.debug & 8)) {
             const uint32_t stage = smem_base + st * STAGE_BYTES;
 #pragma unroll
@@ -2249,12 +2250,20 @@ __device__ __forceinline__ void dsf_producer(const SpmmParams& p, const TileWalk
     if (Q > 0) flag_signal(full_base + prev_st * 4, lane);
 }
 
+// Consumer of the flag-synchronised kernel.  All operands are read one step ahead: while the 16
+// matrix instructions of step q issue, every fragment's registers are re-loaded from the stage
+// of step q+1 as soon as the instructions that read them are out, and the A operands follow
+// after the last one.  The scheduler is asked to alternate matrix instructions and LDS reads,
+// because a wave issues nothing else while it waits on a matrix instruction otherwise.
+// A stage is handed back to the producers as soon as it sits in registers, before it is
+// multiplied, and the next tile's first stage loads while this tile is written out.
 template <class Cfg, int NS, int NP, int OUT_LAYOUT>
 __device__ __forceinline__ void dsf_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, uint32_t smem_base,
                                              int wave, int lane) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN;
     constexpr int B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
     const int S = p.S, N = p.N;
+    const int Q = walk.my_tiles * S;
     const int rb0 = wave & 3, wn = (wave >> 2) & 1;      // 64-row block, column half
     float4_t acc[4][4];
     SPATHA_PROF_DECL
@@ -2267,94 +2276,137 @@ __device__ __forceinline__ void dsf_consumer(const SpmmParams& p, const TileWalk
     const int j16 = lane & 15, ib = lane >> 4;
     const uint32_t full_base = smem_base + Cfg::FLAG_BASE, empty_base = full_base + NS * 4;
 
-    int c_tm = walk.tm0, c_tn = walk.tn0;
-    int st = 0;
-    uint32_t use = 0;
-    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+    half8_t a_cur[4];
+    uint32_t i0, i1;
+    half16_t bf[4];
+    uint32_t base[4];
+    auto set_base = [&](u32x2 g) {
+        base[0] = ((g.x & 0xffffu) ^ col_xor) | col_or;
+        base[1] = ((g.x >> 16) ^ col_xor) | col_or;
+        base[2] = ((g.y & 0xffffu) ^ col_xor) | col_or;
+        base[3] = ((g.y >> 16) ^ col_xor) | col_or;
+    };
+    auto read_frag = [&](const char* stg, int nb) {
+#pragma unroll
+        for (int fb = 0; fb < 4; fb++) {
+            short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + (base[fb] ^ (uint32_t)(nb << 5))));
+            half4_t h4 = __builtin_bit_cast(half4_t, t4);
+            bf[nb][fb * 4 + 0] = h4[0];
+            bf[nb][fb * 4 + 1] = h4[1];
+            bf[nb][fb * 4 + 2] = h4[2];
+            bf[nb][fb * 4 + 3] = h4[3];
+        }
+    };
+    auto read_a = [&](const char* stg) {
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) a_cur[mb] = *(const half8_t*)(stg + a_off + mb * 1024);
+        i0 = *(const uint32_t*)(stg + i_off);
+        i1 = *(const uint32_t*)(stg + i_off + 256);
+    };
+#define SPATHA_MMA4F(NB)                                                                                 \
+    acc[0][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[0], bf[NB], acc[0][NB], (int)i0, 0, 0);  \
+    acc[1][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], bf[NB], acc[1][NB], (int)i0, 0, 1);  \
+    acc[2][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], bf[NB], acc[2][NB], (int)i1, 0, 0);  \
+    acc[3][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], bf[NB], acc[3][NB], (int)i1, 0, 1);
+    auto zero_acc = [&]() {
 #pragma unroll
         for (int a = 0; a < 4; a++)
 #pragma unroll
             for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
-        for (int c_step = 0; c_step < S; c_step++) {
+    };
+
+    int c_tm = walk.tm0, c_tn = walk.tn0, c_step = 0;
+    int st = 0;
+    uint32_t use = 0;
+    zero_acc();
+    // prologue: stage of step 0 into registers
+    flag_wait(full_base, (uint32_t)NP);
+    {
+        const char* stg = smem;
+        set_base(*(const u32x2*)(stg + g_off));
+        read_a(stg);
+        read_frag(stg, 0);
+        read_frag(stg, 1);
+        read_frag(stg, 2);
+        read_frag(stg, 3);
+    }
+    for (int q = 0; q < Q; q++) {
+        int nst = st + 1;
+        uint32_t nuse = use;
+        if (nst == NS) {
+            nst = 0;
+            ++nuse;
+        }
+        const bool have_next = q + 1 < Q;
+        SPATHA_PROF_MARK(0)
+        // the poll's wait also covers this step's operand reads; the last step just waits for them
+        if (have_next) flag_wait(full_base + nst * 4, (uint32_t)NP * (nuse + 1));
+        flag_signal(empty_base + st * 4, lane);
+        SPATHA_PROF_MARK(1)
+        // after the last step there is nothing to prefetch: re-read the current stage (never overwritten again)
+        const char* stg = smem + (have_next ? nst : st) * STAGE_BYTES;
+        __builtin_amdgcn_sched_barrier(0);
+        set_base(*(const u32x2*)(stg + g_off));
+        SPATHA_MMA4F(0)
+        read_frag(stg, 0);
+        SPATHA_MMA4F(1)
+        read_frag(stg, 1);
+        SPATHA_MMA4F(2)
+        read_frag(stg, 2);
+        SPATHA_MMA4F(3)
+        read_frag(stg, 3);
+        read_a(stg);
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 7, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        st = nst;
+        use = nuse;
+        if (++c_step == S) {
+            c_step = 0;
+            const int cm0 = c_tm * BM + rb0 * 64, cn0 = c_tn * BN;
             SPATHA_PROF_MARK(0)
-            flag_wait(full_base + st * 4, (uint32_t)NP * (use + 1));
-            SPATHA_PROF_MARK(1)
-            if (!(p.debug & 16)) {
-                const char* stg = smem + st * STAGE_BYTES;
-                const u32x2 g = *(const u32x2*)(stg + g_off);
-                half8_t a_cur[4];
-#pragma unroll
-                for (int mb = 0; mb < 4; mb++) a_cur[mb] = *(const half8_t*)(stg + a_off + mb * 1024);
-                const uint32_t i0 = *(const uint32_t*)(stg + i_off);
-                const uint32_t i1 = *(const uint32_t*)(stg + i_off + 256);
-                uint32_t base[4];
-                base[0] = ((g.x & 0xffffu) ^ col_xor) | col_or;
-                base[1] = ((g.x >> 16) ^ col_xor) | col_or;
-                base[2] = ((g.y & 0xffffu) ^ col_xor) | col_or;
-                base[3] = ((g.y >> 16) ^ col_xor) | col_or;
-                half16_t bf[4];
-#pragma unroll
-                for (int nb = 0; nb < 4; nb++)
-#pragma unroll
-                    for (int fb = 0; fb < 4; fb++) {
-                        short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + (base[fb] ^ (uint32_t)(nb << 5))));
-                        half4_t h4 = __builtin_bit_cast(half4_t, t4);
-                        bf[nb][fb * 4 + 0] = h4[0];
-                        bf[nb][fb * 4 + 1] = h4[1];
-                        bf[nb][fb * 4 + 2] = h4[2];
-                        bf[nb][fb * 4 + 3] = h4[3];
-                    }
+            if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+                const int64_t row0 = (int64_t)cm0 + ib * 16;
+                half8_t bias_lo, bias_hi;
+                if (p.bias) {
+                    bias_lo = *(const half8_t*)(p.bias + row0);
+                    bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+                }
 #pragma unroll
                 for (int nb = 0; nb < 4; nb++) {
-                    acc[0][nb] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[0], bf[nb], acc[0][nb], (int)i0, 0, 0);
-                    acc[1][nb] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], bf[nb], acc[1][nb], (int)i0, 0, 1);
-                    acc[2][nb] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], bf[nb], acc[2][nb], (int)i1, 0, 0);
-                    acc[3][nb] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], bf[nb], acc[3][nb], (int)i1, 0, 1);
-                }
-            }
-            flag_signal(empty_base + st * 4, lane);
-            if (++st == NS) {
-                st = 0;
-                ++use;
-            }
-        }
-        const int cm0 = c_tm * BM + rb0 * 64, cn0 = c_tn * BN;
-        SPATHA_PROF_MARK(0)
-        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
-            const int64_t row0 = (int64_t)cm0 + ib * 16;
-            half8_t bias_lo, bias_hi;
-            if (p.bias) {
-                bias_lo = *(const half8_t*)(p.bias + row0);
-                bias_hi = *(const half8_t*)(p.bias + row0 + 8);
-            }
+                    const int col = cn0 + wn * 64 + nb * 16 + j16;
+                    half8_t lo, hi;
 #pragma unroll
-            for (int nb = 0; nb < 4; nb++) {
-                const int col = cn0 + wn * 64 + nb * 16 + j16;
-                half8_t lo, hi;
+                    for (int mb = 0; mb < 2; mb++)
 #pragma unroll
-                for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
-                        hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
+                        for (int r = 0; r < 4; r++) {
+                            lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
+                            hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
+                        }
+                    if (p.bias) {
+                        lo = lo + bias_lo;
+                        hi = hi + bias_hi;
                     }
-                if (p.bias) {
-                    lo = lo + bias_lo;
-                    hi = hi + bias_hi;
+                    if (col < N && !(p.debug & 2)) {
+                        uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
+                        *(half8_t*)dst = lo;
+                        *(half8_t*)(dst + 8) = hi;
+                    }
                 }
-                if (col < N && !(p.debug & 2)) {
-                    uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
-                    *(half8_t*)dst = lo;
-                    *(half8_t*)(dst + 8) = hi;
-                }
+            } else if (!(p.debug & 4)) {
+                store_block_row_major_tr<true>(acc, smem + Cfg::EPI_BASE + wave * TR8_SLAB_BYTES, p.C, (int64_t)cm0,
+                                               cn0 + wn * 64, N, lane, !(p.debug & 2));
             }
-        } else if (!(p.debug & 4)) {
-            store_block_row_major_tr<true>(acc, smem + Cfg::EPI_BASE + wave * TR8_SLAB_BYTES, p.C, (int64_t)cm0, cn0 + wn * 64,
-                                           N, lane, !(p.debug & 2));
+            SPATHA_PROF_MARK(2)
+            zero_acc();
+            walk.next(c_tm, c_tn);
         }
-        SPATHA_PROF_MARK(2)
-        walk.next(c_tm, c_tn);
     }
+#undef SPATHA_MMA4F
     SPATHA_PROF_FLUSH
 }
 

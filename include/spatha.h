@@ -165,6 +165,12 @@ int spatha_spmm_time(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
 int spatha_dense_gemm_f16(const uint16_t* A_dev, const uint16_t* B_dev, int rows, int cols, int N, uint16_t* C_dev,
                           void* stream);
 
+/* out[cols x rows] = transpose of in[rows x cols], fp16, both row-major and 16-byte aligned.
+ * The PyTorch layer needs the activation as [in_features, tokens] for spatha_spmm_run; this replaces the
+ * `dense.contiguous()` of a transposed view in sparse_dense_mul_dispatch
+ * (end2end/bert_pytorch.py:85-87, called from SrnmSpmm.forward :126-136). */
+int spatha_transpose_f16(const uint16_t* in_dev, int rows, int cols, uint16_t* out_dev, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -75,3 +75,37 @@ def test_bert_encoder_swap_runs_and_tracks_masked_dense(gpu):
     b = model(ids).last_hidden_state.float()
     assert torch.isfinite(a).all()
     assert (a - b).abs().max().item() <= 5e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,cols", [(64, 64), (200, 328), (16384, 1024), (8, 4104), (37, 50)])
+def test_transpose_matches_torch(gpu, rows, cols):
+    from venom_amd import spatha
+    x = torch.randn((rows, cols), device=gpu).half()
+    assert torch.equal(spatha.transpose(x), x.T.contiguous())
+
+
+@pytest.mark.gpu
+def test_layer_reuses_transposed_input_only_for_the_same_activation(gpu):
+    """Projections of one activation share its transposed copy; a changed or new activation never hits it."""
+    from venom_amd import spatha
+    from venom_amd.bert import SrnmSpmm
+
+    torch.manual_seed(0)
+    sp = [SrnmSpmm(torch.nn.Linear(128, 64).half().to(gpu), 2, 8, 64) for _ in range(2)]
+
+    def direct(layer, x):       # the same product with the transposed copy made by torch
+        rhs = x.reshape(-1, 128).T.contiguous()
+        return spatha.spmm(layer.metadata, layer.columns, layer.values, rhs, layer.bias, 64, 128, rhs.shape[1], 64, 2, 8,
+                           layer.nnz, 0, 32, 4).reshape(4, 32, 64)
+
+    for trial in range(4):
+        x = torch.randn((4, 32, 128), device=gpu).half()
+        for layer in sp:
+            assert torch.equal(layer(x), direct(layer, x))
+        held = SrnmSpmm._last_rhs[2]
+        sp[1](x)
+        assert SrnmSpmm._last_rhs[2] is held            # second projection of the same activation: no new copy
+        x.mul_(2)                                       # in-place change: the version counter moves
+        assert torch.equal(sp[0](x), direct(sp[0], x))
+        del x                                           # the next trial may or may not get the same address

@@ -47,6 +47,7 @@ SIGNATURES = {
     "spatha_spmm_kernel_name": (c_char_p, [c_void_p, c_int, c_int, c_int]),
     "spatha_spmm_time": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, POINTER(c_float)]),
     "spatha_dense_gemm_f16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "spatha_transpose_f16": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
 }
 
 _lib = None

@@ -286,4 +286,12 @@ int spatha_dense_gemm_f16(const uint16_t* A_dev, const uint16_t* B_dev, int rows
     return e == hipSuccess ? SPATHA_OK : hip_fail(e);
 }
 
+int spatha_transpose_f16(const uint16_t* in_dev, int rows, int cols, uint16_t* out_dev, void* stream) {
+    if (!in_dev || !out_dev || rows <= 0 || cols <= 0) return SPATHA_ERR_BAD_ARGUMENT;
+    if (((uintptr_t)in_dev | (uintptr_t)out_dev) & 15u) return SPATHA_ERR_BAD_ARGUMENT;
+    if ((rows + 63) / 64 > 65535) return SPATHA_ERR_TOO_LARGE;
+    hipError_t e = spatha::launch_transpose_f16(in_dev, rows, cols, out_dev, (hipStream_t)stream);
+    return e == hipSuccess ? SPATHA_OK : hip_fail(e);
+}
+
 }  // extern "C"

@@ -120,6 +120,20 @@ def clear_plan_cache():
     _PLAN_CACHE.clear()
 
 
+def transpose(x):
+    """x[rows, cols] fp16, contiguous -> a new contiguous [cols, rows] tensor (what `x.T.contiguous()` returns),
+    through the library's tiled kernel on torch's current stream."""
+    _check_dev(x, torch.float16, "x")
+    if x.dim() != 2:
+        raise ValueError("transpose expects a matrix")
+    out = torch.empty((x.shape[1], x.shape[0]), dtype=torch.float16, device=x.device)
+    if x.numel():
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.lib().spatha_transpose_f16(x.data_ptr(), x.shape[0], x.shape[1], out.data_ptr(),
+                                                       _stream_ptr(x.device)), "spatha_transpose_f16")
+    return out
+
+
 def spmm(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_cols, B_num_cols, vec_length, n, m,
          nnz=0, seed=0, mbrow=32, brow=4):
     """out[B_num_cols, A_num_rows] = (A_vnm @ rhs_matrix).T + bias, fp16.

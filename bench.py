@@ -48,6 +48,8 @@ def main():
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extra", action="store_true", help="also time the other BASELINE shapes (reported under 'extra')")
+    ap.add_argument("--gpt3", action="store_true",
+                    help="also time the GPT-3 FFN shapes (A 49152x12288 128:2:16, N in 16/256/2048; under 'gpt3')")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="before the benchmark, run 5 plain device copies of 256 MiB (a kernel of known HBM traffic, "
                          "for scaling the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
@@ -156,6 +158,24 @@ def main():
                           "pct_smfmac_peak": round(100 * 2.0 * r2 * n2 * 2 * w2["geo"].ksp / (k2 * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2)})
             del w2
         out["extra"] = extra
+
+    if args.gpt3:
+        r2, c2, m2, v2 = 49152, 12288, 16, 128
+        w2 = prepare(r2, c2, 16, m2, v2)
+        gpt3 = []
+        for n2 in (16, 256, 2048):
+            gen = torch.Generator(device=dev)
+            gen.manual_seed(0)
+            w2["B"] = torch.randn((c2, n2), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+            w2["C"] = torch.empty((r2, n2), dtype=torch.float16, device=dev)
+            _, k2 = timed(w2, 50, 100)
+            by = algorithmic_bytes(r2, c2, n2, m2, v2, w2["geo"].ksp)
+            gpt3.append({"shape": "%dx%dx%d %d:2:%d" % (r2, c2, n2, v2, m2), "kernel": w2["plan"].kernel_name(n2, 0, 0),
+                         "us": round(k2 * 1e3, 2), "dense_equiv_tflops": round(2.0 * r2 * c2 * n2 / (k2 * 1e-3) / 1e12, 1),
+                         "hbm_gbs": round(by / (k2 * 1e-3) / 1e9, 1), "hbm_frac": round(by / (k2 * 1e-3) / 1e9 / HBM_PEAK_GBS, 3),
+                         "pct_smfmac_peak": round(100 * 2.0 * r2 * n2 * 2 * w2["geo"].ksp / (k2 * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2)})
+        del w2
+        out["gpt3"] = gpt3
 
     if not args.no_cpu_baseline:
         import oracle

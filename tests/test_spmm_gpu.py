@@ -45,6 +45,9 @@ CASES = [
     (256, 64, 8, 4, 64),          # dense-staged, plain 2:4
     (512, 325, 136, 5, 128),      # dense-staged, m = 5, V = 128, cols % m == 0 but Ksp padded
     (768, 450, 264, 7, 192),      # dense-staged, m = 7, V = 192, two-column tail
+    (256, 2048, 16, 16, 128),     # skinny-N kernel (k split over four waves), N = 16
+    (192, 200, 40, 8, 64),        # skinny-N kernel, three column tiles, ragged N and K
+    (128, 48, 64, 16, 64),        # skinny-N kernel at its widest, half-filled last k-step
 ]
 
 
@@ -69,6 +72,15 @@ def test_integer_operands_bit_exact(gpu, rows, cols, N, m, v, transposed):
         torch.cuda.synchronize()
         assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16)), (variant,)
     assert ran >= 4
+
+
+def test_skinny_kernel_is_selected_for_16_columns(gpu):
+    rows, cols, m, v = 256, 512, 16, 128
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=2, integer_values=True)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    assert "skinny" in plan.kernel_name(16, 0, 0) and "skinny" in plan.kernel_name(8, 1, 0)
+    assert "skinny" not in plan.kernel_name(256, 0, 0)
+    assert plan.kernel_name(72, 0, spatha.num_variants() - 1) is None      # the skinny kernel stops at 64 columns
 
 
 def test_dense_staged_kernel_is_selected_for_v64(gpu):

@@ -47,6 +47,7 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant) {
     } else if (plan->geo.v % bm != 0) {
         return false;
     }
+    if (variant == SPMM_VARIANT_SKINNY && N > 64) return false;
     if (spmm_variant_lds(variant, plan->S) > 160 * 1024) return false;      // row table kept in LDS
     if (variant >= SPMM_VARIANT_R128x128_S4) {
         // buffer-descriptor kernels address B, the packed operands and the row table with 32-bit offsets
@@ -64,6 +65,8 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
     if (variant != SPMM_VARIANT_AUTO) return variant_ok(plan, N, variant) ? variant : -1;
     const int v = plan->geo.v;
     int order[4] = {0, 0, 0, 0};
+    // few columns: streaming A is all that matters, one 64-row tile per workgroup with the k-steps split over its waves
+    if (N <= 16 && variant_ok(plan, N, SPMM_VARIANT_SKINNY)) return SPMM_VARIANT_SKINNY;
     if (v % 128 == 0) {
         const int64_t wide_tiles = (int64_t)(plan->geo.rows / 128) * ((N + 255) / 256);
         order[0] = wide_tiles >= 512 ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x128_S3;

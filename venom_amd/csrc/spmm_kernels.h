@@ -62,7 +62,8 @@ enum {
     SPMM_VARIANT_DS256x128_S3_C8 = 29,  // eight 64 x 64 consumer waves (two per SIMD)
     SPMM_VARIANT_DS256x128_S3_PP = 30,  // eight consumers in two phase groups (ping-pong)
     SPMM_VARIANT_DSF256x128_S3 = 31,    // dense-staged, LDS flag counters instead of workgroup barriers
-    SPMM_VARIANT_COUNT = 32
+    SPMM_VARIANT_SKINNY = 32,           // N <= 64: one 64-row tile per workgroup, k split over four waves, B straight from L2
+    SPMM_VARIANT_COUNT = 33
 };
 
 const char* spmm_variant_name(int variant);

@@ -2081,6 +2081,11 @@ __global__ __launch_bounds__((NC + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
     TileWalk walk;
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
+    if (p.skew > 0) {
+        // workgroups of one XCD start up to 7 * skew * 1024 clocks apart (write-out bursts spread over time)
+        const int units = ((blockIdx.x >> 3) & 7) * p.skew;
+        for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);
+    }
     if (wave < NC) {
         ds_consumer<Cfg, OUT_LAYOUT>(p, walk, smem, wave, lane);
     } else {
@@ -2207,8 +2212,22 @@ __device__ __forceinline__ void dsf_producer(const SpmmParams& p, const TileWalk
     set_voff();
     int st = 0, prev_st = 0;            // ring slot of the batch being issued / of the one before it
     uint32_t use = 0;                   // how often slot `st` has been filled before
+    bool pending = false;               // a batch is in flight whose stage has not been published yet
     for (int q = 0; q < Q; q++) {
-        if (use > 0) flag_wait<8>(empty_base + st * 4, (uint32_t)Cfg::NC * use);
+        if (use > 0) {
+            // if the slot is still being read, publish what is in flight first: a consumer must never wait for a
+            // stage that has landed only because this wave waits for another one to drain
+            uint32_t v;
+            asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(empty_base + st * 4) : "memory");
+            if ((int)((uint32_t)__builtin_amdgcn_readfirstlane((int)v) - (uint32_t)Cfg::NC * use) < 0) {
+                if (pending) {
+                    wait_vmcnt<0>();
+                    flag_signal(full_base + prev_st * 4, lane);
+                    pending = false;
+                }
+                flag_wait(empty_base + st * 4, (uint32_t)Cfg::NC * use);
+            }
+        }
         if (!(p.debug & 8)) {
             const uint32_t stage = smem_base + st * STAGE_BYTES;
 #pragma unroll
@@ -2235,11 +2254,12 @@ __device__ __forceinline__ void dsf_producer(const SpmmParams& p, const TileWalk
             g_soff = (uint32_t)(is_tm * S) * 512u + PR * 256u;
             set_voff();
         }
-        if (q > 0) {
+        if (pending) {
             // everything but the batch just issued has landed: publish the previous batch
             if (!(p.debug & 8)) wait_vmcnt<LOADS>();
             flag_signal(full_base + prev_st * 4, lane);
         }
+        pending = true;
         prev_st = st;
         if (++st == NS) {
             st = 0;
@@ -2247,16 +2267,18 @@ __device__ __forceinline__ void dsf_producer(const SpmmParams& p, const TileWalk
         }
     }
     wait_vmcnt<0>();
-    if (Q > 0) flag_signal(full_base + prev_st * 4, lane);
+    if (pending) flag_signal(full_base + prev_st * 4, lane);
 }
 
 // Consumer of the flag-synchronised kernel.  All operands are read one step ahead: while the 16
 // matrix instructions of step q issue, every fragment's registers are re-loaded from the stage
-// of step q+1 as soon as the instructions that read them are out, and the A operands follow
-// after the last one.  The scheduler is asked to alternate matrix instructions and LDS reads,
-// because a wave issues nothing else while it waits on a matrix instruction otherwise.
-// A stage is handed back to the producers as soon as it sits in registers, before it is
-// multiplied, and the next tile's first stage loads while this tile is written out.
+// of step q+1 as soon as the instructions that read them are out; the A operands go to a second
+// register set early in the step.  The counter of stage q+1 is requested (not waited for) behind
+// the first four instructions of step q and checked behind the next four: LDS reads return in
+// order, so by then the operand reads of step q, issued a whole step earlier, have long landed and
+// the check costs no LDS round trip.  A stage is handed back to the producers as soon as it sits
+// in registers, before it is multiplied, and the next tile's first stage loads while this tile
+// is written out.
 template <class Cfg, int NS, int NP, int OUT_LAYOUT>
 __device__ __forceinline__ void dsf_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, uint32_t smem_base,
                                              int wave, int lane) {
@@ -2319,6 +2341,8 @@ __device__ __forceinline__ void dsf_consumer(const SpmmParams& p, const TileWalk
     int st = 0;
     uint32_t use = 0;
     zero_acc();
+    half8_t a_nxt[4];
+    uint32_t j0, j1;
     // prologue: stage of step 0 into registers
     flag_wait(full_base, (uint32_t)NP);
     {
@@ -2338,31 +2362,51 @@ __device__ __forceinline__ void dsf_consumer(const SpmmParams& p, const TileWalk
             ++nuse;
         }
         const bool have_next = q + 1 < Q;
-        SPATHA_PROF_MARK(0)
-        // the poll's wait also covers this step's operand reads; the last step just waits for them
-        if (have_next) flag_wait(full_base + nst * 4, (uint32_t)NP * (nuse + 1));
-        flag_signal(empty_base + st * 4, lane);
-        SPATHA_PROF_MARK(1)
         // after the last step there is nothing to prefetch: re-read the current stage (never overwritten again)
         const char* stg = smem + (have_next ? nst : st) * STAGE_BYTES;
+        const uint32_t flag_addr = full_base + (have_next ? nst : st) * 4;
+        const uint32_t target = (uint32_t)NP * ((have_next ? nuse : use) + 1);
+        SPATHA_PROF_MARK(0)
         __builtin_amdgcn_sched_barrier(0);
-        set_base(*(const u32x2*)(stg + g_off));
         SPATHA_MMA4F(0)
-        read_frag(stg, 0);
-        SPATHA_MMA4F(1)
-        read_frag(stg, 1);
-        SPATHA_MMA4F(2)
-        read_frag(stg, 2);
-        SPATHA_MMA4F(3)
-        read_frag(stg, 3);
-        read_a(stg);
-#pragma unroll
-        for (int k = 0; k < 16; k++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x100, 7, 0);
         __builtin_amdgcn_sched_barrier(0);
+        // counter and gather-table entry of the next stage, requested behind the first instructions of this step
+        uint32_t flag;
+        asm volatile("ds_read_b32 %0, %1" : "=v"(flag) : "v"(flag_addr) : "memory");
+        u32x2 g = *(const u32x2*)(stg + g_off);
+        __builtin_amdgcn_sched_barrier(0);
+        SPATHA_MMA4F(1)
+        __builtin_amdgcn_sched_barrier(0);
+        // LDS reads return in order: with the counter, everything of this step's stage has landed as well
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(flag), "+v"(g)::"memory");
+        if ((int)((uint32_t)__builtin_amdgcn_readfirstlane((int)flag) - target) < 0) {
+            SPATHA_PROF_MARK(0)
+            flag_wait(flag_addr, target);
+            g = *(const u32x2*)(stg + g_off);
+            SPATHA_PROF_MARK(1)
+        }
+        flag_signal(empty_base + st * 4, lane);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) a_nxt[mb] = *(const half8_t*)(stg + a_off + mb * 1024);
+        j0 = *(const uint32_t*)(stg + i_off);
+        j1 = *(const uint32_t*)(stg + i_off + 256);
+        set_base(g);
+        read_frag(stg, 0);
+        read_frag(stg, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        SPATHA_MMA4F(2)
+        __builtin_amdgcn_sched_barrier(0);
+        read_frag(stg, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        SPATHA_MMA4F(3)
+        __builtin_amdgcn_sched_barrier(0);
+        read_frag(stg, 3);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) a_cur[mb] = a_nxt[mb];
+        i0 = j0;
+        i1 = j1;
         st = nst;
         use = nuse;
         if (++c_step == S) {

@@ -109,3 +109,30 @@ def test_layer_reuses_transposed_input_only_for_the_same_activation(gpu):
         x.mul_(2)                                       # in-place change: the version counter moves
         assert torch.equal(sp[0](x), direct(sp[0], x))
         del x                                           # the next trial may or may not get the same address
+
+
+@pytest.mark.gpu
+def test_gpt2_conv1d_swap_tracks_masked_dense(gpu):
+    """Every Conv1D of a small GPT-2 becomes an SpMM layer over the TRANSPOSED weight; a dense model whose
+    weights carry the same mask gives the same activations."""
+    from transformers.pytorch_utils import Conv1D
+    from venom_amd.bert import SrnmSpmm
+    from venom_amd.gpt2 import build_gpt2_large, conv1d_to_spmm
+
+    torch.set_grad_enabled(False)
+    dense = build_gpt2_large(layers=2, width=256, heads=4).to(gpu).half()
+    sparse = conv1d_to_spmm(build_gpt2_large(layers=2, width=256, heads=4).to(gpu).half(), 2, 8, 64)
+    swapped = [n for n, mod in sparse.named_modules() if isinstance(mod, SrnmSpmm)]
+    assert len(swapped) == 2 * 4 and not any(isinstance(mod, Conv1D) for mod in sparse.modules())
+    for mod in dense.modules():
+        if isinstance(mod, Conv1D):
+            w = mod.weight                                   # [in, out]; the mask runs along `in` for each output row
+            kept = torch.zeros(8, device=gpu, dtype=w.dtype)
+            kept[0] = kept[2] = 1
+            wt = w.t().reshape(w.shape[1], -1, 8) * kept     # [out, in/8, 8]
+            mod.weight.copy_(wt.reshape(w.shape[1], w.shape[0]).t())
+    ids = torch.randint(0, 100, (2, 64), device=gpu)
+    a = sparse(ids).last_hidden_state.float()
+    b = dense(ids).last_hidden_state.float()
+    assert torch.isfinite(a).all()
+    assert (a - b).abs().max().item() <= 5e-2

@@ -1567,42 +1567,46 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
     // as result lane: k = li/4, x = li%4
     const int q_lo = 4 * ((li >> 2) & 1) + (li & 3);
     const int out_col = col0 + 8 * (2 * kb + (li >> 3));
+    const bool live = out_col < N && stores_on;
+    // Eight phases (mb, half of the slab rows).  LDS operations of one wave execute in order, so the slab can be
+    // rewritten for the next phase as soon as this phase's reads are ISSUED; the global store of a phase is issued
+    // one phase late, behind the next phase's LDS traffic, so that no phase waits for a full LDS round trip.
+    u32x4 held = {0u, 0u, 0u, 0u};
+    int held_row = 0;
 #pragma unroll
-    for (int mb = 0; mb < 4; mb++) {
-        half4_t h4[4];
+    for (int ph = 0; ph < 8; ph++) {
+        const int mb = ph >> 1, sidx = ph & 1;
+        if (ROWS8 || sidx == 0) {
+            half4_t h4[4];
 #pragma unroll
-        for (int nb = 0; nb < 4; nb++)
+            for (int nb = 0; nb < 4; nb++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) h4[nb][r] = (_Float16)acc[mb][nb][r];
-        if (!ROWS8) {
-#pragma unroll
-            for (int nb = 0; nb < 4; nb++) *(half4_t*)(stg + (nb * 16 + j16) * PITCH + ib * 8) = h4[nb];
-            __builtin_amdgcn_wave_barrier();
-        }
-#pragma unroll
-        for (int sidx = 0; sidx < 2; sidx++) {
+                for (int r = 0; r < 4; r++) h4[nb][r] = (_Float16)acc[mb][nb][r];
             if (ROWS8) {
                 if ((ib >> 1) == sidx) {
 #pragma unroll
                     for (int nb = 0; nb < 4; nb++) *(half4_t*)(stg + (nb * 16 + j16) * PITCH + (ib & 1) * 8) = h4[nb];
                 }
-                __builtin_amdgcn_wave_barrier();
+            } else {
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++) *(half4_t*)(stg + (nb * 16 + j16) * PITCH + ib * 8) = h4[nb];
             }
-            const int roff = rd_off + (ROWS8 ? 0 : sidx * 16);
-            short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff));
-            short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff + 4 * PITCH));
-            u32x4 v;
-            v.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
-            v.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
-            v.z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
-            v.w = (uint32_t)(uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
-            const int q = 8 * sidx + q_lo;
-            const int row = 16 * (q >> 2) + 4 * mb + (q & 3);
-            if (out_col < N && stores_on) *(u32x4*)(C + (row0 + row) * N + out_col) = v;
-            if (ROWS8) __builtin_amdgcn_wave_barrier();
         }
         __builtin_amdgcn_wave_barrier();
+        const int roff = rd_off + (ROWS8 ? 0 : sidx * 16);
+        short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff));
+        short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff + 4 * PITCH));
+        __builtin_amdgcn_wave_barrier();
+        if (ph > 0 && live) *(u32x4*)(C + (row0 + held_row) * N + out_col) = held;
+        held.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+        held.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+        held.z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+        held.w = (uint32_t)(uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+        const int q = 8 * sidx + q_lo;
+        held_row = 16 * (q >> 2) + 4 * mb + (q & 3);
     }
+    if (live) *(u32x4*)(C + (row0 + held_row) * N + out_col) = held;
+    __builtin_amdgcn_wave_barrier();
 }
 
 // ---------------------------------------------------------------------------

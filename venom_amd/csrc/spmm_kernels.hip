@@ -1742,9 +1742,18 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
     int n_tm = c_tm, n_tn = c_tn;       // tile of the NEXT step's table entries
     SPATHA_PROF_DECL
     uint32_t c_stage = 0;
-    u32x2 g_cur[H], g_next[H];
+    u32x2 g_next[H];
+    // LDS offsets of this step's four fragments (per 64-row block): computed at the end of the previous step,
+    // behind its matrix instructions, so that the first reads can issue right after the barrier
+    uint32_t base[H][4];
+    auto set_base = [&](int h, u32x2 g) {
+        base[h][0] = ((g.x & 0xffffu) ^ col_xor) | col_or;
+        base[h][1] = ((g.x >> 16) ^ col_xor) | col_or;
+        base[h][2] = ((g.y & 0xffffu) ^ col_xor) | col_or;
+        base[h][3] = ((g.y >> 16) ^ col_xor) | col_or;
+    };
 #pragma unroll
-    for (int h = 0; h < H; h++) g_cur[h] = *gtab_ptr(c_tm, h, 0);
+    for (int h = 0; h < H; h++) set_base(h, *gtab_ptr(c_tm, h, 0));
     for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
 #pragma unroll
         for (int h = 0; h < H; h++)
@@ -1773,16 +1782,11 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
                     for (int mb = 0; mb < 4; mb++) a_cur[mb] = *(const half8_t*)(st + a_off + h * APACK_BLOCK + mb * 1024);
                     const uint32_t i0 = *(const uint32_t*)(st + i_off + h * APACK_BLOCK);
                     const uint32_t i1 = *(const uint32_t*)(st + i_off + h * APACK_BLOCK + 256);
-                    uint32_t base[4];
-                    base[0] = ((g_cur[h].x & 0xffffu) ^ col_xor) | col_or;
-                    base[1] = ((g_cur[h].x >> 16) ^ col_xor) | col_or;
-                    base[2] = ((g_cur[h].y & 0xffffu) ^ col_xor) | col_or;
-                    base[3] = ((g_cur[h].y >> 16) ^ col_xor) | col_or;
                     auto read_frag = [&](int nb) {
                         half16_t bf;
 #pragma unroll
                         for (int fb = 0; fb < 4; fb++) {
-                            short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, st + (base[fb] ^ (uint32_t)(nb << 5))));
+                            short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, st + (base[h][fb] ^ (uint32_t)(nb << 5))));
                             half4_t h4 = __builtin_bit_cast(half4_t, t4);
                             bf[fb * 4 + 0] = h4[0];
                             bf[fb * 4 + 1] = h4[1];
@@ -1814,7 +1818,7 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
             }
             c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
 #pragma unroll
-            for (int h = 0; h < H; h++) g_cur[h] = g_next[h];
+            for (int h = 0; h < H; h++) set_base(h, g_next[h]);
         }
         const int cm0 = c_tm * BM + rb0 * 64, cn0 = c_tn * BN;
         SPATHA_PROF_MARK(0)

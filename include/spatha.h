@@ -30,7 +30,8 @@ typedef enum spatha_status {
     SPATHA_ERR_UNSUPPORTED = 3,    /* valid format, but no kernel for it (e.g. V = 32)      */
     SPATHA_ERR_HIP = 4,            /* a HIP runtime call failed; see spatha_last_hip_error  */
     SPATHA_ERR_NO_DEVICE = 5,      /* no HIP device visible                                 */
-    SPATHA_ERR_TOO_LARGE = 6       /* beyond a fixed capacity of the entry point            */
+    SPATHA_ERR_TOO_LARGE = 6,      /* beyond a fixed capacity of the entry point            */
+    SPATHA_ERR_IO = 7              /* file missing, truncated, not a V:N:M container, or corrupt */
 } spatha_status;
 
 const char* spatha_status_string(int status);
@@ -111,6 +112,17 @@ int spatha_vnm_select_columns_f32(const float* dense_abs, int rows, int cols, in
 int spatha_vnm_pack_meta_blob(const uint32_t* metadata, int64_t n_metadata, const uint32_t* columns,
                               int64_t n_columns, uint32_t* blob, int64_t* columns_offset_words,
                               int64_t* blob_words);
+
+/* On-disk container of an encoded matrix (64-byte header: magic "VNMF", version, value width, shape,
+ * array lengths, FNV-1a checksum; then values, metadata, column-loc).  The reference parses
+ * --path_to_dset (src/util/argparse.h:123-126, src/benchmark_spmm.cpp) but never opens the file; these
+ * three functions give the flag a meaning: an encoded matrix can be cached instead of re-encoded.
+ * value_bits is 16 (fp16 values) or 32 (fp32).  spatha_vnm_file_info reports the sizes the caller has to
+ * allocate before spatha_vnm_file_read; a checksum or size mismatch is SPATHA_ERR_IO. */
+int spatha_vnm_file_write(const char* path, int rows, int cols, int n, int m, int v, int value_bits, const void* values,
+                          const uint32_t* metadata, const uint32_t* columns);
+int spatha_vnm_file_info(const char* path, spatha_vnm_geometry* geometry, int* value_bits);
+int spatha_vnm_file_read(const char* path, void* values, uint32_t* metadata, uint32_t* columns);
 
 /* ------------------------------------------------------------------------ *
  * SpMM on the GPU:  C[rows x N] = A_vnm[rows x cols] * B[cols x N],

@@ -147,3 +147,38 @@ def test_bad_shapes_are_reported_not_fatal():
     with pytest.raises(_lib.SpathaError) as e:
         F.geometry(64, 64, 2, 3, 32)         # m < 4
     assert e.value.status == 1
+
+
+def test_file_container_round_trip_and_rejects_damage(tmp_path):
+    rows, cols, n, m, v = 128, 100, 2, 8, 64
+    vals, meta, columns = F.synthetic_vnm(rows, cols, n, m, v, seed=3, value_std=1.0)
+    path = tmp_path / "a.vnm"
+    F.save(path, vals, meta, columns, rows, cols, n, m, v)
+    v2, m2, c2, g = F.load(path)
+    assert (g.rows, g.cols, g.n, g.m, g.v) == (rows, cols, n, m, v)
+    assert v2.dtype == np.float16 and np.array_equal(v2.view(np.uint16), vals.view(np.uint16))
+    assert np.array_equal(m2, meta.view(np.uint32)) and np.array_equal(c2, columns.reshape(-1))
+    # fp32 values keep their width
+    F.save(path, vals.astype(np.float32), meta, columns, rows, cols, n, m, v)
+    assert F.load(path)[0].dtype == np.float32
+    raw = bytearray(path.read_bytes())
+    for damage in ("flip", "truncate", "append", "magic", "shape"):
+        bad = bytearray(raw)
+        if damage == "flip":
+            bad[64 + 10] ^= 1                      # one payload bit: checksum
+        elif damage == "truncate":
+            bad = bad[:-4]
+        elif damage == "append":
+            bad += b"\0"
+        elif damage == "magic":
+            bad[0] = ord("X")
+        else:
+            bad[12] ^= 64                          # rows no longer match the stored array lengths
+        p2 = tmp_path / (damage + ".vnm")
+        p2.write_bytes(bytes(bad))
+        with pytest.raises(_lib.SpathaError) as e:
+            F.load(p2)
+        assert e.value.status == 7, damage
+    with pytest.raises(_lib.SpathaError) as e:
+        F.load(tmp_path / "missing.vnm")
+    assert e.value.status == 7

@@ -164,6 +164,20 @@ int main(int argc, const char** argv) {
     SPATHA_OK_OR_DIE(spatha_fill_rand_small_ints_f16(hB.data(), (int64_t)hB.size()));
     SPATHA_OK_OR_DIE(spatha_vnm_random_pattern(m, k, nn_row, mm_row, V, hMeta.data(), hCols.data()));
     SPATHA_OK_OR_DIE(spatha_fill_rand_small_ints_f16(hVal.data(), (int64_t)hVal.size()));
+    // --path_to_dset (parsed and ignored by the reference, src/util/argparse.h:123-126): the encoded A is read
+    // from that container when it exists (its shape must match the flags), and written there otherwise
+    if (!path_to_dset.empty()) {
+        spatha_vnm_geometry fg;
+        int bits = 0;
+        if (spatha_vnm_file_info(path_to_dset.c_str(), &fg, &bits) == SPATHA_OK) {
+            if (bits != 16 || fg.rows != m || fg.cols != k || fg.n != nn_row || fg.m != mm_row || fg.v != V)
+                die("--path_to_dset: the stored matrix does not match --m/--k/--nn_row/--mm_row/--bm (or is not fp16).");
+            SPATHA_OK_OR_DIE(spatha_vnm_file_read(path_to_dset.c_str(), hVal.data(), hMeta.data(), hCols.data()));
+        } else {
+            SPATHA_OK_OR_DIE(spatha_vnm_file_write(path_to_dset.c_str(), m, k, nn_row, mm_row, V, 16, hVal.data(), hMeta.data(),
+                                                   hCols.data()));
+        }
+    }
 
     // ---- host format conversion, timed: decode (the dense operand of the check) and re-encode
     const int threads = (int)std::thread::hardware_concurrency();

@@ -99,6 +99,7 @@ const char* spatha_status_string(int status) {
         case SPATHA_ERR_HIP: return "HIP runtime error";
         case SPATHA_ERR_NO_DEVICE: return "no HIP device";
         case SPATHA_ERR_TOO_LARGE: return "size beyond the entry point's capacity";
+        case SPATHA_ERR_IO: return "file missing, truncated, not a V:N:M container, or corrupt";
         default: return "unknown status";
     }
 }
@@ -143,6 +144,19 @@ int spatha_vnm_select_columns_f32(const float* dense_abs, int rows, int cols, in
                                   int32_t* columns, int threads) {
     return spatha::select_columns_f32(dense_abs, rows, cols, n, m, v, masks, columns, threads);
 }
+int spatha_vnm_file_write(const char* path, int rows, int cols, int n, int m, int v, int value_bits, const void* values,
+                          const uint32_t* metadata, const uint32_t* columns) {
+    return spatha::file_write(path, rows, cols, n, m, v, value_bits, values, metadata, columns);
+}
+
+int spatha_vnm_file_info(const char* path, spatha_vnm_geometry* geometry, int* value_bits) {
+    return spatha::file_info(path, geometry, value_bits);
+}
+
+int spatha_vnm_file_read(const char* path, void* values, uint32_t* metadata, uint32_t* columns) {
+    return spatha::file_read(path, values, metadata, columns);
+}
+
 int spatha_vnm_pack_meta_blob(const uint32_t* metadata, int64_t n_metadata, const uint32_t* columns,
                               int64_t n_columns, uint32_t* blob, int64_t* columns_offset_words,
                               int64_t* blob_words) {

@@ -19,6 +19,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <numeric>
@@ -472,6 +473,101 @@ int pack_meta_blob(const uint32_t* metadata, int64_t n_metadata, const uint32_t*
         std::memcpy(blob, metadata, sizeof(uint32_t) * (size_t)n_metadata);
         std::memcpy(blob + off, columns, sizeof(uint32_t) * (size_t)n_columns);
     }
+    return SPATHA_OK;
+}
+
+// ---------------------------------------------------------------------------
+// On-disk container for an encoded matrix.  The reference parses --path_to_dset
+// (src/util/argparse.h:123-126) but never reads a file; this format lets an
+// encoded model be cached instead of re-encoded at every load.
+//   bytes  0.. 3  "VNMF"            4.. 7  version (1)       8..11  value bits (16 or 32)
+//         12..31  rows, cols, n, m, v (int32 each)          32..55  n_values, n_metadata, n_columns (int64)
+//         56..63  FNV-1a 64 of the payload
+//   payload: values, metadata words, column-loc words, in this order, little endian.
+// ---------------------------------------------------------------------------
+namespace {
+struct FileHeader {
+    char magic[4];
+    uint32_t version, value_bits;
+    int32_t rows, cols, n, m, v;
+    int64_t n_values, n_metadata, n_columns;
+    uint64_t checksum;
+};
+static_assert(sizeof(FileHeader) == 64, "header layout");
+
+uint64_t fnv1a(uint64_t h, const void* data, size_t bytes) {
+    const unsigned char* p = (const unsigned char*)data;
+    for (size_t i = 0; i < bytes; i++) {
+        h ^= p[i];
+        h *= 1099511628211ull;
+    }
+    return h;
+}
+constexpr uint64_t FNV_SEED = 14695981039346656037ull;
+
+int read_header(std::FILE* f, FileHeader& h) {
+    if (std::fread(&h, sizeof(h), 1, f) != 1) return SPATHA_ERR_IO;
+    if (std::memcmp(h.magic, "VNMF", 4) != 0 || h.version != 1) return SPATHA_ERR_IO;
+    if (h.value_bits != 16 && h.value_bits != 32) return SPATHA_ERR_IO;
+    spatha_vnm_geometry g;
+    int st = geometry_init(h.rows, h.cols, h.n, h.m, h.v, &g);
+    if (st != SPATHA_OK) return SPATHA_ERR_IO;
+    if (g.n_values != h.n_values || g.n_metadata != h.n_metadata || g.n_columns != h.n_columns) return SPATHA_ERR_IO;
+    return SPATHA_OK;
+}
+}  // namespace
+
+int file_write(const char* path, int rows, int cols, int n, int m, int v, int value_bits, const void* values,
+               const uint32_t* metadata, const uint32_t* columns) {
+    if (!path || !values || !metadata || !columns || (value_bits != 16 && value_bits != 32)) return SPATHA_ERR_BAD_ARGUMENT;
+    spatha_vnm_geometry g;
+    int st = geometry_init(rows, cols, n, m, v, &g);
+    if (st != SPATHA_OK) return st;
+    FileHeader h;
+    std::memcpy(h.magic, "VNMF", 4);
+    h.version = 1;
+    h.value_bits = (uint32_t)value_bits;
+    h.rows = rows; h.cols = cols; h.n = n; h.m = m; h.v = v;
+    h.n_values = g.n_values; h.n_metadata = g.n_metadata; h.n_columns = g.n_columns;
+    const size_t vb = (size_t)g.n_values * (value_bits / 8), mb = (size_t)g.n_metadata * 4, cb = (size_t)g.n_columns * 4;
+    h.checksum = fnv1a(fnv1a(fnv1a(FNV_SEED, values, vb), metadata, mb), columns, cb);
+    std::FILE* f = std::fopen(path, "wb");
+    if (!f) return SPATHA_ERR_IO;
+    bool ok = std::fwrite(&h, sizeof(h), 1, f) == 1 && std::fwrite(values, 1, vb, f) == vb &&
+              std::fwrite(metadata, 1, mb, f) == mb && std::fwrite(columns, 1, cb, f) == cb;
+    ok = (std::fclose(f) == 0) && ok;
+    return ok ? SPATHA_OK : SPATHA_ERR_IO;
+}
+
+int file_info(const char* path, spatha_vnm_geometry* geo, int* value_bits) {
+    if (!path || !geo) return SPATHA_ERR_BAD_ARGUMENT;
+    std::FILE* f = std::fopen(path, "rb");
+    if (!f) return SPATHA_ERR_IO;
+    FileHeader h;
+    int st = read_header(f, h);
+    std::fclose(f);
+    if (st != SPATHA_OK) return st;
+    if (value_bits) *value_bits = (int)h.value_bits;
+    return geometry_init(h.rows, h.cols, h.n, h.m, h.v, geo);
+}
+
+int file_read(const char* path, void* values, uint32_t* metadata, uint32_t* columns) {
+    if (!path || !values || !metadata || !columns) return SPATHA_ERR_BAD_ARGUMENT;
+    std::FILE* f = std::fopen(path, "rb");
+    if (!f) return SPATHA_ERR_IO;
+    FileHeader h;
+    int st = read_header(f, h);
+    if (st != SPATHA_OK) {
+        std::fclose(f);
+        return st;
+    }
+    const size_t vb = (size_t)h.n_values * (h.value_bits / 8), mb = (size_t)h.n_metadata * 4, cb = (size_t)h.n_columns * 4;
+    bool ok = std::fread(values, 1, vb, f) == vb && std::fread(metadata, 1, mb, f) == mb && std::fread(columns, 1, cb, f) == cb;
+    char extra;
+    ok = ok && std::fread(&extra, 1, 1, f) == 0;          // nothing may follow the payload
+    std::fclose(f);
+    if (!ok) return SPATHA_ERR_IO;
+    if (fnv1a(fnv1a(fnv1a(FNV_SEED, values, vb), metadata, mb), columns, cb) != h.checksum) return SPATHA_ERR_IO;
     return SPATHA_OK;
 }
 

@@ -23,6 +23,11 @@ int decode_f16(const uint16_t* values, const uint32_t* metadata, const uint32_t*
 int select_columns_f32(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
                        int32_t* columns, int threads);
 
+int file_write(const char* path, int rows, int cols, int n, int m, int v, int value_bits, const void* values,
+               const uint32_t* metadata, const uint32_t* columns);
+int file_info(const char* path, spatha_vnm_geometry* geo, int* value_bits);
+int file_read(const char* path, void* values, uint32_t* metadata, uint32_t* columns);
+
 int pack_meta_blob(const uint32_t* metadata, int64_t n_metadata, const uint32_t* columns, int64_t n_columns,
                    uint32_t* blob, int64_t* columns_offset_words, int64_t* blob_words);
 

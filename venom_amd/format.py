@@ -104,6 +104,34 @@ def pack_meta_blob(metadata, columns):
     return blob, off.value
 
 
+def save(path, values, metadata, columns, rows, cols, n, m, v):
+    """Writes an encoded matrix to the library's on-disk container (values fp16 or fp32)."""
+    values = np.ascontiguousarray(values)
+    metadata = np.ascontiguousarray(metadata).view(np.uint32)
+    columns = np.ascontiguousarray(columns, dtype=np.uint32).reshape(-1)
+    g = geometry(rows, cols, n, m, v)
+    if values.size != g.n_values or metadata.size != g.n_metadata or columns.size != g.n_columns:
+        raise ValueError("array sizes do not match the format geometry")
+    bits = {np.dtype(np.float16): 16, np.dtype(np.float32): 32}.get(values.dtype)
+    if bits is None:
+        raise TypeError("values must be float16 or float32")
+    _lib.check(_lib.lib().spatha_vnm_file_write(str(path).encode(), rows, cols, n, m, v, bits, _p(values), _p(metadata),
+                                                _p(columns)), "spatha_vnm_file_write")
+
+
+def load(path):
+    """Reads a container written by `save`: (values, metadata, columns, geometry)."""
+    L = _lib.lib()
+    g = _lib.Geometry()
+    bits = ctypes.c_int(0)
+    _lib.check(L.spatha_vnm_file_info(str(path).encode(), ctypes.byref(g), ctypes.byref(bits)), "spatha_vnm_file_info")
+    values = np.empty(g.n_values, np.float16 if bits.value == 16 else np.float32)
+    metadata = np.empty(g.n_metadata, np.uint32)
+    columns = np.empty(g.n_columns, np.uint32)
+    _lib.check(L.spatha_vnm_file_read(str(path).encode(), _p(values), _p(metadata), _p(columns)), "spatha_vnm_file_read")
+    return values, metadata, columns, g
+
+
 def synthetic_vnm(rows, cols, n, m, v, seed=0, value_std=1.0, integer_values=False):
     """Seeded synthetic V:N:M matrix in compressed form (values fp16, metadata, columns):
     per V x m block 4 of the m columns drawn uniformly, per row 2 of those 4 kept uniformly;

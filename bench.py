@@ -48,6 +48,8 @@ def main():
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extra", action="store_true", help="also time the other BASELINE shapes (reported under 'extra')")
+    ap.add_argument("--ablation", action="store_true",
+                    help="also time the same matrix with identity column-loc (the reference's IDEAL_KERNEL ablation)")
     ap.add_argument("--gpt3", action="store_true",
                     help="also time the GPT-3 FFN shapes (A 49152x12288 128:2:16, N in 16/256/2048; under 'gpt3')")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -158,6 +160,17 @@ def main():
                           "pct_smfmac_peak": round(100 * 2.0 * r2 * n2 * 2 * w2["geo"].ksp / (k2 * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2)})
             del w2
         out["extra"] = extra
+
+    if args.ablation:
+        # the reference's IDEAL_KERNEL switch (CMakeLists.txt:25-33, blockwise_kernel.h): column-loc ignored, i.e. the
+        # four gathered rows of every group are its first four -> the cost of the indirection is the difference
+        ident = np.tile(np.arange(4, dtype=np.uint32), w["columns"].size // 4)
+        w_id = dict(w)
+        w_id["plan"] = spatha.SpmmPlan(torch.from_numpy(w["vals"]).to(dev), torch.from_numpy(w["meta"].view(np.int32)).to(dev),
+                                       torch.from_numpy(ident.view(np.int32)).to(dev), rows, cols, 2, m, v)
+        _, k_id = timed(w_id, args.steps, args.warmup, args.variant)
+        _, k_nm = timed(w, args.steps, 50, args.variant)
+        out["ablation"] = {"column_loc_us": round(k_nm * 1e3, 2), "ideal_identity_column_loc_us": round(k_id * 1e3, 2)}
 
     if args.gpt3:
         r2, c2, m2, v2 = 49152, 12288, 16, 128

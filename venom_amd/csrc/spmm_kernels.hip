@@ -1338,6 +1338,45 @@ __device__ __forceinline__ void ws_consumer_deferred(const SpmmParams& p, const 
         for (int part = 0; part < 4; part++) flush_part(part);
 }
 
+// Transposed write-out (C^T[N][rows], + bias) of one wave's 64 x 64 block through an LDS slab of 8 columns x 64 rows.
+// Straight from the accumulators a lane could only store 16-byte pieces 32 bytes apart; through the slab every
+// store instruction writes 8 output rows (columns of C) x 128 contiguous bytes.
+constexpr int TT_PITCH = 144;                      // 64 rows x 2 B + 16 B pad (keeps 16-byte alignment)
+constexpr int TT_SLAB_BYTES = 8 * TT_PITCH;        // per wave
+__device__ __forceinline__ void store_block_transposed_slab(const float4_t (&acc)[4][4], char* stg, uint16_t* C,
+                                                            const uint16_t* bias, int64_t row0, int col0, int rows_total, int N,
+                                                            int lane, bool stores_on) {
+    const int j16 = lane & 15, ib = lane >> 4;     // as accumulator lane: column j16 of a 16-column block, rows 16*ib + 4*mb + r
+    const int rn = lane >> 3, rc = lane & 7;       // as reader: slab column rn, 16-byte chunk rc (rows 8*rc .. 8*rc + 7)
+    half4_t b4[4];
+    if (bias) {
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) b4[mb] = *(const half4_t*)(bias + row0 + 16 * ib + 4 * mb);
+    }
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        half4_t h4[4];
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) h4[mb][r] = (_Float16)acc[mb][nb][r];
+            if (bias) h4[mb] = h4[mb] + b4[mb];
+        }
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++) {
+            if ((j16 >> 3) == hf) {
+#pragma unroll
+                for (int mb = 0; mb < 4; mb++) *(half4_t*)(stg + (j16 & 7) * TT_PITCH + (16 * ib + 4 * mb) * 2) = h4[mb];
+            }
+            __builtin_amdgcn_wave_barrier();
+            const u32x4 v = *(const u32x4*)(stg + rn * TT_PITCH + rc * 16);
+            __builtin_amdgcn_wave_barrier();
+            const int col = col0 + nb * 16 + hf * 8 + rn;
+            if (col < N && stores_on) *(u32x4*)(C + (int64_t)col * rows_total + row0 + rc * 8) = v;
+        }
+    }
+}
+
 // ---- tall consumer: one wave owns a 128 x 64 tile (two stacked 64-row halves sharing the B
 // fragments): 32 matrix instructions per k-step for the same 16 transposing reads, so the
 // LDS and issue cost per matrix instruction drops by a third and one consumer per SIMD is enough.
@@ -1415,33 +1454,9 @@ __device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const Tile
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
-                const int64_t row0 = (int64_t)cm0 + h * 64 + ib * 16;
-                half8_t bias_lo, bias_hi;
-                if (p.bias) {
-                    bias_lo = *(const half8_t*)(p.bias + row0);
-                    bias_hi = *(const half8_t*)(p.bias + row0 + 8);
-                }
-#pragma unroll
-                for (int nb = 0; nb < 4; nb++) {
-                    const int col = cn0 + wn * 64 + nb * 16 + j16;
-                    half8_t lo, hi;
-#pragma unroll
-                    for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            lo[mb * 4 + r] = (_Float16)acc[h][mb][nb][r];
-                            hi[mb * 4 + r] = (_Float16)acc[h][mb + 2][nb][r];
-                        }
-                    if (p.bias) {
-                        lo = lo + bias_lo;
-                        hi = hi + bias_hi;
-                    }
-                    if (col < N && !(p.debug & 2)) {
-                        uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
-                        *(half8_t*)dst = lo;
-                        *(half8_t*)(dst + 8) = hi;
-                    }
-                }
+                if (!(p.debug & 4))
+                    store_block_transposed_slab(acc[h], smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH), p.C, p.bias,
+                                                (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !(p.debug & 2));
             } else if (!(p.debug & 4)) {
                 char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
 #pragma unroll
@@ -1607,45 +1622,6 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
     }
     if (live) *(u32x4*)(C + (row0 + held_row) * N + out_col) = held;
     __builtin_amdgcn_wave_barrier();
-}
-
-// Transposed write-out (C^T[N][rows], + bias) of one wave's 64 x 64 block through an LDS slab of 8 columns x 64 rows.
-// Straight from the accumulators a lane could only store 16-byte pieces 32 bytes apart; through the slab every
-// store instruction writes 8 output rows (columns of C) x 128 contiguous bytes.
-constexpr int TT_PITCH = 144;                      // 64 rows x 2 B + 16 B pad (keeps 16-byte alignment)
-constexpr int TT_SLAB_BYTES = 8 * TT_PITCH;        // per wave
-__device__ __forceinline__ void store_block_transposed_slab(const float4_t (&acc)[4][4], char* stg, uint16_t* C,
-                                                            const uint16_t* bias, int64_t row0, int col0, int rows_total, int N,
-                                                            int lane, bool stores_on) {
-    const int j16 = lane & 15, ib = lane >> 4;     // as accumulator lane: column j16 of a 16-column block, rows 16*ib + 4*mb + r
-    const int rn = lane >> 3, rc = lane & 7;       // as reader: slab column rn, 16-byte chunk rc (rows 8*rc .. 8*rc + 7)
-    half4_t b4[4];
-    if (bias) {
-#pragma unroll
-        for (int mb = 0; mb < 4; mb++) b4[mb] = *(const half4_t*)(bias + row0 + 16 * ib + 4 * mb);
-    }
-#pragma unroll
-    for (int nb = 0; nb < 4; nb++) {
-        half4_t h4[4];
-#pragma unroll
-        for (int mb = 0; mb < 4; mb++) {
-#pragma unroll
-            for (int r = 0; r < 4; r++) h4[mb][r] = (_Float16)acc[mb][nb][r];
-            if (bias) h4[mb] = h4[mb] + b4[mb];
-        }
-#pragma unroll
-        for (int hf = 0; hf < 2; hf++) {
-            if ((j16 >> 3) == hf) {
-#pragma unroll
-                for (int mb = 0; mb < 4; mb++) *(half4_t*)(stg + (j16 & 7) * TT_PITCH + (16 * ib + 4 * mb) * 2) = h4[mb];
-            }
-            __builtin_amdgcn_wave_barrier();
-            const u32x4 v = *(const u32x4*)(stg + rn * TT_PITCH + rc * 16);
-            __builtin_amdgcn_wave_barrier();
-            const int col = col0 + nb * 16 + hf * 8 + rn;
-            if (col < N && stores_on) *(u32x4*)(C + (int64_t)col * rows_total + row0 + rc * 8) = v;
-        }
-    }
 }
 
 // ---------------------------------------------------------------------------

@@ -76,8 +76,11 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
     } else if (v % 64 == 0) {
         // m <= 8: staging the dense B rows once for four 64-row blocks halves the L2 -> LDS traffic
         order[0] = SPMM_VARIANT_DS256x128_S3_C8;
-        order[1] = SPMM_VARIANT_P64x256_S2;
-        order[2] = SPMM_VARIANT_W64x256_S3;
+        // m > 8: gathered 64 x 256 tiles; with many k-steps per tile the persistent pipeline (which keeps loading
+        // across tile boundaries) is 1.6x faster than the per-tile one, with few it is a few percent slower
+        const bool long_k = plan->S >= 24;
+        order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : SPMM_VARIANT_P64x256_S2;
+        order[2] = long_k ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_R64x256_S3;
         order[3] = SPMM_VARIANT_64x256;
     } else {
         return -1;

@@ -71,6 +71,13 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
         const int64_t wide_tiles = (int64_t)(plan->geo.rows / 128) * ((N + 255) / 256);
         order[0] = wide_tiles >= 512 ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x128_S3;
         order[1] = SPMM_VARIANT_W128x128_S3;
+        // measured on the BERT-large shapes (N = 16384): plain 2:4 runs 6-8 % faster with dense-staged 256 x 128
+        // tiles, m >= 16 3-5 % faster with two 128 x 128 workgroups per CU (two stages each)
+        if (wide_tiles >= 512 && plan->geo.m <= 4) order[0] = SPMM_VARIANT_DS256x128_S3_C8;
+        if (wide_tiles >= 512 && plan->geo.m >= 16) {
+            order[1] = order[0];
+            order[0] = SPMM_VARIANT_W128x128_S2;
+        }
         order[2] = SPMM_VARIANT_P128x128_S3;
         order[3] = SPMM_VARIANT_128x128;
     } else if (v % 64 == 0) {
@@ -79,7 +86,7 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
         // m > 8: gathered 64 x 256 tiles; with many k-steps per tile the persistent pipeline (which keeps loading
         // across tile boundaries) is 1.6x faster than the per-tile one, with few it is a few percent slower
         const bool long_k = plan->S >= 24;
-        order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : SPMM_VARIANT_P64x256_S2;
+        order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : (plan->geo.m >= 32 ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_P64x256_S2);
         order[2] = long_k ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_R64x256_S3;
         order[3] = SPMM_VARIANT_64x256;
     } else {

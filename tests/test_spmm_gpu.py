@@ -161,6 +161,29 @@ def test_full_size_checksums(gpu, rows, cols, N, m, v):
     assert torch.equal(Ct.t(), C)
 
 
+@pytest.mark.parametrize("N", [16, 256])
+def test_gpt3_ffn_shape_blocks_within_tolerance(gpu, N):
+    """BASELINE config 4: A 49152 x 12288 in 128:2:16, values ~N(0, 0.02), B ~N(0, 1); N = 16 runs on the skinny
+    kernel.  Three V-row blocks of C are compared with the float64 product of their decoded rows."""
+    rows, cols, m, v = 49152, 12288, 16, 128
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=0, value_std=0.02)
+    g = F.geometry(rows, cols, 2, m, v)
+    gen = torch.Generator(device=gpu)
+    gen.manual_seed(0)
+    B = torch.randn((cols, N), generator=gen, device=gpu).half()
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    assert ("skinny" in plan.kernel_name(N, 0, 0)) == (N <= 16)
+    C = plan.run(B)
+    Bh = B.cpu().numpy().astype(np.float64)
+    nm, nc = (v // 2) * (g.ksp // 8), (g.ksp // 2) * 4
+    for b in (0, 200, rows // v - 1):
+        dense = F.decode(vals[b * v * g.ksp:(b + 1) * v * g.ksp], meta[b * nm:(b + 1) * nm], columns.reshape(-1)[b * nc:(b + 1) * nc],
+                         v, cols, 2, m, v).astype(np.float64)
+        want = dense @ Bh
+        got = C[b * v:(b + 1) * v].cpu().numpy().astype(np.float64)
+        assert (np.abs(got - want) / np.maximum(np.abs(want), 1.0)).max() <= REL_TOL
+
+
 def test_linearity_in_B(gpu):
     rows, cols, N, m, v = 512, 2048, 1024, 16, 128
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=3, integer_values=True)

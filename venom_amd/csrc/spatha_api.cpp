@@ -74,7 +74,7 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
         // measured on the BERT-large shapes (N = 16384): plain 2:4 runs 6-8 % faster with dense-staged 256 x 128
         // tiles, m >= 16 3-5 % faster with two 128 x 128 workgroups per CU (two stages each)
         if (wide_tiles >= 512 && plan->geo.m <= 4) order[0] = SPMM_VARIANT_DS256x128_S3_C8;
-        if (wide_tiles >= 512 && plan->geo.m >= 16) {
+        if (wide_tiles >= 512 && plan->geo.m >= 16 && plan->S <= 16) {      // (long k-loops: the tall tile stays ahead)
             order[1] = order[0];
             order[0] = SPMM_VARIANT_W128x128_S2;
         }

@@ -74,13 +74,64 @@ def test_integer_operands_bit_exact(gpu, rows, cols, N, m, v, transposed):
     assert ran >= 4
 
 
+HALF_TILE_CASES = [
+    # rows, cols, N, m, v : V a multiple of 32 only, a 64-row tile spans two V blocks
+    (64, 64, 64, 8, 32),
+    (128, 256, 264, 8, 32),       # ragged N
+    (192, 200, 136, 8, 96),       # V = 96, K tail
+    (128, 48, 72, 4, 32),         # plain 2:4, half-filled last k-step
+    (256, 1024, 520, 16, 32),     # 16 k-steps, three 256-wide tiles
+    (320, 330, 40, 20, 160),      # V = 160, m not a power of two
+    (128, 1280, 16, 32, 32),      # few columns: the skinny kernel does not take this operand order
+]
+
+
+@pytest.mark.parametrize("rows,cols,N,m,v", HALF_TILE_CASES)
+@pytest.mark.parametrize("transposed", [False, True])
+def test_half_tile_kernels_bit_exact(gpu, rows, cols, N, m, v, transposed):
+    print("case", rows, cols, N, m, v, transposed, flush=True)
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=rows + N, integer_values=True)
+    rng = np.random.default_rng(N)
+    B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+    bias = rng.integers(-3, 4, size=rows).astype(np.float16) if transposed else None
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias, transposed_out=transposed)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    assert "halftile" in plan.kernel_name(N, 1 if transposed else 0, 0)
+    ran = 0
+    for variant in range(spatha.num_variants()):
+        name = plan.kernel_name(N, 1 if transposed else 0, variant)
+        if name is None:
+            continue
+        assert "halftile" in name            # the other kernels read a different operand order
+        ran += 1
+        print("   variant", variant, name, flush=True)
+        got = plan.run(_dev(B, gpu), bias=None if bias is None else _dev(bias, gpu), transposed_out=transposed,
+                       variant=variant)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16)), (variant,)
+    assert ran == 4                          # automatic choice + three tile shapes
+
+
+def test_half_tile_gaussian_within_tolerance(gpu):
+    """The reference's V = 32 ablation shape (1024 x 4096 x 4096, 32:2:8), Gaussian operands."""
+    rows, cols, N, m, v = 1024, 4096, 4096, 8, 32
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=0, value_std=1.0)
+    rng = np.random.default_rng(0)
+    B = rng.uniform(-1, 1, size=(cols, N)).astype(np.float16)
+    exact = oracle.decode(vals, meta, columns, rows, cols, 2, m, v).astype(np.float64) @ B.astype(np.float64)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    for variant in (0, spatha.num_variants() - 2):
+        got = plan.run(_dev(B, gpu), variant=variant).cpu().numpy().astype(np.float64)
+        assert (np.abs(got - exact) / np.maximum(np.abs(exact), 1.0)).max() <= REL_TOL
+
+
 def test_skinny_kernel_is_selected_for_16_columns(gpu):
     rows, cols, m, v = 256, 512, 16, 128
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=2, integer_values=True)
     plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
     assert "skinny" in plan.kernel_name(16, 0, 0) and "skinny" in plan.kernel_name(8, 1, 0)
     assert "skinny" not in plan.kernel_name(256, 0, 0)
-    assert plan.kernel_name(72, 0, spatha.num_variants() - 1) is None      # the skinny kernel stops at 64 columns
+    assert plan.kernel_name(72, 0, 32) is None      # the skinny kernel (variant 32) stops at 64 columns
 
 
 def test_dense_staged_kernel_is_selected_for_v64(gpu):
@@ -95,13 +146,16 @@ def test_dense_staged_kernel_is_selected_for_v64(gpu):
     assert "densestage" not in _plan(vals, meta, columns, 128, cols, m, v, gpu).kernel_name(N, 0, 0)
 
 
-@pytest.mark.parametrize("path", [p for p in golden_cases() if "_v64" in p or "_v128" in p],
+@pytest.mark.parametrize("path", [p for p in golden_cases() if "vnm_z_" not in p],
                          ids=lambda p: p.split("vnm_")[-1][:-4])
 def test_reference_encoded_matrices(gpu, path):
-    """Arrays written by the reference's own encoder go straight into the kernel."""
+    """Arrays written by the reference's own encoder go straight into the kernel (all but the all-zero-block case,
+    whose unused value slots the reference leaves uninitialised)."""
     z = np.load(path)
     n, m, v = int(z["n"]), int(z["m"]), int(z["v"])
     rows, cols = z["dense"].shape
+    if rows % 64:
+        pytest.skip("the kernels own 64-row tiles")
     vals = z["values"].astype(np.float16)
     rng = np.random.default_rng(1)
     N = 72

@@ -16,6 +16,7 @@
 struct spatha_spmm_plan {
     spatha_vnm_geometry geo;
     int S;                 // k-steps of 64 compressed B rows
+    int half_tiles;        // V % 64 != 0: operands packed in the order of the half-tile kernels
     int device;
     uint16_t* apack;
     uint32_t* rowtab;
@@ -39,6 +40,10 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant) {
     if (variant <= 0 || variant >= SPMM_VARIANT_COUNT) return false;
     const int bm = spmm_variant_bm(variant);
     if (bm == 0) return false;
+    const bool half_variant = variant == SPMM_VARIANT_H64x256_S2 || variant == SPMM_VARIANT_H64x128_S3 ||
+                              variant == SPMM_VARIANT_H64x128_S2;
+    if (half_variant != (plan->half_tiles != 0)) return false;       // the packed operand order differs
+    if (half_variant) return plan->geo.cols <= 65535 && spmm_variant_lds(variant, plan->S) <= 160 * 1024;
     if (variant == SPMM_VARIANT_DS256x128_S3 || variant == SPMM_VARIANT_DS256x128_S2 ||
         variant == SPMM_VARIANT_DS256x128_S3_C8 || variant == SPMM_VARIANT_DS256x128_S3_PP ||
         variant == SPMM_VARIANT_DSF256x128_S3) {
@@ -67,6 +72,16 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
     int order[4] = {0, 0, 0, 0};
     // few columns: streaming A is all that matters, one 64-row tile per workgroup with the k-steps split over its waves
     if (N <= 16 && variant_ok(plan, N, SPMM_VARIANT_SKINNY)) return SPMM_VARIANT_SKINNY;
+    if (plan->half_tiles) {
+        // measured (1024 x 4096 x 4096 and 4096 x 1024 x 16384, m = 8..32): the 256-wide tile is never behind the
+        // 128-wide one with two stages by more than 7 %, and up to 2x ahead; three stages of 128 leave two waves per CU
+        order[0] = N > 128 ? SPMM_VARIANT_H64x256_S2 : SPMM_VARIANT_H64x128_S2;
+        order[1] = SPMM_VARIANT_H64x128_S2;
+        order[2] = SPMM_VARIANT_H64x128_S3;
+        for (int i = 0; i < 3; i++)
+            if (variant_ok(plan, N, order[i])) return order[i];
+        return -1;
+    }
     if (v % 128 == 0) {
         const int64_t wide_tiles = (int64_t)(plan->geo.rows / 128) * ((N + 255) / 256);
         order[0] = wide_tiles >= 512 ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x128_S3;
@@ -182,7 +197,7 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     int st = spatha::geometry_init(rows, cols, n, m, v, &geo);
     if (st) return st;
     if (!values_dev || !metadata_dev || !columns_dev) return SPATHA_ERR_BAD_ARGUMENT;
-    if (v % 64 != 0) return SPATHA_ERR_UNSUPPORTED;   // kernels own 64-row wave tiles inside one V block
+    if (rows % 64 != 0) return SPATHA_ERR_UNSUPPORTED;   // kernels own 64-row wave tiles
     int ndev = 0;
     hipError_t e = hipGetDeviceCount(&ndev);
     if (e != hipSuccess || ndev == 0) { g_last_hip_error = (int)e; return SPATHA_ERR_NO_DEVICE; }
@@ -190,6 +205,7 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     if (!plan) return SPATHA_ERR_BAD_ARGUMENT;
     plan->geo = geo;
     plan->S = (geo.ksp + 31) / 32;
+    plan->half_tiles = (v % 64 != 0);      // V = 32, 96, ...: a wave tile spans two V blocks
     plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr; plan->gtab_tiles = nullptr; plan->gtab_tiles_bytes = 0;
     e = hipGetDevice(&plan->device);
     if (e != hipSuccess) { delete plan; return hip_fail(e); }
@@ -203,8 +219,8 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
         spatha_spmm_plan_destroy(plan);
         return hip_fail(e);
     }
-    e = spatha::launch_pack(values_dev, metadata_dev, columns_dev, rows, cols, m, v, geo.ksp, plan->S, plan->apack,
-                            plan->rowtab, (hipStream_t)stream);
+    e = spatha::launch_pack(values_dev, metadata_dev, columns_dev, rows, cols, m, v, geo.ksp, plan->S, plan->half_tiles,
+                            plan->apack, plan->rowtab, (hipStream_t)stream);
     if (e != hipSuccess) { spatha_spmm_plan_destroy(plan); return hip_fail(e); }
     if (v % 64 == 0 && m <= 8 && rows % 256 == 0) {
         const size_t g_bytes = (size_t)(rows / 64) * plan->S * 64 * 2;

@@ -63,7 +63,10 @@ enum {
     SPMM_VARIANT_DS256x128_S3_PP = 30,  // eight consumers in two phase groups (ping-pong)
     SPMM_VARIANT_DSF256x128_S3 = 31,    // dense-staged, LDS flag counters instead of workgroup barriers
     SPMM_VARIANT_SKINNY = 32,           // N <= 64: one 64-row tile per workgroup, k split over four waves, B straight from L2
-    SPMM_VARIANT_COUNT = 33
+    SPMM_VARIANT_H64x256_S2 = 33,       // V % 64 != 0: a 64-row tile spans two V blocks, two gathered B sets per stage
+    SPMM_VARIANT_H64x128_S3 = 34,
+    SPMM_VARIANT_H64x128_S2 = 35,
+    SPMM_VARIANT_COUNT = 36
 };
 
 const char* spmm_variant_name(int variant);
@@ -74,7 +77,7 @@ int spmm_variant_lds(int variant, int S);
 hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
-                       int m, int v, int ksp, int S, uint16_t* apack, uint32_t* rowtab, hipStream_t stream);
+                       int m, int v, int ksp, int S, int half_tiles, uint16_t* apack, uint32_t* rowtab, hipStream_t stream);
 
 hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, uint16_t* gtab,
                             hipStream_t stream);

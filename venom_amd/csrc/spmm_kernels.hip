@@ -55,7 +55,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 // One thread per (wave tile, step, mb, lane) for apack/ipack; rowtab separately.
 // ---------------------------------------------------------------------------
 __global__ void pack_a_kernel(const uint16_t* __restrict__ values, const uint32_t* __restrict__ metadata, int rows,
-                              int ksp, int S, uint16_t* __restrict__ apack) {
+                              int ksp, int S, int half_tiles, uint16_t* __restrict__ apack) {
     const int64_t total = (int64_t)(rows / 64) * S * 4 * 64;
     const int ngroups = ksp / 2;
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
@@ -66,7 +66,8 @@ __global__ void pack_a_kernel(const uint16_t* __restrict__ values, const uint32_
         int64_t wt = ws / S;
         int i = lane & 15, kq = lane >> 4;
         int ib = i >> 2, rr = i & 3;
-        int64_t r = wt * 64 + 16 * ib + 4 * mb + rr;      // matrix row
+        // matrix row; half_tiles: the order of the V = 32 kernels (instructions 0, 1 = rows 0..31 of the tile)
+        int64_t r = wt * 64 + (half_tiles ? 32 * (mb >> 1) + 8 * ib + 4 * (mb & 1) + rr : 16 * ib + 4 * mb + rr);
         // canonical coordinates of the row
         int64_t R16 = r >> 4;
         int q = (int)((r >> 2) & 3), p = (int)((r >> 1) & 1), sbit = (int)(r & 1);
@@ -593,6 +594,239 @@ static hipError_t launch_pipe(const SpmmParams& p, hipStream_t stream) {
     const int tiles = p.tiles_m * p.tiles_n;
     const int chunk = (tiles + 7) / 8;
     hipLaunchKernelGGL(kern, dim3(chunk * 8), dim3(WM * WN * 64), lds, stream, p);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Pipelined kernel for V = 32 (any V that is a multiple of 32 but not of 64).
+//
+// A 64-row wave tile then spans two V blocks, each with its own column-loc, so a stage holds TWO
+// gathered sets of 64 B rows and the packed operands use the "half tile" row order: instruction
+// row (mb, 4*ib + r) holds tile row 32*(mb/2) + 8*ib + 4*(mb%2) + r, so that instructions 0, 1
+// multiply the first set and instructions 2, 3 the second.  A lane ends up with two runs of 8
+// consecutive matrix rows (8*ib .. +7 and 32 + 8*ib .. +7) of one output column.
+// The row tables of the tile's two halves sit in LDS as 16-bit row numbers (0xffff = zero row).
+// Tile 64 x (64*WN), one wave per 64 columns; everything else as in spmm_pipe_kernel.
+// ---------------------------------------------------------------------------
+#define SPATHA_MMA2LO(NB, BF)                                                                                 \
+    acc[0][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[0], BF, acc[0][NB], (int)i0, 0, 0);           \
+    acc[1][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], BF, acc[1][NB], (int)i0, 0, 1);
+#define SPATHA_MMA2HI(NB, BF)                                                                                 \
+    acc[2][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], BF, acc[2][NB], (int)i1, 0, 0);           \
+    acc[3][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], BF, acc[3][NB], (int)i1, 0, 1);
+
+template <int WN, int NS, int OUT_LAYOUT>
+__global__ __launch_bounds__(WN * 64) void spmm_half_kernel(SpmmParams p) {
+    constexpr int BN = WN * 64;
+    constexpr int ROW_BYTES = BN * 2;
+    constexpr int B_BYTES = 64 * ROW_BYTES;          // one gathered set
+    constexpr int STAGE_BYTES = 2 * B_BYTES + APACK_BLOCK;
+    constexpr int CHUNKS = BN / 8;
+    constexpr int RPI = 1024 / ROW_BYTES;            // rows one DMA instruction covers
+    constexpr int NB_LOADS = 128 / RPI / WN;         // B DMA instructions per wave per stage (both sets)
+    constexpr int NA_X4 = 4 / WN;
+    constexpr int L = NB_LOADS + NA_X4 + 1;
+    constexpr int PA = NS - 1;
+    constexpr int PITCH_C = 144;
+    static_assert(WN == 2 || WN == 4, "A operand split");
+    static_assert((NS - 2) * L < 64, "vmcnt range");
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    uint16_t* lds_rt = (uint16_t*)(smem + NS * STAGE_BYTES);      // [S][2 halves][64] row numbers
+
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int chunk = (tiles + 7) >> 3;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int tile = xcd * chunk + local;
+    if (local >= chunk || tile >= tiles) return;
+    const int tile_n = tile / p.tiles_m, tile_m = tile - tile_n * p.tiles_m;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wn = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m0 = tile_m * 64, n0 = tile_n * BN;
+    const int S = p.S, N = p.N;
+    const char* a_src = (const char*)p.apack + ((int64_t)tile_m * S) * APACK_BLOCK;
+
+    const int slot_row = lane / CHUNKS;
+    const int slot_chunk = lane % CHUNKS;
+    int64_t b_col_off[NB_LOADS];
+    const char* zero_src = (const char*)p.zeros + lane * 16;
+#pragma unroll
+    for (int j = 0; j < NB_LOADS; j++) {
+        const int rho = (wn * NB_LOADS + j) * RPI + slot_row;          // 0..127; the swizzle only sees rho % 8
+        const int src_chunk = slot_chunk ^ ((rho & 7) << 1);
+        const int col = n0 + src_chunk * 8;
+        b_col_off[j] = (col < N) ? (int64_t)col * 2 : -1;
+    }
+    auto issue_stage = [&](int s) {
+        const uint32_t stage = smem_base + (s % NS) * STAGE_BYTES;
+        uint32_t rows[NB_LOADS];
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) rows[j] = lds_rt[s * 128 + (wn * NB_LOADS + j) * RPI + slot_row];
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) {
+            const int inst = wn * NB_LOADS + j;
+            const bool ok = (rows[j] != 0xffffu) && (b_col_off[j] >= 0);
+            const char* src = (const char*)p.B + (int64_t)rows[j] * N * 2 + b_col_off[j];
+            src = ok ? src : zero_src;
+            dma_b128(src, stage + inst * 1024);                        // set 1 starts at B_BYTES = 64 rows
+        }
+        const char* ab = a_src + (int64_t)s * APACK_BLOCK;
+        const uint32_t a_lds = stage + 2 * B_BYTES;
+#pragma unroll
+        for (int k = 0; k < NA_X4; k++) {
+            const int mb = (WN >= 4) ? wn : wn * NA_X4 + k;
+            dma_b128(ab + mb * 1024 + lane * 16, a_lds + mb * 1024);
+        }
+        const int d = wn & 1;
+        dma_b32(ab + 4096 + d * 256 + lane * 4, a_lds + 4096 + d * 256);
+    };
+
+    float4_t acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+    const int li = lane & 15, kb = lane >> 4;
+    const int rrow = kb * 4 + (li >> 2);
+    const int sw = rrow & 7;
+    int tr_off[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int ch = (wn * 8 + nb * 2 + ((li & 3) >> 1)) ^ (sw << 1);
+        tr_off[nb] = rrow * ROW_BYTES + ch * 16 + (li & 1) * 8;
+    }
+    const int a_off = 2 * B_BYTES + lane * 16;
+    const int i_off = 2 * B_BYTES + 4096 + lane * 4;
+
+    // ---- row tables of the two halves -> LDS (ordinary loads, before any DMA is in flight)
+    {
+        const uint32_t* rt0 = p.rowtab + (int64_t)(m0 / p.v) * S * 64;
+        const uint32_t* rt1 = p.rowtab + (int64_t)((m0 + 32) / p.v) * S * 64;
+        for (int i = tid; i < S * 128; i += WN * 64) {
+            const int s = i >> 7, rho = i & 63;
+            const uint32_t r = ((i & 64) ? rt1 : rt0)[s * 64 + rho];
+            lds_rt[i] = (r == 0xffffffffu) ? (uint16_t)0xffffu : (uint16_t)r;
+        }
+    }
+    __syncthreads();
+
+#pragma unroll
+    for (int t = 0; t < PA; t++)
+        if (t < S) issue_stage(t);
+
+    for (int s = 0; s < S; s++) {
+        const int later = (S - 1 - s) < (NS - 2) ? (S - 1 - s) : (NS - 2);
+        wait_stages<L, NS - 2>(later);
+        __syncthreads();
+        const char* st = smem + (s % NS) * STAGE_BYTES;
+        half8_t a_cur[4];
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) a_cur[mb] = *(const half8_t*)(st + a_off + mb * 1024);
+        const uint32_t i0 = *(const uint32_t*)(st + i_off), i1 = *(const uint32_t*)(st + i_off + 256);
+        half16_t lo0 = read_b_fragment<ROW_BYTES>(st, tr_off[0]);
+        half16_t hi0 = read_b_fragment<ROW_BYTES>(st + B_BYTES, tr_off[0]);
+        half16_t lo1 = read_b_fragment<ROW_BYTES>(st, tr_off[1]);
+        half16_t hi1 = read_b_fragment<ROW_BYTES>(st + B_BYTES, tr_off[1]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s + PA < S) issue_stage(s + PA);
+        __builtin_amdgcn_sched_barrier(0);
+        SPATHA_MMA2LO(0, lo0)
+        SPATHA_MMA2HI(0, hi0)
+        __builtin_amdgcn_sched_barrier(0);
+        lo0 = read_b_fragment<ROW_BYTES>(st, tr_off[2]);
+        hi0 = read_b_fragment<ROW_BYTES>(st + B_BYTES, tr_off[2]);
+        __builtin_amdgcn_sched_barrier(0);
+        SPATHA_MMA2LO(1, lo1)
+        SPATHA_MMA2HI(1, hi1)
+        __builtin_amdgcn_sched_barrier(0);
+        lo1 = read_b_fragment<ROW_BYTES>(st, tr_off[3]);
+        hi1 = read_b_fragment<ROW_BYTES>(st + B_BYTES, tr_off[3]);
+        __builtin_amdgcn_sched_barrier(0);
+        SPATHA_MMA2LO(2, lo0)
+        SPATHA_MMA2HI(2, hi0)
+        SPATHA_MMA2LO(3, lo1)
+        SPATHA_MMA2HI(3, hi1)
+    }
+
+    // ------------------------------------------------------------------ write-out
+    const int j = lane & 15, ib = lane >> 4;
+    if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+        // per output column the lane holds rows 8*ib .. +7 (instructions 0, 1) and 32 + 8*ib .. +7 (2, 3)
+        const int64_t row_lo = (int64_t)m0 + ib * 8, row_hi = row_lo + 32;
+        half8_t bias_lo, bias_hi;
+        if (p.bias) {
+            bias_lo = *(const half8_t*)(p.bias + row_lo);
+            bias_hi = *(const half8_t*)(p.bias + row_hi);
+        }
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+            const int col = n0 + wn * 64 + nb * 16 + j;
+            half8_t lo, hi;
+#pragma unroll
+            for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
+                    hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
+                }
+            if (p.bias) {
+                lo = lo + bias_lo;
+                hi = hi + bias_hi;
+            }
+            if (col < N) {
+                uint16_t* dst = p.C + (int64_t)col * p.rows;
+                *(half8_t*)(dst + row_lo) = lo;
+                *(half8_t*)(dst + row_hi) = hi;
+            }
+        }
+    } else {
+        __syncthreads();                 // every wave is done reading the stages
+        char* stg = smem + wn * (64 * PITCH_C);
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int Lr = (4 * mb + r) * 4 + ib;
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++)
+                    *(_Float16*)(stg + Lr * PITCH_C + (nb * 16 + j) * 2) = (_Float16)acc[mb][nb][r];
+            }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+            const int Lr = it * 8 + (lane >> 3), ch = lane & 7;
+            // slab row Lr = (4*mb + r)*4 + ib  ->  tile row 32*(mb/2) + 8*ib + 4*(mb%2) + r
+            const int row = 32 * (Lr >> 5) + 8 * (Lr & 3) + 4 * ((Lr >> 4) & 1) + ((Lr >> 2) & 3);
+            const int col = n0 + wn * 64 + ch * 8;
+            u32x4 v = *(const u32x4*)(stg + Lr * PITCH_C + ch * 16);
+            if (col < N) *(u32x4*)(p.C + ((int64_t)m0 + row) * N + col) = v;
+        }
+    }
+}
+
+template <int WN, int NS>
+constexpr int half_stage_bytes() { return NS * (2 * 64 * WN * 128 + APACK_BLOCK); }
+
+template <int WN, int NS, int OUT_LAYOUT>
+static hipError_t launch_half(const SpmmParams& p, hipStream_t stream) {
+    constexpr int stage_bytes = half_stage_bytes<WN, NS>();
+    static_assert(stage_bytes >= WN * 64 * 144, "the write-out staging reuses the stage buffers");
+    const int lds = stage_bytes + p.S * 256;
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    static bool attr_set = false;
+    auto kern = spmm_half_kernel<WN, NS, OUT_LAYOUT>;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int chunk = (tiles + 7) / 8;
+    hipLaunchKernelGGL(kern, dim3(chunk * 8), dim3(WN * 64), lds, stream, p);
     return hipGetLastError();
 }
 
@@ -2797,6 +3031,9 @@ const char* spmm_variant_name(int variant) {
         case SPMM_VARIANT_DS256x128_S3_PP: return "smfmac16x16x64_warpspec_densestage_tile256x128_3stage_pingpong";
         case SPMM_VARIANT_DSF256x128_S3: return "smfmac16x16x64_warpspec_densestage_flagsync_tile256x128_3stage";
         case SPMM_VARIANT_SKINNY: return "smfmac16x16x64_skinny_tile64xN_splitk4";
+        case SPMM_VARIANT_H64x256_S2: return "smfmac16x16x64_halftile_ldsdirect_tile64x256_2stage";
+        case SPMM_VARIANT_H64x128_S3: return "smfmac16x16x64_halftile_ldsdirect_tile64x128_3stage";
+        case SPMM_VARIANT_H64x128_S2: return "smfmac16x16x64_halftile_ldsdirect_tile64x128_2stage";
         default: return nullptr;
     }
 }
@@ -2834,6 +3071,9 @@ int spmm_variant_lds(int variant, int S) {
         case SPMM_VARIANT_DS256x128_S3_PP: return DsCfg<8, 3, 4, 8>::LDS_BYTES;
         case SPMM_VARIANT_DSF256x128_S3: return DsfCfg<8, 3, 4>::LDS_BYTES;
         case SPMM_VARIANT_SKINNY: return 64 * 1024;
+        case SPMM_VARIANT_H64x256_S2: return half_stage_bytes<4, 2>() + S * 256;
+        case SPMM_VARIANT_H64x128_S3: return half_stage_bytes<2, 3>() + S * 256;
+        case SPMM_VARIANT_H64x128_S2: return half_stage_bytes<2, 2>() + S * 256;
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_64x256: return 1;
         default: return 0;
     }
@@ -2848,7 +3088,7 @@ int spmm_variant_bm(int variant) {
         case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5: return 128;
         case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_D64x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4:
-        case SPMM_VARIANT_SKINNY: return 64;
+        case SPMM_VARIANT_SKINNY: case SPMM_VARIANT_H64x256_S2: case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2: return 64;
         case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3: return 256;
         default: return 0;
     }
@@ -2859,8 +3099,10 @@ int spmm_variant_bn(int variant) {
         case SPMM_VARIANT_R128x128_S4: case SPMM_VARIANT_R128x128_S5: case SPMM_VARIANT_R128x128_S2:
         case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2:
         case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5:
-        case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3: return 128;
+        case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3:
+        case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2: return 128;
         case SPMM_VARIANT_SKINNY: return 64;
+        case SPMM_VARIANT_H64x256_S2: return 256;
         case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D64x256_S3: case SPMM_VARIANT_T128x256_S3:
         case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_W128x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4: return 256;
@@ -2934,6 +3176,14 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
     SPATHA_DS_CASE(SPMM_VARIANT_DS256x128_S2, 2, 4)
     SPATHA_DS_CASE(SPMM_VARIANT_DS256x128_S3_C8, 3, 8)
 #undef SPATHA_DS_CASE
+#define SPATHA_HALF_CASE(ID, WN_, NS_)                                                                  \
+    if (variant == ID)                                                                                  \
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_half<WN_, NS_, SPATHA_OUT_TRANSPOSED>(p, stream) \
+                                                   : launch_half<WN_, NS_, SPATHA_OUT_ROW_MAJOR>(p, stream);
+    SPATHA_HALF_CASE(SPMM_VARIANT_H64x256_S2, 4, 2)
+    SPATHA_HALF_CASE(SPMM_VARIANT_H64x128_S3, 2, 3)
+    SPATHA_HALF_CASE(SPMM_VARIANT_H64x128_S2, 2, 2)
+#undef SPATHA_HALF_CASE
     if (variant == SPMM_VARIANT_SKINNY)
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_skinny<SPATHA_OUT_TRANSPOSED>(p, stream)
                                                    : launch_skinny<SPATHA_OUT_ROW_MAJOR>(p, stream);
@@ -2947,11 +3197,11 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
 }
 
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
-                       int m, int v, int ksp, int S, uint16_t* apack, uint32_t* rowtab, hipStream_t stream) {
+                       int m, int v, int ksp, int S, int half_tiles, uint16_t* apack, uint32_t* rowtab, hipStream_t stream) {
     int64_t total_a = (int64_t)(rows / 64) * S * 256;
     int blocks_a = (int)((total_a + 255) / 256);
     if (blocks_a > 65535 * 8) blocks_a = 65535 * 8;
-    hipLaunchKernelGGL(pack_a_kernel, dim3(blocks_a), dim3(256), 0, stream, values, metadata, rows, ksp, S, apack);
+    hipLaunchKernelGGL(pack_a_kernel, dim3(blocks_a), dim3(256), 0, stream, values, metadata, rows, ksp, S, half_tiles, apack);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     int64_t total_r = (int64_t)(rows / v) * S * 64;

@@ -189,7 +189,16 @@ int main(int argc, const char** argv) {
     // ---- device
     uint16_t *dB, *dC, *dVal, *dDense, *dCref;
     uint32_t *dMeta, *dCols;
-    HIP_OK(hipMalloc((void**)&dB, hB.size() * 2));
+    // the dense baseline wants K to be a multiple of 8: zero columns of A / zero rows of B are appended for it
+    // (the SpMM is given the same B buffer with its true K)
+    const int kpad = (k + 7) / 8 * 8;
+    if (kpad != k) {
+        std::vector<uint16_t> padded((size_t)m * kpad, 0);
+        for (int r = 0; r < m; r++) std::memcpy(&padded[(size_t)r * kpad], &hDense[(size_t)r * k], (size_t)k * 2);
+        hDense.swap(padded);
+    }
+    HIP_OK(hipMalloc((void**)&dB, (size_t)kpad * n * 2));
+    HIP_OK(hipMemset(dB, 0, (size_t)kpad * n * 2));
     HIP_OK(hipMalloc((void**)&dC, (size_t)m * n * 2));
     HIP_OK(hipMalloc((void**)&dCref, (size_t)m * n * 2));
     HIP_OK(hipMalloc((void**)&dVal, hVal.size() * 2));
@@ -223,10 +232,10 @@ int main(int argc, const char** argv) {
         hipEvent_t e0, e1;
         HIP_OK(hipEventCreate(&e0));
         HIP_OK(hipEventCreate(&e1));
-        for (int i = 0; i < 3; i++) SPATHA_OK_OR_DIE(spatha_dense_gemm_f16(dDense, dB, m, k, n, dCref, nullptr));
+        for (int i = 0; i < 3; i++) SPATHA_OK_OR_DIE(spatha_dense_gemm_f16(dDense, dB, m, kpad, n, dCref, nullptr));
         const int reps = 20;
         HIP_OK(hipEventRecord(e0, nullptr));
-        for (int i = 0; i < reps; i++) SPATHA_OK_OR_DIE(spatha_dense_gemm_f16(dDense, dB, m, k, n, dCref, nullptr));
+        for (int i = 0; i < reps; i++) SPATHA_OK_OR_DIE(spatha_dense_gemm_f16(dDense, dB, m, kpad, n, dCref, nullptr));
         HIP_OK(hipEventRecord(e1, nullptr));
         HIP_OK(hipEventSynchronize(e1));
         HIP_OK(hipEventElapsedTime(&gemm_ms, e0, e1));

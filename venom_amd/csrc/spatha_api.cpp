@@ -71,7 +71,8 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
     const int v = plan->geo.v;
     int order[4] = {0, 0, 0, 0};
     // few columns: streaming A is all that matters, one 64-row tile per workgroup with the k-steps split over its waves
-    if (N <= 16 && variant_ok(plan, N, SPMM_VARIANT_SKINNY)) return SPMM_VARIANT_SKINNY;
+    // (N = 32: equal on the GPT-3 FFN matrix, 1.3-1.5x ahead on the BERT-large ones; N = 48, 64: behind the 128-wide tiles)
+    if (N <= 32 && variant_ok(plan, N, SPMM_VARIANT_SKINNY)) return SPMM_VARIANT_SKINNY;
     if (plan->half_tiles) {
         // measured (1024 x 4096 x 4096 and 4096 x 1024 x 16384, m = 8..32): the 256-wide tile is never behind the
         // 128-wide one with two stages by more than 7 %, and up to 2x ahead; three stages of 128 leave two waves per CU
@@ -273,10 +274,11 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
     p.b_bytes = (uint32_t)((uint64_t)plan->geo.cols * (uint64_t)N * 2u);     // only read by variants that passed variant_ok
     p.apack_bytes = (uint32_t)plan->apack_bytes;
     p.rowtab_bytes = (uint32_t)plan->rowtab_bytes;
+    p.debug = 0; p.skew = 0; p.prof = nullptr;
+#ifdef SPATHA_DEV_PROFILE
+    // development builds only: switch parts of a kernel off for time accounting (results are then wrong on purpose)
     { const char* d = std::getenv("SPATHA_DEBUG_KNOBS"); p.debug = d ? std::atoi(d) : 0; }
     { const char* d = std::getenv("SPATHA_SKEW"); p.skew = d ? std::atoi(d) : 0; }
-    p.prof = nullptr;
-#ifdef SPATHA_DEV_PROFILE
     { const char* d = std::getenv("SPATHA_PROF_PTR"); if (d) p.prof = (long long*)std::strtoull(d, nullptr, 0); }
 #endif
     hipError_t e = spatha::launch_spmm(var, out_layout, p, (hipStream_t)stream);

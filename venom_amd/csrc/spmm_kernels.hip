@@ -35,6 +35,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "spmm_kernels.h"
 
 namespace spatha {
@@ -49,6 +51,20 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+// "Dynamic LDS limit raised" flags, one per (kernel, device): the attribute is a per-device property of a kernel.
+static bool& lds_attr_flag(const void* kern) {
+    struct Entry { const void* kern; bool set[16]; };
+    static Entry table[256] = {};
+    static std::mutex lock;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    std::lock_guard<std::mutex> guard(lock);
+    int i = 0;
+    while (i < 255 && table[i].kern && table[i].kern != kern) i++;
+    table[i].kern = kern;
+    return table[i].set[dev & 15];
+}
 
 // ---------------------------------------------------------------------------
 // pack_kernel: canonical (values, metadata, columns) -> (apack, ipack, rowtab)
@@ -584,8 +600,8 @@ static hipError_t launch_pipe(const SpmmParams& p, hipStream_t stream) {
     static_assert(stage_bytes >= WM * WN * 64 * 144, "the epilogue staging reuses the stage buffers");
     const int lds = stage_bytes + p.S * 256;
     if (lds > 160 * 1024) return hipErrorInvalidValue;     // callers check with spmm_variant_fits first
-    static bool attr_set = false;
     auto kern = spmm_pipe_kernel<WM, WN, NS, OUT_LAYOUT>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
@@ -817,8 +833,8 @@ static hipError_t launch_half(const SpmmParams& p, hipStream_t stream) {
     static_assert(stage_bytes >= WN * 64 * 144, "the write-out staging reuses the stage buffers");
     const int lds = stage_bytes + p.S * 256;
     if (lds > 160 * 1024) return hipErrorInvalidValue;
-    static bool attr_set = false;
     auto kern = spmm_half_kernel<WN, NS, OUT_LAYOUT>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
@@ -1136,9 +1152,9 @@ static hipError_t launch_persist(const SpmmParams& p, hipStream_t stream) {
     using Cfg = PersistCfg<WM, WN, NS>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static bool attr_set = false;
     static int cus = 0;
     auto kern = spmm_persist_kernel<WM, WN, NS, OUT_LAYOUT>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
@@ -1748,9 +1764,9 @@ static hipError_t launch_wst(const SpmmParams& p, hipStream_t stream) {
     using Cfg = WsCfg<2, WN, NS, NP>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static bool attr_set = false;
     static int cus = 0;
     auto kern = spmm_wst_kernel<WN, NS, NP, OUT_LAYOUT>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
@@ -2336,11 +2352,11 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static_assert(!PINGPONG || NC == 8, "ping-pong needs eight consumer waves");
-    static bool attr_set = false;
     static int cus = 0;
     void (*kern)(SpmmParams);
     if constexpr (PINGPONG) kern = spmm_dspp_kernel<M, NS, NP, OUT_LAYOUT>;
     else kern = spmm_ds_kernel<M, NS, NP, NC, OUT_LAYOUT>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
@@ -2715,9 +2731,9 @@ static hipError_t launch_dsf(const SpmmParams& p, hipStream_t stream) {
     using Cfg = DsfCfg<M, NS, NP>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static bool attr_set = false;
     static int cus = 0;
     auto kern = spmm_dsf_kernel<M, NS, NP, OUT_LAYOUT>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
@@ -2953,9 +2969,9 @@ static hipError_t launch_ws(const SpmmParams& p, hipStream_t stream) {
     using Cfg = WsCfg<WM, WN, NS, NP>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static bool attr_set = false;
     static int cus = 0;
     auto kern = spmm_ws_kernel<WM, WN, NS, NP, OUT_LAYOUT, DEFER>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
@@ -2984,8 +3000,8 @@ static hipError_t launch_variant(const SpmmParams& p, hipStream_t stream) {
     constexpr int stage_bytes = 2 * 64 * (BN * 2 + 32);
     constexpr int epi_bytes = WM * WN * 64 * 144;
     constexpr int lds = stage_bytes > epi_bytes ? stage_bytes : epi_bytes;
-    static bool attr_set = false;
     auto kern = spmm_kernel<WM, WN, OUT_LAYOUT>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set && lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;

@@ -156,6 +156,22 @@ int spatha_spmm_plan_destroy(spatha_spmm_plan* plan);
 int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
                     uint16_t* out_dev, int out_layout, int variant, void* stream);
 
+#define SPATHA_ACT_NONE 0
+#define SPATHA_ACT_GELU 1        /* 0.5 x (1 + erf(x / sqrt 2))                                   */
+#define SPATHA_ACT_GELU_TANH 2   /* 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))  ("gelu_new") */
+
+/* spatha_spmm_run with the layer's elementwise tail fused into the write-out: in either layout
+ *   out = act(fp16(fp16(A B) + bias[row]))
+ * (bias may be NULL, act may be SPATHA_ACT_NONE; the activation is evaluated in fp32 on the fp16 sum and
+ * rounded once).  The bias part is the reference's fused epilogue (blockwise_kernel.h:294-343) made available
+ * to the row-major layout as well; the activation has no counterpart in the reference's kernels, whose
+ * callers apply it as a separate elementwise pass over the output (the feed-forward block of the models in
+ * end2end/).  Row-major output with bias lets a following spatha_spmm_run consume `out` as its B operand
+ * without a transposed copy.  Kernels without the fused write-out are skipped by the automatic choice and
+ * refused (SPATHA_ERR_UNSUPPORTED) when named. */
+int spatha_spmm_run_fused(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
+                          uint16_t* out_dev, int out_layout, int activation, int variant, void* stream);
+
 /* Kernel variants are numbered 1 .. spatha_spmm_num_variants() - 1; 0 selects automatically. */
 int spatha_spmm_num_variants(void);
 

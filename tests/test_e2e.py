@@ -136,3 +136,53 @@ def test_gpt2_conv1d_swap_tracks_masked_dense(gpu):
     b = dense(ids).last_hidden_state.float()
     assert torch.isfinite(a).all()
     assert (a - b).abs().max().item() <= 5e-2
+
+
+@pytest.mark.gpu
+def test_fused_feed_forward_tracks_the_unfused_layers(gpu):
+    """BertIntermediate as one kernel (bias + GELU in the write-out, feature-major result consumed by the next
+    layer without a copy) against the same model with the drop-in layers."""
+    from venom_amd.bert import FusedFeedForwardIn, SrnmSpmm, build_bert_large, fuse_feed_forward, linear_to_spmm
+
+    torch.set_grad_enabled(False)
+    plain = linear_to_spmm(build_bert_large(layers=2).to(gpu).half(), 2, 8, 64)
+    fused = fuse_feed_forward(linear_to_spmm(build_bert_large(layers=2).to(gpu).half(), 2, 8, 64))
+    in_kernel = fuse_feed_forward(linear_to_spmm(build_bert_large(layers=2).to(gpu).half(), 2, 8, 64), activation_in_kernel=True)
+    assert sum(isinstance(mod, FusedFeedForwardIn) for mod in fused.modules()) == 2
+    ids = torch.randint(0, 30522, (2, 64), device=gpu)
+    a = plain(ids).last_hidden_state
+    b = fused(ids).last_hidden_state
+    c = in_kernel(ids).last_hidden_state.float()
+    # bias in the kernel, torch's GELU on the feature-major buffer: the same numbers in another layout, bit for bit
+    assert torch.equal(a, b)
+    # GELU in the write-out as well: one fp16 step here and there
+    assert torch.isfinite(c).all() and (a.float() - c).abs().max().item() <= 1e-2
+    # the feature-major intermediate reaches the second feed-forward layer as a view: no transposed copy is made
+    layer = fused.encoder.layer[0]
+    x = torch.randn((2, 64, 1024), device=gpu).half()
+    mid = layer.intermediate(x)
+    assert mid.shape == (2, 64, 4096) and mid.stride() == (64, 1, 128)
+    flat = torch.flatten(mid, 0, -2)
+    assert SrnmSpmm._transposed(flat).data_ptr() == mid.data_ptr()
+    want = torch.nn.functional.gelu(plain.encoder.layer[0].intermediate.dense(x))
+    assert torch.equal(mid, want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("in_kernel", [False, True])
+def test_fused_gpt2_mlp_tracks_the_unfused_block(gpu, in_kernel):
+    from venom_amd.bert import FusedFeedForwardIn, fuse_feed_forward
+    from venom_amd.gpt2 import build_gpt2_large, conv1d_to_spmm
+
+    torch.set_grad_enabled(False)
+    plain = conv1d_to_spmm(build_gpt2_large(layers=2, width=256, heads=4).to(gpu).half(), 2, 8, 64)
+    fused = fuse_feed_forward(conv1d_to_spmm(build_gpt2_large(layers=2, width=256, heads=4).to(gpu).half(), 2, 8, 64),
+                              activation_in_kernel=in_kernel)
+    assert sum(isinstance(mod, FusedFeedForwardIn) for mod in fused.modules()) == 2
+    ids = torch.randint(0, 100, (2, 64), device=gpu)
+    a = plain(ids).last_hidden_state
+    b = fused(ids).last_hidden_state
+    if in_kernel:      # one rounding instead of the eight of the block's elementwise chain
+        assert (a.float() - b.float()).abs().max().item() <= 2e-2
+    else:              # same operations on the same numbers in another layout
+        assert torch.equal(a, b)

@@ -73,6 +73,8 @@ class SrnmSpmm(torch.nn.Module):
 
     @classmethod
     def _transposed(cls, flat):
+        if flat.stride(0) == 1 and flat.stride(1) == flat.shape[0]:
+            return flat.T              # feature-major already (the output of a fused feed-forward layer): no copy
         key = (flat.data_ptr(), tuple(flat.shape), tuple(flat.stride()), flat._version, flat.device)
         if cls._last_rhs[0] == key:
             return cls._last_rhs[2]
@@ -90,6 +92,70 @@ class SrnmSpmm(torch.nn.Module):
         out = spatha.spmm(self.metadata, self.columns, self.values, rhs, bias, self.nrows_sp, self.ncols_sp,
                           rhs.shape[1], self.v, self.n, self.m, self.nnz, 0, 32, 4)   # [tokens, out]
         return out.reshape(*input.shape[:-1], -1)
+
+    def forward_feature_major(self, input, activation="none"):
+        """act(x W^T + b) as a [..., out] VIEW of a feature-major buffer [out, tokens]: bias and activation run in
+        the kernel's write-out, and the next SrnmSpmm takes the buffer as its right-hand side without a copy."""
+        flat = torch.flatten(input, start_dim=0, end_dim=-2)
+        rhs = self._transposed(flat)
+        out = spatha.spmm_fused(self.metadata, self.columns, self.values, rhs, self.bias, self.nrows_sp, self.ncols_sp,
+                                self.v, self.n, self.m, activation=activation)              # [out, tokens]
+        return out.T.reshape(*input.shape[:-1], -1)     # strides (.., 1, tokens): a view, nothing moves
+
+
+class FusedFeedForwardIn(torch.nn.Module):
+    """Stands in for the Linear that opens a feed-forward block: one kernel computes x W^T + b (bias in the write-out)
+    and leaves it feature-major, [out, tokens], which the block's second SrnmSpmm takes as its right-hand side as it
+    lies, so the [tokens, 4*hidden] activation is never transposed.  The value returned is a [..., out] VIEW of that
+    buffer; elementwise code between the two layers keeps its strides.
+    activation: None (the caller applies its own), or "gelu" / "gelu_tanh" applied here, by torch's elementwise kernel
+    (same bits as the unfused layers) or, with activation_in_kernel, in the SpMM's write-out (one pass less)."""
+
+    def __init__(self, spmm_layer, activation=None, activation_in_kernel=False):
+        super().__init__()
+        self.dense = spmm_layer
+        self.activation = activation
+        self.activation_in_kernel = activation_in_kernel
+
+    def forward(self, hidden_states):
+        if self.activation is None:
+            return self.dense.forward_feature_major(hidden_states, "none")
+        if self.activation_in_kernel:
+            return self.dense.forward_feature_major(hidden_states, self.activation)
+        approx = "tanh" if self.activation != "gelu" else "none"
+        return torch.nn.functional.gelu(self.dense.forward_feature_major(hidden_states, "none"), approximate=approx)
+
+
+def fuse_feed_forward(model, activation_in_kernel=False):
+    """Rewires, in place, every feed-forward block whose two projections are SrnmSpmm layers already: transformers'
+    BertIntermediate (Linear + GELU) and GPT2MLP (c_fc, activation, c_proj).  Layers with V = 32, 96, ... keep the
+    drop-in path (their kernels have no fused write-out)."""
+    from transformers import activations as A
+    from transformers.models.bert.modeling_bert import BertIntermediate
+    from transformers.models.gpt2.modeling_gpt2 import GPT2MLP
+
+    def kernel_name_of(fn):
+        if isinstance(fn, A.GELUActivation) or fn is torch.nn.functional.gelu:
+            return "gelu"
+        if isinstance(fn, (A.NewGELUActivation, getattr(A, "PytorchGELUTanh", ()), getattr(A, "GELUTanh", ()))):
+            return "gelu_tanh"
+        return None
+
+    for mod in model.modules():
+        for name, child in list(mod.named_children()):
+            if isinstance(child, BertIntermediate) and isinstance(child.dense, SrnmSpmm) and child.dense.v % 64 == 0:
+                act = kernel_name_of(child.intermediate_act_fn)
+                if act == "gelu":
+                    setattr(mod, name, FusedFeedForwardIn(child.dense, act, activation_in_kernel))
+            elif isinstance(child, GPT2MLP) and isinstance(child.c_fc, SrnmSpmm) and isinstance(child.c_proj, SrnmSpmm) \
+                    and child.c_fc.v % 64 == 0:
+                act = kernel_name_of(child.act)
+                if activation_in_kernel and act is not None:
+                    child.c_fc = FusedFeedForwardIn(child.c_fc, act, True)
+                    child.act = torch.nn.Identity()
+                else:
+                    child.c_fc = FusedFeedForwardIn(child.c_fc, None)       # the block's own activation follows
+    return model
 
 
 def linear_to_spmm(mod, n, m, v, magnitude=False, prefix="", only=("encoder.layer",)):
@@ -130,12 +196,20 @@ def main(argv=None):
     ap.add_argument("--seq", type=int, default=512)
     ap.add_argument("--repeats", type=int, default=30)
     ap.add_argument("--magnitude", action="store_true", help="magnitude column selection instead of the fixed pattern")
+    ap.add_argument("--fuse-ffn", action="store_true",
+                    help="first feed-forward layer of every block as one kernel (bias + GELU in the write-out, feature-major "
+                         "result handed to the second layer without a transposed copy)")
+    ap.add_argument("--kernel-gelu", action="store_true",
+                    help="with --fuse-ffn: GELU in the kernel's write-out too (default: torch's elementwise pass over the "
+                         "feature-major buffer, which keeps the model's output bit-identical to the unfused layers)")
     args = ap.parse_args(argv)
     torch.set_grad_enabled(False)
     dev = torch.device("cuda:0")
     dense_model = build_bert_large(args.layers).to(dev).half()
     sparse_model = build_bert_large(args.layers)
     sparse_model = linear_to_spmm(sparse_model.to(dev).half(), args.n, args.m, args.v, args.magnitude)
+    if args.fuse_ffn:
+        fuse_feed_forward(sparse_model, activation_in_kernel=args.kernel_gelu)
     ids = torch.randint(0, 30522, (args.batch, args.seq), device=dev)
 
     def run(model):
@@ -148,7 +222,9 @@ def main(argv=None):
     t_dense = report_time("dense", timeit.repeat(lambda: run(dense_model), repeat=args.repeats, number=1), 1, args.n, args.m, args.v)
     timeit.repeat(lambda: run(sparse_model), repeat=5, number=1)
     t_sparse = report_time("n:m", timeit.repeat(lambda: run(sparse_model), repeat=args.repeats, number=1), 1, args.n, args.m, args.v)
-    print("# dense %.2f ms, %d:%d:%d %.2f ms, speed-up %.2fx" % (t_dense, args.v, args.n, args.m, t_sparse, t_dense / t_sparse))
+    print("# dense %.2f ms, %d:%d:%d%s %.2f ms, speed-up %.2fx" % (t_dense, args.v, args.n, args.m,
+                                                                    " (fused feed-forward)" if args.fuse_ffn else "", t_sparse,
+                                                                    t_dense / t_sparse))
 
 
 if __name__ == "__main__":

@@ -35,9 +35,18 @@ inline int hip_fail(hipError_t e) {
     return SPATHA_ERR_HIP;
 }
 
-bool variant_ok(const spatha_spmm_plan* plan, int N, int variant) {
+// kernels whose write-out can apply bias and activation ahead of either output layout
+bool variant_has_fused_writeout(int variant) {
+    using namespace spatha;
+    return (variant >= SPMM_VARIANT_P128x128_S4 && variant <= SPMM_VARIANT_P64x256_S4) ||
+           (variant >= SPMM_VARIANT_W128x128_S5 && variant <= SPMM_VARIANT_W64x256_S3) ||
+           (variant >= SPMM_VARIANT_T128x256_S3 && variant <= SPMM_VARIANT_DS256x128_S3_C8);
+}
+
+bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = false) {
     using namespace spatha;
     if (variant <= 0 || variant >= SPMM_VARIANT_COUNT) return false;
+    if (fused && !variant_has_fused_writeout(variant)) return false;
     const int bm = spmm_variant_bm(variant);
     if (bm == 0) return false;
     const bool half_variant = variant == SPMM_VARIANT_H64x256_S2 || variant == SPMM_VARIANT_H64x128_S3 ||
@@ -65,14 +74,14 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant) {
 // Kernel choice.  V a multiple of 128: producer/consumer kernel on 128-row tiles; 256 columns wide
 // with 128 x 64 consumer waves when that still gives every CU at least two tiles, else 128 wide.  Otherwise (V a
 // multiple of 64 only) the 64 x 256 tile whose B rows are gathered per 64-row block.
-int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
+int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = false) {
     using namespace spatha;
-    if (variant != SPMM_VARIANT_AUTO) return variant_ok(plan, N, variant) ? variant : -1;
+    if (variant != SPMM_VARIANT_AUTO) return variant_ok(plan, N, variant, fused) ? variant : -1;
     const int v = plan->geo.v;
     int order[4] = {0, 0, 0, 0};
     // few columns: streaming A is all that matters, one 64-row tile per workgroup with the k-steps split over its waves
     // (N = 32: equal on the GPT-3 FFN matrix, 1.3-1.5x ahead on the BERT-large ones; N = 48, 64: behind the 128-wide tiles)
-    if (N <= 32 && variant_ok(plan, N, SPMM_VARIANT_SKINNY)) return SPMM_VARIANT_SKINNY;
+    if (N <= 32 && variant_ok(plan, N, SPMM_VARIANT_SKINNY, fused)) return SPMM_VARIANT_SKINNY;
     if (plan->half_tiles) {
         // measured (1024 x 4096 x 4096 and 4096 x 1024 x 16384, m = 8..32): the 256-wide tile is never behind the
         // 128-wide one with two stages by more than 7 %, and up to 2x ahead; three stages of 128 leave two waves per CU
@@ -80,7 +89,7 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
         order[1] = SPMM_VARIANT_H64x128_S2;
         order[2] = SPMM_VARIANT_H64x128_S3;
         for (int i = 0; i < 3; i++)
-            if (variant_ok(plan, N, order[i])) return order[i];
+            if (variant_ok(plan, N, order[i], fused)) return order[i];
         return -1;
     }
     if (v % 128 == 0) {
@@ -109,7 +118,7 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant) {
         return -1;
     }
     for (int i = 0; i < 4; i++)
-        if (variant_ok(plan, N, order[i])) return order[i];
+        if (variant_ok(plan, N, order[i], fused)) return order[i];
     return -1;
 }
 }  // namespace
@@ -254,14 +263,18 @@ int spatha_spmm_plan_destroy(spatha_spmm_plan* plan) {
     return first == hipSuccess ? SPATHA_OK : hip_fail(first);
 }
 
-int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
-                    uint16_t* out_dev, int out_layout, int variant, void* stream) {
+static int run_spmm(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, uint16_t* out_dev,
+                    int out_layout, int activation, bool fused_entry, int variant, void* stream) {
     if (!plan || !B_dev || !out_dev || N <= 0) return SPATHA_ERR_BAD_ARGUMENT;
     if (out_layout != SPATHA_OUT_ROW_MAJOR && out_layout != SPATHA_OUT_TRANSPOSED) return SPATHA_ERR_BAD_ARGUMENT;
-    if (out_layout == SPATHA_OUT_ROW_MAJOR && bias_dev) return SPATHA_ERR_BAD_ARGUMENT;
+    if (!fused_entry && out_layout == SPATHA_OUT_ROW_MAJOR && bias_dev) return SPATHA_ERR_BAD_ARGUMENT;
+    if (activation != SPATHA_ACT_NONE && activation != SPATHA_ACT_GELU && activation != SPATHA_ACT_GELU_TANH)
+        return SPATHA_ERR_BAD_ARGUMENT;
     if (N % 8 != 0) return SPATHA_ERR_BAD_SHAPE;      // 16-byte row segments of B and C
     if (((uintptr_t)B_dev & 15) || ((uintptr_t)out_dev & 15) || ((uintptr_t)bias_dev & 15)) return SPATHA_ERR_BAD_ARGUMENT;
-    int var = pick_variant(plan, N, variant);
+    // the bias of the transposed layout alone stays in the write-out itself
+    const bool fuse = activation != SPATHA_ACT_NONE || (out_layout == SPATHA_OUT_ROW_MAJOR && bias_dev);
+    int var = pick_variant(plan, N, variant, fuse);
     if (var < 0) return SPATHA_ERR_UNSUPPORTED;
     spatha::SpmmParams p;
     p.apack = plan->apack; p.rowtab = plan->rowtab;
@@ -274,6 +287,7 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
     p.b_bytes = (uint32_t)((uint64_t)plan->geo.cols * (uint64_t)N * 2u);     // only read by variants that passed variant_ok
     p.apack_bytes = (uint32_t)plan->apack_bytes;
     p.rowtab_bytes = (uint32_t)plan->rowtab_bytes;
+    p.fuse = fuse ? 1 : 0; p.act = activation;
     p.debug = 0; p.skew = 0; p.prof = nullptr;
 #ifdef SPATHA_DEV_PROFILE
     // development builds only: switch parts of a kernel off for time accounting (results are then wrong on purpose)
@@ -283,6 +297,16 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
 #endif
     hipError_t e = spatha::launch_spmm(var, out_layout, p, (hipStream_t)stream);
     return e == hipSuccess ? SPATHA_OK : hip_fail(e);
+}
+
+int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
+                    uint16_t* out_dev, int out_layout, int variant, void* stream) {
+    return run_spmm(plan, B_dev, N, bias_dev, out_dev, out_layout, SPATHA_ACT_NONE, false, variant, stream);
+}
+
+int spatha_spmm_run_fused(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
+                          uint16_t* out_dev, int out_layout, int activation, int variant, void* stream) {
+    return run_spmm(plan, B_dev, N, bias_dev, out_dev, out_layout, activation, true, variant, stream);
 }
 
 int spatha_spmm_num_variants(void) { return spatha::SPMM_VARIANT_COUNT; }

@@ -26,6 +26,8 @@ struct SpmmParams {
     int tiles_m, tiles_n;
     int skew;                 // start-up skew between workgroups, in units of 1024 clocks (0 = none)
     long long* prof;          // development cycle-accounting buffer (SPATHA_DEV_PROFILE builds), else null
+    int fuse;                 // 1: bias and activation are applied ahead of the write-out (fused_bias_act)
+    int act;                  // SPATHA_ACT_*
     int debug;                // development knobs (0 in production): 1 = skip B loads, 2 = skip C stores
 };
 

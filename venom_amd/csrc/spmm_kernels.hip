@@ -325,6 +325,64 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_kernel(SpmmParams p) {
 
 
 // ---------------------------------------------------------------------------
+// Fused epilogue ahead of a write-out, for a lane that holds rows row16 + 4*mb + r (standard operand order) of
+// its output columns:  t = fp16(acc);  t += bias[row] (one fp16 addition, as in the reference's fused bias,
+// end2end blockwise_kernel.h:324-341);  t = act(t), evaluated in fp32.  The write-out's own conversion to fp16 is
+// then exact without an activation and the single rounding of the activation's value with one.
+// Used when SpmmParams::fuse is set (row-major output with a bias, or any activation); the write-out is then
+// given no bias.
+// ---------------------------------------------------------------------------
+// x * Phi(x) with Phi through the complementary error function in its "t * exp(polynomial in t)" form
+// (t = 1 / (1 + z/2), z = |x| / sqrt 2; relative error of erfc below 1.2e-7 for every z), so that the negative
+// tail keeps its relative accuracy where 1 + erf(x / sqrt 2) would cancel: ~20 instructions instead of erff's ~70.
+__device__ __forceinline__ float act_gelu_erf(float x) {
+    const float z = fabsf(x) * 0.70710678118654752f;
+    const float t = __frcp_rn(fmaf(0.5f, z, 1.0f));
+    float q = fmaf(t, 0.17087277f, -0.82215223f);
+    q = fmaf(t, q, 1.48851587f);
+    q = fmaf(t, q, -1.13520398f);
+    q = fmaf(t, q, 0.27886807f);
+    q = fmaf(t, q, -0.18628806f);
+    q = fmaf(t, q, 0.09678418f);
+    q = fmaf(t, q, 0.37409196f);
+    q = fmaf(t, q, 1.00002368f);
+    q = fmaf(t, q, -1.26551223f);
+    const float half_erfc = 0.5f * t * __expf(fmaf(-z, z, q));       // 0.5 erfc(z) = Phi(-|x|)
+    return x * (x < 0.0f ? half_erfc : 1.0f - half_erfc);
+}
+__device__ __forceinline__ float act_gelu_tanh(float x) {
+    // 0.5 (1 + tanh u) = 1 / (1 + exp(-2u)): no cancellation for negative x; exp -> inf gives -0, exp -> 0 gives x
+    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    return x * __frcp_rn(1.0f + __expf(-2.0f * u));
+}
+template <int ACT>
+__device__ __forceinline__ void fused_bias_act_impl(float4_t (&acc)[4][4], const uint16_t* bias, int64_t row16) {
+    // one (mb, nb) group of four values at a time, fenced, so that the scheduler does not interleave all 64 chains
+    // of the activation and run out of registers next to the accumulators
+#pragma unroll
+    for (int mb = 0; mb < 4; mb++) {
+        half4_t bv = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+        if (bias) bv = *(const half4_t*)(bias + row16 + 4 * mb);
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+            float4_t v = acc[mb][nb];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float t = (float)((_Float16)v[r] + bv[r]);
+                v[r] = ACT == SPATHA_ACT_GELU ? act_gelu_erf(t) : ACT == SPATHA_ACT_GELU_TANH ? act_gelu_tanh(t) : t;
+            }
+            acc[mb][nb] = v;
+            if (ACT != SPATHA_ACT_NONE) __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+__device__ __forceinline__ void fused_bias_act(float4_t (&acc)[4][4], const uint16_t* bias, int64_t row16, int act) {
+    if (act == SPATHA_ACT_GELU) fused_bias_act_impl<SPATHA_ACT_GELU>(acc, bias, row16);
+    else if (act == SPATHA_ACT_GELU_TANH) fused_bias_act_impl<SPATHA_ACT_GELU_TANH>(acc, bias, row16);
+    else fused_bias_act_impl<SPATHA_ACT_NONE>(acc, bias, row16);
+}
+
+// ---------------------------------------------------------------------------
 // One k-step of a wave's 64 x 64 tile out of an LDS stage: 4 A operands + index words,
 // 4 B fragments (16 transposing reads), 16 sparse matrix instructions.  The B fragments are
 // double buffered in registers and `between` (the next stage's DMA issue) runs after the
@@ -540,12 +598,14 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_pipe_kernel(SpmmParams p) {
 
     // ------------------------------------------------------------------ epilogue
     const int j = lane & 15, ib = lane >> 4;
+    if (p.fuse) fused_bias_act(acc, p.bias, (int64_t)m0 + wm * 64 + ib * 16, p.act);
+    const uint16_t* bias = p.fuse ? nullptr : p.bias;
     if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
         const int64_t row0 = (int64_t)m0 + wm * 64 + ib * 16;
         half8_t bias_lo, bias_hi;
-        if (p.bias) {
-            bias_lo = *(const half8_t*)(p.bias + row0);
-            bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+        if (bias) {
+            bias_lo = *(const half8_t*)(bias + row0);
+            bias_hi = *(const half8_t*)(bias + row0 + 8);
         }
 #pragma unroll
         for (int nb = 0; nb < 4; nb++) {
@@ -558,7 +618,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_pipe_kernel(SpmmParams p) {
                     lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
                     hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
                 }
-            if (p.bias) {
+            if (bias) {
                 lo = lo + bias_lo;
                 hi = hi + bias_hi;
             }
@@ -1395,13 +1455,15 @@ __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk&
             c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
         }
         const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+        if (p.fuse) fused_bias_act(acc, p.bias, (int64_t)cm0 + wm * 64 + ib * 16, p.act);
+        const uint16_t* bias = p.fuse ? nullptr : p.bias;
         if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
             // the lane owns 16 consecutive matrix rows of one output column: 32 contiguous bytes
             const int64_t row0 = (int64_t)cm0 + wm * 64 + ib * 16;
             half8_t bias_lo, bias_hi;
-            if (p.bias) {
-                bias_lo = *(const half8_t*)(p.bias + row0);
-                bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+            if (bias) {
+                bias_lo = *(const half8_t*)(bias + row0);
+                bias_hi = *(const half8_t*)(bias + row0 + 8);
             }
 #pragma unroll
             for (int nb = 0; nb < 4; nb++) {
@@ -1414,7 +1476,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk&
                         lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
                         hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
                     }
-                if (p.bias) {
+                if (bias) {
                     lo = lo + bias_lo;
                     hi = hi + bias_hi;
                 }
@@ -1703,9 +1765,10 @@ __device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const Tile
         const int cm0 = c_tm * BM, cn0 = c_tn * BN;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
+            if (p.fuse) fused_bias_act(acc[h], p.bias, (int64_t)cm0 + h * 64 + ib * 16, p.act);
             if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
                 if (!(p.debug & 4))
-                    store_block_transposed_slab(acc[h], smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH), p.C, p.bias,
+                    store_block_transposed_slab(acc[h], smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH), p.C, p.fuse ? nullptr : p.bias,
                                                 (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !(p.debug & 2));
             } else if (!(p.debug & 4)) {
                 char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
@@ -1823,7 +1886,8 @@ constexpr int TR8_PITCH = 16;                      // 8 rows x 2 B
 constexpr int TR8_SLAB_BYTES = 64 * TR8_PITCH;     // per wave, 8 slab rows at a time (ROWS8: half the lanes write)
 template <bool ROWS8>
 __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4][4], char* stg, uint16_t* C, int64_t row0,
-                                                         int col0, int N, int lane, bool stores_on) {
+                                                         int col0, int N, int lane, bool stores_on,
+                                                         const uint16_t* bias = nullptr) {
     constexpr int PITCH = ROWS8 ? TR8_PITCH : TR_PITCH;
     const int j16 = lane & 15, ib = lane >> 4;     // as accumulator lane: column j16, rows 4*ib + r
     const int li = lane & 15, kb = lane >> 4;
@@ -1847,6 +1911,11 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
             for (int nb = 0; nb < 4; nb++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) h4[nb][r] = (_Float16)acc[mb][nb][r];
+            if (bias) {          // fp16 addition on the rounded product, rows row0 + 16*ib + 4*mb + r
+                const half4_t bv = *(const half4_t*)(bias + row0 + 16 * ib + 4 * mb);
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++) h4[nb] = h4[nb] + bv;
+            }
             if (ROWS8) {
                 if ((ib >> 1) == sidx) {
 #pragma unroll
@@ -2089,13 +2158,17 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
         SPATHA_PROF_MARK(0)
 #pragma unroll
         for (int h = 0; h < H; h++) {
+            // a bias alone rides in the row-major write-out itself (packed fp16 additions); anything else goes first
+            const bool pre = p.fuse && (p.act != SPATHA_ACT_NONE || OUT_LAYOUT == SPATHA_OUT_TRANSPOSED);
+            if (pre) fused_bias_act(acc[h], p.bias, (int64_t)cm0 + h * 64 + ib * 16, p.act);
             if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
                 if (!(p.debug & 4))
-                    store_block_transposed_slab(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, p.bias,
+                    store_block_transposed_slab(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, p.fuse ? nullptr : p.bias,
                                                 (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !(p.debug & 2));
             } else if (!(p.debug & 4)) {
                 store_block_row_major_tr<Cfg::NC == 8>(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C,
-                                                        (int64_t)cm0 + h * 64, cn0 + wn * 64, N, lane, !(p.debug & 2));
+                                                        (int64_t)cm0 + h * 64, cn0 + wn * 64, N, lane, !(p.debug & 2),
+                                                        (p.fuse && !pre) ? p.bias : nullptr);
             }
         }
         SPATHA_PROF_MARK(2)

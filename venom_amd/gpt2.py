@@ -66,11 +66,18 @@ def main(argv=None):
     ap.add_argument("--seq", type=int, default=512)
     ap.add_argument("--repeats", type=int, default=30)
     ap.add_argument("--magnitude", action="store_true", help="magnitude column selection instead of the fixed pattern")
+    ap.add_argument("--fuse-ffn", action="store_true",
+                    help="c_fc leaves its output (bias added in the kernel) feature-major for c_proj: no transposed copy of the "
+                         "[tokens, 4*width] activation")
+    ap.add_argument("--kernel-gelu", action="store_true", help="with --fuse-ffn: the activation in the kernel's write-out too")
     args = ap.parse_args(argv)
     torch.set_grad_enabled(False)
     dev = torch.device("cuda:0")
     dense_model = build_gpt2_large(args.layers).to(dev).half()
     sparse_model = conv1d_to_spmm(build_gpt2_large(args.layers).to(dev).half(), args.n, args.m, args.v, args.magnitude)
+    if args.fuse_ffn:
+        from .bert import fuse_feed_forward
+        fuse_feed_forward(sparse_model, activation_in_kernel=args.kernel_gelu)
     ids = torch.randint(0, 100, (args.batch, args.seq), device=dev)
 
     def run(model):

@@ -46,12 +46,17 @@ def main(argv=None):
     ap.add_argument("--tokens", type=int, default=4096)
     ap.add_argument("--repeats", type=int, default=30)
     ap.add_argument("--magnitude", action="store_true")
+    ap.add_argument("--fuse-ffn", action="store_true", help="c_fc leaves its output feature-major for c_proj (bias in the kernel)")
+    ap.add_argument("--kernel-gelu", action="store_true", help="with --fuse-ffn: the activation in the kernel's write-out too")
     args = ap.parse_args(argv)
     torch.set_grad_enabled(False)
     dev = torch.device("cuda:0")
     dense_block = build_gpt3_block(args.width, args.heads, args.tokens).half().to(dev)
     sparse_block = conv1d_to_spmm(build_gpt3_block(args.width, args.heads, args.tokens).half().to(dev), args.n, args.m, args.v,
                                   args.magnitude)
+    if args.fuse_ffn:
+        from .bert import fuse_feed_forward
+        fuse_feed_forward(sparse_block, activation_in_kernel=args.kernel_gelu)
     x = torch.rand((1, args.tokens, args.width), device=dev).half()
 
     def run(block):

@@ -15,13 +15,16 @@ def main(argv=None):
     ap.add_argument("--models", default="bert,gpt2,gpt3")
     ap.add_argument("--v", default="64,128")
     ap.add_argument("--m", default="8,16,32")
+    ap.add_argument("--fuse-ffn", action="store_true", help="passed on to the three harnesses")
+    ap.add_argument("--kernel-gelu", action="store_true", help="passed on to the three harnesses")
     args = ap.parse_args(argv)
+    extra = (["--fuse-ffn"] if args.fuse_ffn else []) + (["--kernel-gelu"] if args.kernel_gelu else [])
     print("algo,n,m,v,mean,median,std,len", flush=True)
     mains = {"bert": bert.main, "gpt2": gpt2.main, "gpt3": gpt3.main}
     for v in [int(x) for x in args.v.split(",")]:
         for name in args.models.split(","):
             for m in [int(x) for x in args.m.split(",")]:
-                mains[name](["-m", str(m), "-n", "2", "-v", str(v), "--repeats", str(args.repeats)])
+                mains[name](["-m", str(m), "-n", "2", "-v", str(v), "--repeats", str(args.repeats)] + extra)
 
 
 if __name__ == "__main__":

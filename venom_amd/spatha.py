@@ -12,6 +12,9 @@ from . import _lib
 
 OUT_ROW_MAJOR = 0
 OUT_TRANSPOSED = 1
+ACT_NONE, ACT_GELU, ACT_GELU_TANH = 0, 1, 2
+_ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "gelu": ACT_GELU, "gelu_tanh": ACT_GELU_TANH, "gelu_new": ACT_GELU_TANH,
+                "gelu_pytorch_tanh": ACT_GELU_TANH}
 
 
 def num_variants():
@@ -60,7 +63,10 @@ class SpmmPlan:
         name = _lib.lib().spatha_spmm_kernel_name(self._handle, N, out_layout, variant)
         return None if name is None else name.decode()
 
-    def run(self, B, bias=None, transposed_out=False, variant=0, out=None):
+    def run(self, B, bias=None, transposed_out=False, variant=0, out=None, activation=None):
+        """C = A B (or its transpose), fp16.  Without `activation`, a bias needs the transposed layout (the
+        reference operator's contract).  With `activation` given ("none", "gelu", "gelu_tanh") the call goes through
+        the fused entry point: out = act(fp16(A B) + bias) in either layout."""
         _check_dev(B, torch.float16, "rhs")
         if B.dim() != 2 or B.shape[0] != self.cols:
             raise ValueError("rhs must be [%d, N], got %s" % (self.cols, tuple(B.shape)))
@@ -76,11 +82,19 @@ class SpmmPlan:
             _check_dev(out, torch.float16, "out")
             if tuple(out.shape) != shape:
                 raise ValueError("out must be %s" % (shape,))
+        layout = OUT_TRANSPOSED if transposed_out else OUT_ROW_MAJOR
         with torch.cuda.device(self.device):
-            _lib.check(_lib.lib().spatha_spmm_run(self._handle, B.data_ptr(), N,
-                                                  None if bias is None else bias.data_ptr(), out.data_ptr(),
-                                                  OUT_TRANSPOSED if transposed_out else OUT_ROW_MAJOR, variant,
-                                                  _stream_ptr(self.device)), "spatha_spmm_run")
+            if activation is None:
+                _lib.check(_lib.lib().spatha_spmm_run(self._handle, B.data_ptr(), N,
+                                                      None if bias is None else bias.data_ptr(), out.data_ptr(), layout,
+                                                      variant, _stream_ptr(self.device)), "spatha_spmm_run")
+            else:
+                if activation not in _ACTIVATIONS:
+                    raise ValueError("unknown activation %r" % (activation,))
+                _lib.check(_lib.lib().spatha_spmm_run_fused(self._handle, B.data_ptr(), N,
+                                                            None if bias is None else bias.data_ptr(), out.data_ptr(),
+                                                            layout, _ACTIVATIONS[activation], variant,
+                                                            _stream_ptr(self.device)), "spatha_spmm_run_fused")
         return out
 
     def time(self, B, out, bias=None, transposed_out=False, variant=0, warmup=10, iters=100):
@@ -148,3 +162,11 @@ def spmm(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_co
         raise ValueError("B_num_cols does not match rhs_matrix")
     plan = _plan_for(A_values.detach(), A_metadata, A_indices, A_num_rows, A_num_cols, n, m, vec_length)
     return plan.run(rhs_matrix, bias=bias, transposed_out=True)
+
+
+def spmm_fused(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_cols, vec_length, n, m,
+               activation="none", transposed_out=False):
+    """act((A_vnm @ rhs_matrix) + bias), fp16, as [A_num_rows, tokens] (default: ready to be the rhs of the next
+    spmm without a transposed copy) or, with transposed_out, as [tokens, A_num_rows] like `spmm`."""
+    plan = _plan_for(A_values.detach(), A_metadata, A_indices, A_num_rows, A_num_cols, n, m, vec_length)
+    return plan.run(rhs_matrix, bias=bias, transposed_out=transposed_out, activation=activation)

@@ -223,7 +223,7 @@ def main(argv=None):
     timeit.repeat(lambda: run(sparse_model), repeat=5, number=1)
     t_sparse = report_time("n:m", timeit.repeat(lambda: run(sparse_model), repeat=args.repeats, number=1), 1, args.n, args.m, args.v)
     print("# dense %.2f ms, %d:%d:%d%s %.2f ms, speed-up %.2fx" % (t_dense, args.v, args.n, args.m,
-                                                                    " (fused feed-forward)" if args.fuse_ffn else "", t_sparse,
+                                                                    (" (fused feed-forward%s)" % (", activation in the kernel" if args.kernel_gelu else "")) if args.fuse_ffn else "", t_sparse,
                                                                     t_dense / t_sparse))
 
 

@@ -38,8 +38,7 @@ inline int hip_fail(hipError_t e) {
 // kernels whose write-out can apply bias and activation ahead of either output layout
 bool variant_has_fused_writeout(int variant) {
     using namespace spatha;
-    return (variant >= SPMM_VARIANT_P128x128_S4 && variant <= SPMM_VARIANT_P64x256_S4) ||
-           (variant >= SPMM_VARIANT_W128x128_S5 && variant <= SPMM_VARIANT_W64x256_S3) ||
+    return (variant >= SPMM_VARIANT_P128x128_S4 && variant <= SPMM_VARIANT_W64x256_S3) ||      // pipelined, persistent, wave-specialised
            (variant >= SPMM_VARIANT_T128x256_S3 && variant <= SPMM_VARIANT_DS256x128_S3_C8);
 }
 

@@ -1153,12 +1153,14 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_persist_kernel(SpmmParams p)
         }
         // ------------------------------------------------ tile finished: write it out
         const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+        if (p.fuse) fused_bias_act(acc, p.bias, (int64_t)cm0 + wm * 64 + ib * 16, p.act);
+        const uint16_t* bias = p.fuse ? nullptr : p.bias;
         if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
             const int64_t row0 = (int64_t)cm0 + wm * 64 + ib * 16;
             half8_t bias_lo, bias_hi;
-            if (p.bias) {
-                bias_lo = *(const half8_t*)(p.bias + row0);
-                bias_hi = *(const half8_t*)(p.bias + row0 + 8);
+            if (bias) {
+                bias_lo = *(const half8_t*)(bias + row0);
+                bias_hi = *(const half8_t*)(bias + row0 + 8);
             }
 #pragma unroll
             for (int nb = 0; nb < 4; nb++) {
@@ -1171,7 +1173,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_persist_kernel(SpmmParams p)
                         lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
                         hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
                     }
-                if (p.bias) {
+                if (bias) {
                     lo = lo + bias_lo;
                     hi = hi + bias_hi;
                 }

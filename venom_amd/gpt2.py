@@ -90,7 +90,8 @@ def main(argv=None):
     t_dense = report_time("dense", timeit.repeat(lambda: run(dense_model), repeat=args.repeats, number=1), args.n, args.m, args.v)
     timeit.repeat(lambda: run(sparse_model), repeat=5, number=1)
     t_sparse = report_time("n:m", timeit.repeat(lambda: run(sparse_model), repeat=args.repeats, number=1), args.n, args.m, args.v)
-    print("# dense %.2f ms, %d:%d:%d %.2f ms, speed-up %.2fx" % (t_dense, args.v, args.n, args.m, t_sparse, t_dense / t_sparse))
+    how = (" (fused feed-forward%s)" % (", activation in the kernel" if args.kernel_gelu else "")) if args.fuse_ffn else ""
+    print("# dense %.2f ms, %d:%d:%d%s %.2f ms, speed-up %.2fx" % (t_dense, args.v, args.n, args.m, how, t_sparse, t_dense / t_sparse))
 
 
 if __name__ == "__main__":

@@ -73,7 +73,7 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = f
 // Kernel choice.  V a multiple of 128: producer/consumer kernel on 128-row tiles; 256 columns wide
 // with 128 x 64 consumer waves when that still gives every CU at least two tiles, else 128 wide.  Otherwise (V a
 // multiple of 64 only) the 64 x 256 tile whose B rows are gathered per 64-row block.
-int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = false) {
+int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = false, int out_layout = SPATHA_OUT_ROW_MAJOR) {
     using namespace spatha;
     if (variant != SPMM_VARIANT_AUTO) return variant_ok(plan, N, variant, fused) ? variant : -1;
     const int v = plan->geo.v;
@@ -102,6 +102,24 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
             order[1] = order[0];
             order[0] = SPMM_VARIANT_W128x128_S2;
         }
+        if (out_layout == SPATHA_OUT_TRANSPOSED) {
+            // measured with transposed output + bias on the BERT-large layer shapes (N = 16384): the kernels that write
+            // through the 8-column slab (dense-staged, tall) lead by 10-25 % once there is enough work per tile column
+            if (plan->geo.m <= 8) {
+                // short k-loops only: with many k-steps per tile the gathered 128 x 256 tile moves fewer bytes per
+                // output element (GPT-3 block at 128:2:8: 6.95 ms against 8.26 ms with dense staging)
+                if (plan->S <= 16) {
+                    order[1] = order[0];
+                    order[0] = SPMM_VARIANT_DS256x128_S3_C8;
+                }
+            } else if (wide_tiles >= 1024 || plan->S >= 8) {
+                order[0] = SPMM_VARIANT_T128x256_S3;
+                order[1] = SPMM_VARIANT_W128x128_S3;
+            } else {
+                order[0] = SPMM_VARIANT_W128x128_S3;
+                order[1] = SPMM_VARIANT_T128x256_S3;
+            }
+        }
         order[2] = SPMM_VARIANT_P128x128_S3;
         order[3] = SPMM_VARIANT_128x128;
     } else if (v % 64 == 0) {
@@ -110,7 +128,8 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         // m > 8: gathered 64 x 256 tiles; with many k-steps per tile the persistent pipeline (which keeps loading
         // across tile boundaries) is 1.6x faster than the per-tile one, with few it is a few percent slower
         const bool long_k = plan->S >= 24;
-        order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : (plan->geo.m >= 32 ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_P64x256_S2);
+        const bool ws_short = plan->geo.m >= 32 && out_layout != SPATHA_OUT_TRANSPOSED;   // transposed: the pipeline leads by 6-8 %
+        order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : (ws_short ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_P64x256_S2);
         order[2] = long_k ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_R64x256_S3;
         order[3] = SPMM_VARIANT_64x256;
     } else {
@@ -271,9 +290,11 @@ static int run_spmm(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
         return SPATHA_ERR_BAD_ARGUMENT;
     if (N % 8 != 0) return SPATHA_ERR_BAD_SHAPE;      // 16-byte row segments of B and C
     if (((uintptr_t)B_dev & 15) || ((uintptr_t)out_dev & 15) || ((uintptr_t)bias_dev & 15)) return SPATHA_ERR_BAD_ARGUMENT;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev != plan->device) return SPATHA_ERR_BAD_ARGUMENT;   // plans live on one device
     // the bias of the transposed layout alone stays in the write-out itself
     const bool fuse = activation != SPATHA_ACT_NONE || (out_layout == SPATHA_OUT_ROW_MAJOR && bias_dev);
-    int var = pick_variant(plan, N, variant, fuse);
+    int var = pick_variant(plan, N, variant, fuse, out_layout);
     if (var < 0) return SPATHA_ERR_UNSUPPORTED;
     spatha::SpmmParams p;
     p.apack = plan->apack; p.rowtab = plan->rowtab;
@@ -311,9 +332,8 @@ int spatha_spmm_run_fused(const spatha_spmm_plan* plan, const uint16_t* B_dev, i
 int spatha_spmm_num_variants(void) { return spatha::SPMM_VARIANT_COUNT; }
 
 const char* spatha_spmm_kernel_name(const spatha_spmm_plan* plan, int N, int out_layout, int variant) {
-    (void)out_layout;
     if (!plan) return nullptr;
-    int var = pick_variant(plan, N, variant);
+    int var = pick_variant(plan, N, variant, false, out_layout);
     return var < 0 ? nullptr : spatha::spmm_variant_name(var);
 }
 

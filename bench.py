@@ -49,7 +49,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extra", action="store_true", help="also time the other BASELINE shapes (reported under 'extra')")
     ap.add_argument("--ablation", action="store_true",
-                    help="also time the same matrix with identity column-loc (the reference's IDEAL_KERNEL ablation)")
+                    help="also time the same matrix with identity column-loc (the reference's IDEAL_KERNEL ablation) and, "
+                         "if `python -m venom_amd.build --ablation` has been run, the OUT_32B build (4-byte stores of C)")
     ap.add_argument("--gpt3", action="store_true",
                     help="also time the GPT-3 FFN shapes (A 49152x12288 128:2:16, N in 16/256/2048; under 'gpt3')")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -60,6 +61,19 @@ def main():
         print("bench.py: this build measures one GPU only (the SpMM path has no multi-GPU part); run with --gpus 1",
               file=sys.stderr)
         sys.exit(2)
+
+    out32 = None
+    if args.ablation and not os.environ.get("SPATHA_LIBRARY"):
+        # the OUT_32B build of the library (python -m venom_amd.build --ablation), timed in a child process of its own
+        # BEFORE this process touches the GPU
+        alt = os.path.join(ROOT, "venom_amd", "lib", "libspatha_out32b.so")
+        if os.path.exists(alt):
+            import subprocess
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu-baseline", "--steps", str(args.steps),
+                                "--warmup", str(args.warmup), "--variant", str(args.variant)],
+                               env=dict(os.environ, SPATHA_LIBRARY=alt), stdout=subprocess.PIPE, text=True)
+            if r.returncode == 0 and r.stdout.strip():
+                out32 = json.loads(r.stdout.strip().splitlines()[-1])["roofline"]["kernel_us"]
 
     import numpy as np
     import torch
@@ -170,7 +184,8 @@ def main():
                                        torch.from_numpy(ident.view(np.int32)).to(dev), rows, cols, 2, m, v)
         _, k_id = timed(w_id, args.steps, args.warmup, args.variant)
         _, k_nm = timed(w, args.steps, 50, args.variant)
-        out["ablation"] = {"column_loc_us": round(k_nm * 1e3, 2), "ideal_identity_column_loc_us": round(k_id * 1e3, 2)}
+        out["ablation"] = {"column_loc_us": round(k_nm * 1e3, 2), "ideal_identity_column_loc_us": round(k_id * 1e3, 2),
+                           "out_32b_stores_us": out32}      # null: libspatha_out32b.so has not been built
 
     if args.gpt3:
         r2, c2, m2, v2 = 49152, 12288, 16, 128

@@ -143,3 +143,17 @@ def test_path_to_dset_writes_then_reads_the_matrix(gpu, tmp_path):
     # a container of another shape is refused
     third = _run(_replace(args, "--k", 1024))
     assert third.returncode == 1 and "--path_to_dset" in third.stderr
+
+
+@pytest.mark.gpu
+def test_out_32b_ablation_build_computes_the_same_numbers(gpu):
+    """The OUT_32B build (4-byte stores of C) only changes how the result leaves the GPU."""
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    alt = os.path.join(root, "venom_amd", "lib", "libspatha_out32b.so")
+    if not os.path.exists(alt):
+        pytest.skip("libspatha_out32b.so has not been built (python -m venom_amd.build --ablation)")
+    r = subprocess.run([sys.executable, "-c", "import __graft_entry__ as g; g.smoke()"], cwd=root,
+                       env=dict(os.environ, SPATHA_LIBRARY=alt), stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                       timeout=300)
+    assert r.returncode == 0 and "smoke ok" in r.stdout, r.stderr[-2000:]

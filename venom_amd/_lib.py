@@ -8,7 +8,8 @@ import os
 from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libspatha.so")
+# SPATHA_LIBRARY names another build of the same library (e.g. the OUT_32B ablation build)
+LIB_PATH = os.environ.get("SPATHA_LIBRARY") or os.path.join(_HERE, "lib", "libspatha.so")
 
 
 class SpathaError(RuntimeError):

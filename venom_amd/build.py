@@ -2,6 +2,7 @@
 benchmark_spmm driver.
 
     python -m venom_amd.build          # compile everything for gfx950
+    python -m venom_amd.build --ablation   # ... and the OUT_32B ablation variant of the library
 
 Host-only sources go through g++ (OpenMP via libgomp), HIP sources through
 hipcc --offload-arch=gfx950; hipcc links.  Everything is built in-tree.
@@ -54,6 +55,20 @@ def build(verbose=False, with_driver=True):
     return LIB
 
 
+def build_out_32b(verbose=False):
+    """The OUT_32B ablation build (the reference's compile-time switch of that name, CMakeLists.txt:25-33): the same
+    library with every 16-byte row-major store of C issued as four 4-byte stores -> venom_amd/lib/libspatha_out32b.so.
+    Needs the objects of a normal build; `SPATHA_LIBRARY=<that file>` makes the Python binding load it."""
+    lib = os.path.join(LIBDIR, "libspatha_out32b.so")
+    obj = os.path.join(OBJDIR, "spmm_kernels.out32b.o")
+    _run([HIPCC] + HIP_FLAGS + ["-DSPATHA_OUT_32B", "-x", "hip", "-c", os.path.join(CSRC, "spmm_kernels.hip"), "-o", obj], verbose)
+    objs = [os.path.join(OBJDIR, s + ".o") for s in CXX_SOURCES + HIP_SOURCES if s != "spmm_kernels.hip"] + [obj]
+    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", lib] + objs + ["-lgomp"], verbose)
+    return lib
+
+
 if __name__ == "__main__":
     build(verbose=True)
+    if "--ablation" in sys.argv[1:]:
+        build_out_32b(verbose=True)
     sys.exit(0)

@@ -52,6 +52,22 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 
+// Row-major stores of C: 16 bytes per lane.  Built with -DSPATHA_OUT_32B (the counterpart of the reference's OUT_32B
+// ablation switch, CMakeLists.txt:25-33) the same bytes leave as four 4-byte stores, to measure what the wide
+// stores are worth; assembly, so that the compiler cannot merge them again.
+__device__ __forceinline__ void store_c16(uint16_t* dst, u32x4 v) {
+#ifdef SPATHA_OUT_32B
+    asm volatile(
+        "global_store_dword %0, %1, off\n\t"
+        "global_store_dword %0, %2, off offset:4\n\t"
+        "global_store_dword %0, %3, off offset:8\n\t"
+        "global_store_dword %0, %4, off offset:12" ::"v"(dst), "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w)
+        : "memory");
+#else
+    *(u32x4*)dst = v;
+#endif
+}
+
 // "Dynamic LDS limit raised" flags, one per (kernel, device): the attribute is a per-device property of a kernel.
 static bool& lds_attr_flag(const void* kern) {
     struct Entry { const void* kern; bool set[16]; };
@@ -318,7 +334,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_kernel(SpmmParams p) {
             const int row = 16 * (L & 3) + (L >> 2);
             const int col = n0 + wn * 64 + ch * 8;
             u32x4 v = *(const u32x4*)(st + L * PITCH_C + ch * 16);
-            if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)m0 + wm * 64 + row) * N + col) = v;
+            if (col < N && !(p.debug & 2)) store_c16(p.C + ((int64_t)m0 + wm * 64 + row) * N + col, v);
         }
     }
 }
@@ -648,7 +664,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_pipe_kernel(SpmmParams p) {
             const int row = 16 * (Lr & 3) + (Lr >> 2);
             const int col = n0 + wn * 64 + ch * 8;
             u32x4 v = *(const u32x4*)(stg + Lr * PITCH_C + ch * 16);
-            if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)m0 + wm * 64 + row) * N + col) = v;
+            if (col < N && !(p.debug & 2)) store_c16(p.C + ((int64_t)m0 + wm * 64 + row) * N + col, v);
         }
     }
 }
@@ -879,7 +895,7 @@ __global__ __launch_bounds__(WN * 64) void spmm_half_kernel(SpmmParams p) {
             const int row = 32 * (Lr >> 5) + 8 * (Lr & 3) + 4 * ((Lr >> 4) & 1) + ((Lr >> 2) & 3);
             const int col = n0 + wn * 64 + ch * 8;
             u32x4 v = *(const u32x4*)(stg + Lr * PITCH_C + ch * 16);
-            if (col < N) *(u32x4*)(p.C + ((int64_t)m0 + row) * N + col) = v;
+            if (col < N) store_c16(p.C + ((int64_t)m0 + row) * N + col, v);
         }
     }
 }
@@ -1200,7 +1216,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_persist_kernel(SpmmParams p)
                     const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
                     const int col = cn0 + wn * 64 + ch * 8;
                     u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
-                    if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col) = v;
+                    if (col < N && !(p.debug & 2)) store_c16(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col, v);
                 }
                 __builtin_amdgcn_wave_barrier();
             }
@@ -1505,7 +1521,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk&
                     const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
                     const int col = cn0 + wn * 64 + ch * 8;
                     u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
-                    if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col) = v;
+                    if (col < N && !(p.debug & 2)) store_c16(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col, v);
                 }
                 __builtin_amdgcn_wave_barrier();
             }
@@ -1544,7 +1560,7 @@ __device__ __forceinline__ void store_slab_row_major(const uint32_t (&pend)[4][4
         const int row = 16 * (Lr & 3) + 4 * MB + (Lr >> 2);
         const int col = col_base + ch * 8;
         u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
-        if (col < N && enable) *(u32x4*)(C + (row_base + row) * N + col) = v;
+        if (col < N && enable) store_c16(C + (row_base + row) * N + col, v);
     }
     __builtin_amdgcn_wave_barrier();
 }
@@ -1788,7 +1804,7 @@ __device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const Tile
                         const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
                         const int col = cn0 + wn * 64 + ch * 8;
                         u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
-                        if (col < N && !(p.debug & 2)) *(u32x4*)(p.C + ((int64_t)cm0 + h * 64 + row) * N + col) = v;
+                        if (col < N && !(p.debug & 2)) store_c16(p.C + ((int64_t)cm0 + h * 64 + row) * N + col, v);
                     }
                     __builtin_amdgcn_wave_barrier();
                 }
@@ -1933,7 +1949,7 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
         short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff));
         short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff + 4 * PITCH));
         __builtin_amdgcn_wave_barrier();
-        if (ph > 0 && live) *(u32x4*)(C + (row0 + held_row) * N + out_col) = held;
+        if (ph > 0 && live) store_c16(C + (row0 + held_row) * N + out_col, held);
         held.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
         held.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
         held.z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
@@ -1941,7 +1957,7 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
         const int q = 8 * sidx + q_lo;
         held_row = 16 * (q >> 2) + 4 * mb + (q & 3);
     }
-    if (live) *(u32x4*)(C + (row0 + held_row) * N + out_col) = held;
+    if (live) store_c16(C + (row0 + held_row) * N + out_col, held);
     __builtin_amdgcn_wave_barrier();
 }
 

@@ -83,6 +83,10 @@ HALF_TILE_CASES = [
     (256, 1024, 520, 16, 32),     # 16 k-steps, three 256-wide tiles
     (320, 330, 40, 20, 160),      # V = 160, m not a power of two
     (128, 1280, 16, 32, 32),      # few columns: the skinny kernel does not take this operand order
+    (256, 512, 264, 8, 32),       # 256-row tiles, m <= 8: dense-staged B with two gather-table entries per wave
+    (512, 200, 136, 8, 32),       # ... K tail, padded last k-step
+    (768, 330, 72, 5, 96),        # ... V = 96, m = 5
+    (256, 64, 8, 4, 32),          # ... plain 2:4, one column tile
 ]
 
 
@@ -109,7 +113,9 @@ def test_half_tile_kernels_bit_exact(gpu, rows, cols, N, m, v, transposed):
                        variant=variant)
         torch.cuda.synchronize()
         assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16)), (variant,)
-    assert ran == 4                          # automatic choice + three tile shapes
+    assert ran >= 4                          # automatic choice + three gathered tile shapes (+ dense-staged when it applies)
+    if m <= 8 and rows % 256 == 0:
+        assert ran == 5 and "densestage" in plan.kernel_name(N, 1 if transposed else 0, 0)
 
 
 def test_half_tile_gaussian_within_tolerance(gpu):

@@ -39,7 +39,8 @@ inline int hip_fail(hipError_t e) {
 bool variant_has_fused_writeout(int variant) {
     using namespace spatha;
     return (variant >= SPMM_VARIANT_P128x128_S4 && variant <= SPMM_VARIANT_W64x256_S3) ||      // pipelined, persistent, wave-specialised
-           (variant >= SPMM_VARIANT_T128x256_S3 && variant <= SPMM_VARIANT_DS256x128_S3_C8);
+           (variant >= SPMM_VARIANT_T128x256_S3 && variant <= SPMM_VARIANT_DS256x128_S3_C8) ||
+           variant == SPMM_VARIANT_DSH256x128_S3_C8;
 }
 
 bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = false) {
@@ -49,8 +50,13 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = f
     const int bm = spmm_variant_bm(variant);
     if (bm == 0) return false;
     const bool half_variant = variant == SPMM_VARIANT_H64x256_S2 || variant == SPMM_VARIANT_H64x128_S3 ||
-                              variant == SPMM_VARIANT_H64x128_S2;
+                              variant == SPMM_VARIANT_H64x128_S2 || variant == SPMM_VARIANT_DSH256x128_S3_C8;
     if (half_variant != (plan->half_tiles != 0)) return false;       // the packed operand order differs
+    if (variant == SPMM_VARIANT_DSH256x128_S3_C8) {
+        if (plan->geo.m > 8 || plan->geo.rows % 256 != 0 || !plan->gtab) return false;
+        const uint64_t bb = (uint64_t)plan->geo.cols * (uint64_t)N * 2u;       // 32-bit buffer offsets
+        return bb < 0xE0000000ull && plan->apack_bytes < 0xE0000000ull;
+    }
     if (half_variant) return plan->geo.cols <= 65535 && spmm_variant_lds(variant, plan->S) <= 160 * 1024;
     if (variant == SPMM_VARIANT_DS256x128_S3 || variant == SPMM_VARIANT_DS256x128_S2 ||
         variant == SPMM_VARIANT_DS256x128_S3_C8 || variant == SPMM_VARIANT_DS256x128_S3_PP ||
@@ -84,10 +90,12 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
     if (plan->half_tiles) {
         // measured (1024 x 4096 x 4096 and 4096 x 1024 x 16384, m = 8..32): the 256-wide tile is never behind the
         // 128-wide one with two stages by more than 7 %, and up to 2x ahead; three stages of 128 leave two waves per CU
-        order[0] = N > 128 ? SPMM_VARIANT_H64x256_S2 : SPMM_VARIANT_H64x128_S2;
-        order[1] = SPMM_VARIANT_H64x128_S2;
-        order[2] = SPMM_VARIANT_H64x128_S3;
-        for (int i = 0; i < 3; i++)
+        // m <= 8: the dense B stage is shared by eight 32-row blocks, the fill does not grow with the smaller V
+        order[0] = SPMM_VARIANT_DSH256x128_S3_C8;
+        order[1] = N > 128 ? SPMM_VARIANT_H64x256_S2 : SPMM_VARIANT_H64x128_S2;
+        order[2] = SPMM_VARIANT_H64x128_S2;
+        order[3] = SPMM_VARIANT_H64x128_S3;
+        for (int i = 0; i < 4; i++)
             if (variant_ok(plan, N, order[i], fused)) return order[i];
         return -1;
     }
@@ -250,13 +258,18 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     e = spatha::launch_pack(values_dev, metadata_dev, columns_dev, rows, cols, m, v, geo.ksp, plan->S, plan->half_tiles,
                             plan->apack, plan->rowtab, (hipStream_t)stream);
     if (e != hipSuccess) { spatha_spmm_plan_destroy(plan); return hip_fail(e); }
-    if (v % 64 == 0 && m <= 8 && rows % 256 == 0) {
-        const size_t g_bytes = (size_t)(rows / 64) * plan->S * 64 * 2;
+    if (m <= 8 && rows % 256 == 0) {
+        // gather table of the dense-staged kernels: one entry per 64-row block, or per 32-row block when V % 64 != 0
+        const int block_rows = plan->half_tiles ? 32 : 64;
+        const size_t g_bytes = (size_t)(rows / block_rows) * plan->S * 64 * 2;
         if ((e = hipMalloc((void**)&plan->gtab, g_bytes)) != hipSuccess ||
-            (e = spatha::launch_pack_gtab(columns_dev, rows, m, v, geo.ksp, plan->S, plan->gtab, (hipStream_t)stream)) != hipSuccess) {
+            (e = spatha::launch_pack_gtab(columns_dev, rows, m, v, geo.ksp, plan->S, block_rows, plan->gtab,
+                                          (hipStream_t)stream)) != hipSuccess) {
             spatha_spmm_plan_destroy(plan);
             return hip_fail(e);
         }
+    }
+    if (v % 64 == 0 && m <= 8 && rows % 256 == 0) {
         plan->gtab_tiles_bytes = (size_t)(rows / 256) * plan->S * 512;
         if ((e = hipMalloc((void**)&plan->gtab_tiles, plan->gtab_tiles_bytes)) != hipSuccess ||
             (e = spatha::launch_pack_gtab_tiles(columns_dev, rows, m, v, geo.ksp, plan->S, plan->gtab_tiles,

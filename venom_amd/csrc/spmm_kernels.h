@@ -68,7 +68,8 @@ enum {
     SPMM_VARIANT_H64x256_S2 = 33,       // V % 64 != 0: a 64-row tile spans two V blocks, two gathered B sets per stage
     SPMM_VARIANT_H64x128_S3 = 34,
     SPMM_VARIANT_H64x128_S2 = 35,
-    SPMM_VARIANT_COUNT = 36
+    SPMM_VARIANT_DSH256x128_S3_C8 = 36, // V % 64 != 0, m <= 8: dense-staged B, two gather-table entries per consumer wave
+    SPMM_VARIANT_COUNT = 37
 };
 
 const char* spmm_variant_name(int variant);
@@ -81,7 +82,7 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
                        int m, int v, int ksp, int S, int half_tiles, uint16_t* apack, uint32_t* rowtab, hipStream_t stream);
 
-hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, uint16_t* gtab,
+hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, int block_rows, uint16_t* gtab,
                             hipStream_t stream);
 
 hipError_t launch_pack_gtab_tiles(const uint32_t* columns, int rows, int m, int v, int ksp, int S, uint16_t* gtab,

@@ -2195,6 +2195,142 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
     SPATHA_PROF_FLUSH
 }
 
+// Accumulators in half-tile order (lane group a = lane / 16 holds, in register mb = 2h + b, tile rows 32h + 8a + 4b + r)
+// -> standard order (lane group g holds, in register mb', rows 16g + 4mb' + r), so that every write-out routine
+// applies: the value of (g, mb') sits in lane group 2(g % 2) + mb'/2, register 2(g / 2) + mb' % 2.  Two lane
+// permutes per value (one per candidate source register), the lane's own g picks.
+__device__ __forceinline__ void half_to_standard_order(float4_t (&acc)[4][4], int lane) {
+    const int g = lane >> 4, j = lane & 15;
+    // the permutation stays inside a column block nb: sixteen temporaries at a time
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        float out[4][4];
+#pragma unroll
+        for (int mbp = 0; mbp < 4; mbp++) {
+            const int addr = (((2 * (g & 1) + (mbp >> 1)) << 4) | j) << 2;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float s0 = acc[mbp & 1][nb][r], s1 = acc[2 + (mbp & 1)][nb][r];
+                const int v0 = __builtin_amdgcn_ds_bpermute(addr, __float_as_int(s0));
+                const int v1 = __builtin_amdgcn_ds_bpermute(addr, __float_as_int(s1));
+                out[mbp][r] = __int_as_float((g >> 1) ? v1 : v0);
+            }
+        }
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) acc[mb][nb] = (float4_t){out[mb][0], out[mb][1], out[mb][2], out[mb][3]};
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// Consumer of the dense-staged kernel for V = 32 (96, 160, ...): eight 64 x 64 waves as in ds_consumer, but a wave's
+// 64 rows span two V blocks.  The operands are packed in half-tile order (see spmm_half_kernel): instructions 0, 1
+// multiply a fragment gathered with the first half's table entry, instructions 2, 3 one gathered with the second's
+// (gtab then has one entry per 32-row block).  The dense B stage is the same, so the fill traffic does not grow with
+// the smaller V; only the consumers read twice as many fragments.
+template <class Cfg, int OUT_LAYOUT>
+__device__ __forceinline__ void ds_consumer_half(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+    static_assert(Cfg::NC == 8, "one 64-row block per consumer wave");
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
+    constexpr int B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    const int S = p.S, N = p.N;
+    const int rb0 = wave >> 1, wn = wave & 1;
+    float4_t acc[4][4];
+    const int li = lane & 15, kb = lane >> 4;
+    const uint32_t col_xor = (uint32_t)((wn * 8 + ((li & 3) >> 1)) << 4);
+    const uint32_t col_or = (uint32_t)(li & 1) * 8u;
+    const int a_off = B_BYTES + rb0 * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + rb0 * APACK_BLOCK + 4096 + lane * 4;
+    const int ib = lane >> 4;
+    const int lane_class = kb * 4 + (li >> 2);
+    auto gtab_ptr = [&](int tm, int half, int step) {
+        const int64_t vb = ((int64_t)tm * 4 + rb0) * 2 + half;          // 32-row block
+        return (const u32x2*)(p.gtab + ((vb * S + step) * 16 + lane_class) * 4);
+    };
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    int n_tm = c_tm, n_tn = c_tn;
+    uint32_t c_stage = 0;
+    u32x2 g_next[2];
+    uint32_t base[2][4];
+    auto set_base = [&](int h, u32x2 g) {
+        base[h][0] = ((g.x & 0xffffu) ^ col_xor) | col_or;
+        base[h][1] = ((g.x >> 16) ^ col_xor) | col_or;
+        base[h][2] = ((g.y & 0xffffu) ^ col_xor) | col_or;
+        base[h][3] = ((g.y >> 16) ^ col_xor) | col_or;
+    };
+    set_base(0, *gtab_ptr(c_tm, 0, 0));
+    set_base(1, *gtab_ptr(c_tm, 1, 0));
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            int ns = c_step + 1;
+            if (ns == S) {
+                ns = 0;
+                if (c_tile + 1 < walk.my_tiles) walk.next(n_tm, n_tn);
+            }
+            g_next[0] = *gtab_ptr(n_tm, 0, ns);
+            g_next[1] = *gtab_ptr(n_tm, 1, ns);
+            __syncthreads();
+            const char* st = smem + c_stage;
+            half8_t a_cur[4];
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) a_cur[mb] = *(const half8_t*)(st + a_off + mb * 1024);
+            const uint32_t i0 = *(const uint32_t*)(st + i_off);
+            const uint32_t i1 = *(const uint32_t*)(st + i_off + 256);
+            auto read_frag = [&](int h, int nb) {
+                half16_t bf;
+#pragma unroll
+                for (int fb = 0; fb < 4; fb++) {
+                    short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, st + (base[h][fb] ^ (uint32_t)(nb << 5))));
+                    half4_t h4 = __builtin_bit_cast(half4_t, t4);
+                    bf[fb * 4 + 0] = h4[0];
+                    bf[fb * 4 + 1] = h4[1];
+                    bf[fb * 4 + 2] = h4[2];
+                    bf[fb * 4 + 3] = h4[3];
+                }
+                return bf;
+            };
+            // three fragments in flight at most (the register budget of three waves per SIMD): the next block's first-half
+            // fragment is requested before the current first-half instructions, its second-half one before the second-half ones
+            half16_t lo = read_frag(0, 0), hi = read_frag(1, 0);
+#define SPATHA_HALF_STEP(NB)                                    \
+    {                                                           \
+        half16_t lo_n, hi_n;                                    \
+        __builtin_amdgcn_sched_barrier(0);                      \
+        if (NB < 3) lo_n = read_frag(0, NB + 1);                \
+        __builtin_amdgcn_sched_barrier(0);                      \
+        SPATHA_MMA2LO(NB, lo)                                   \
+        __builtin_amdgcn_sched_barrier(0);                      \
+        if (NB < 3) hi_n = read_frag(1, NB + 1);                \
+        __builtin_amdgcn_sched_barrier(0);                      \
+        SPATHA_MMA2HI(NB, hi)                                   \
+        if (NB < 3) { lo = lo_n; hi = hi_n; }                   \
+    }
+            SPATHA_HALF_STEP(0)
+            SPATHA_HALF_STEP(1)
+            SPATHA_HALF_STEP(2)
+            SPATHA_HALF_STEP(3)
+#undef SPATHA_HALF_STEP
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+            set_base(0, g_next[0]);
+            set_base(1, g_next[1]);
+        }
+        const int cm0 = c_tm * BM + rb0 * 64, cn0 = c_tn * BN;
+        half_to_standard_order(acc, lane);
+        const bool pre = p.fuse && (p.act != SPATHA_ACT_NONE || OUT_LAYOUT == SPATHA_OUT_TRANSPOSED);
+        if (pre) fused_bias_act(acc, p.bias, (int64_t)cm0 + ib * 16, p.act);
+        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
+            store_block_transposed_slab(acc, smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, p.fuse ? nullptr : p.bias,
+                                        (int64_t)cm0, cn0 + wn * 64, p.rows, N, lane, true);
+        else
+            store_block_row_major_tr<true>(acc, smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, (int64_t)cm0, cn0 + wn * 64, N,
+                                           lane, true, (p.fuse && !pre) ? p.bias : nullptr);
+        walk.next(c_tm, c_tn);
+    }
+}
+
 // Ping-pong consumer of the dense-staged kernel (eight 64 x 64 consumer waves, two per SIMD).
 // Waves 0-3 ("early") read a stage's operands right after its barrier and multiply as the
 // fragments arrive.  Waves 4-7 ("late") run one phase behind: after the barrier of step s they
@@ -2411,7 +2547,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void spmm_dspp_kernel(SpmmParams p) 
     }
 }
 
-template <int M, int NS, int NP, int NC, int OUT_LAYOUT>
+template <int M, int NS, int NP, int NC, int OUT_LAYOUT, bool HALF = false>
 __global__ __launch_bounds__((NC + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
     using Cfg = DsCfg<M, NS, NP, NC>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -2427,7 +2563,8 @@ __global__ __launch_bounds__((NC + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
         for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);
     }
     if (wave < NC) {
-        ds_consumer<Cfg, OUT_LAYOUT>(p, walk, smem, wave, lane);
+        if constexpr (HALF) ds_consumer_half<Cfg, OUT_LAYOUT>(p, walk, smem, wave, lane);
+        else ds_consumer<Cfg, OUT_LAYOUT>(p, walk, smem, wave, lane);
     } else {
         const int pr = wave - NC;
         if (pr == 0) ds_producer<Cfg, M, NP, 0>(p, walk, smem_base, lane);
@@ -2437,7 +2574,7 @@ __global__ __launch_bounds__((NC + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
     }
 }
 
-template <int M, int NS, int NP, int NC, int OUT_LAYOUT, bool PINGPONG = false>
+template <int M, int NS, int NP, int NC, int OUT_LAYOUT, bool PINGPONG = false, bool HALF = false>
 static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
     using Cfg = DsCfg<M, NS, NP, NC>;
     constexpr int lds = Cfg::LDS_BYTES;
@@ -2446,7 +2583,7 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
     static int cus = 0;
     void (*kern)(SpmmParams);
     if constexpr (PINGPONG) kern = spmm_dspp_kernel<M, NS, NP, OUT_LAYOUT>;
-    else kern = spmm_ds_kernel<M, NS, NP, NC, OUT_LAYOUT>;
+    else kern = spmm_ds_kernel<M, NS, NP, NC, OUT_LAYOUT, HALF>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -2999,14 +3136,14 @@ static hipError_t launch_skinny(const SpmmParams& p, hipStream_t stream) {
 // gather table of the dense-staged kernel: [64-row block][step][kb][c][fb] u16 = LDS byte offset of dense
 // row d = gamma*m + column-loc (gamma = 4*fb + kb): d*256 + (d % 8)*32 (the swizzle of that row)
 __global__ void pack_gtab_kernel(const uint32_t* __restrict__ columns, int rows, int m, int v, int ksp, int S,
-                                 uint16_t* __restrict__ gtab) {
+                                 int block_rows, uint16_t* __restrict__ gtab) {
     const int ngroups = ksp / 2;
-    const int64_t total = (int64_t)(rows / 64) * S * 64;
+    const int64_t total = (int64_t)(rows / block_rows) * S * 64;
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
         const int fb = (int)(t & 3), c = (int)((t >> 2) & 3), kb = (int)((t >> 4) & 3);
         const int64_t bs = t >> 6;
         const int s = (int)(bs % S);
-        const int64_t b = (bs / S) * 64 / v;
+        const int64_t b = (bs / S) * block_rows / v;          // V block of this 64-row (or, for V = 32, 32-row) block
         const int gamma = fb * 4 + kb;
         const int g = s * 16 + gamma;
         uint32_t d = (uint32_t)gamma * m;
@@ -3015,12 +3152,12 @@ __global__ void pack_gtab_kernel(const uint32_t* __restrict__ columns, int rows,
     }
 }
 
-hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, uint16_t* gtab,
+hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, int block_rows, uint16_t* gtab,
                             hipStream_t stream) {
-    int64_t total = (int64_t)(rows / 64) * S * 64;
+    int64_t total = (int64_t)(rows / block_rows) * S * 64;
     int blocks = (int)((total + 255) / 256);
     if (blocks > 65535 * 8) blocks = 65535 * 8;
-    hipLaunchKernelGGL(pack_gtab_kernel, dim3(blocks), dim3(256), 0, stream, columns, rows, m, v, ksp, S, gtab);
+    hipLaunchKernelGGL(pack_gtab_kernel, dim3(blocks), dim3(256), 0, stream, columns, rows, m, v, ksp, S, block_rows, gtab);
     return hipGetLastError();
 }
 
@@ -3141,6 +3278,7 @@ const char* spmm_variant_name(int variant) {
         case SPMM_VARIANT_H64x256_S2: return "smfmac16x16x64_halftile_ldsdirect_tile64x256_2stage";
         case SPMM_VARIANT_H64x128_S3: return "smfmac16x16x64_halftile_ldsdirect_tile64x128_3stage";
         case SPMM_VARIANT_H64x128_S2: return "smfmac16x16x64_halftile_ldsdirect_tile64x128_2stage";
+        case SPMM_VARIANT_DSH256x128_S3_C8: return "smfmac16x16x64_halftile_densestage_tile256x128_3stage_8consumers";
         default: return nullptr;
     }
 }
@@ -3181,6 +3319,7 @@ int spmm_variant_lds(int variant, int S) {
         case SPMM_VARIANT_H64x256_S2: return half_stage_bytes<4, 2>() + S * 256;
         case SPMM_VARIANT_H64x128_S3: return half_stage_bytes<2, 3>() + S * 256;
         case SPMM_VARIANT_H64x128_S2: return half_stage_bytes<2, 2>() + S * 256;
+        case SPMM_VARIANT_DSH256x128_S3_C8: return DsCfg<8, 3, 4, 8>::LDS_BYTES;
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_64x256: return 1;
         default: return 0;
     }
@@ -3196,7 +3335,7 @@ int spmm_variant_bm(int variant) {
         case SPMM_VARIANT_R64x256_S3: case SPMM_VARIANT_R64x256_S4: case SPMM_VARIANT_W64x256_S2: case SPMM_VARIANT_W64x256_S3: case SPMM_VARIANT_D64x256_S3:
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4:
         case SPMM_VARIANT_SKINNY: case SPMM_VARIANT_H64x256_S2: case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2: return 64;
-        case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3: return 256;
+        case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3: case SPMM_VARIANT_DSH256x128_S3_C8: return 256;
         default: return 0;
     }
 }
@@ -3207,7 +3346,7 @@ int spmm_variant_bn(int variant) {
         case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2:
         case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5:
         case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3:
-        case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2: return 128;
+        case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2: case SPMM_VARIANT_DSH256x128_S3_C8: return 128;
         case SPMM_VARIANT_SKINNY: return 64;
         case SPMM_VARIANT_H64x256_S2: return 256;
         case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D64x256_S3: case SPMM_VARIANT_T128x256_S3:
@@ -3294,6 +3433,9 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
     if (variant == SPMM_VARIANT_SKINNY)
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_skinny<SPATHA_OUT_TRANSPOSED>(p, stream)
                                                    : launch_skinny<SPATHA_OUT_ROW_MAJOR>(p, stream);
+    if (variant == SPMM_VARIANT_DSH256x128_S3_C8)
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ds<8, 3, 4, 8, SPATHA_OUT_TRANSPOSED, false, true>(p, stream)
+                                                   : launch_ds<8, 3, 4, 8, SPATHA_OUT_ROW_MAJOR, false, true>(p, stream);
     if (variant == SPMM_VARIANT_DSF256x128_S3)
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_dsf<8, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
                                                    : launch_dsf<8, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);

@@ -186,3 +186,22 @@ def test_fused_gpt2_mlp_tracks_the_unfused_block(gpu, in_kernel):
         assert (a.float() - b.float()).abs().max().item() <= 2e-2
     else:              # same operations on the same numbers in another layout
         assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
+def test_merged_qkv_projection_gives_the_same_bits(gpu):
+    from venom_amd.bert import build_bert_large, fuse_feed_forward, linear_to_spmm, merge_qkv
+
+    torch.set_grad_enabled(False)
+    plain = linear_to_spmm(build_bert_large(layers=2).to(gpu).half(), 2, 8, 64)
+    merged = merge_qkv(fuse_feed_forward(linear_to_spmm(build_bert_large(layers=2).to(gpu).half(), 2, 8, 64)))
+    for trial in range(2):          # a second input must not be served from the first one's result
+        ids = torch.randint(0, 30522, (2, 64), device=gpu)
+        assert torch.equal(plain(ids).last_hidden_state, merged(ids).last_hidden_state)
+    att = merged.encoder.layer[0].attention.self
+    x = torch.randn((2, 64, 1024), device=gpu).half()
+    q, k, v = att.query(x), att.key(x), att.value(x)
+    assert q.shape == (2, 64, 1024) and q.data_ptr() != k.data_ptr()
+    for got, layer in ((q, plain.encoder.layer[0].attention.self.query), (k, plain.encoder.layer[0].attention.self.key),
+                       (v, plain.encoder.layer[0].attention.self.value)):
+        assert torch.equal(got, layer(x))

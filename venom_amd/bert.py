@@ -85,7 +85,12 @@ class SrnmSpmm(torch.nn.Module):
         cls._last_rhs = (key, flat, rhs)
         return rhs
 
+    _group = None          # set by merge_qkv: the projections this layer is computed together with
+    _group_index = 0
+
     def forward(self, input):
+        if self._group is not None:
+            return self._group.output(self._group_index, self.nrows_sp, input)
         flat = torch.flatten(input, start_dim=0, end_dim=-2)          # [tokens, in]
         rhs = self._transposed(flat)                                  # [in, tokens], as the operator expects
         bias = self.bias if self.bias is not None else torch.zeros(self.nrows_sp, dtype=rhs.dtype, device=rhs.device)
@@ -101,6 +106,53 @@ class SrnmSpmm(torch.nn.Module):
         out = spatha.spmm_fused(self.metadata, self.columns, self.values, rhs, self.bias, self.nrows_sp, self.ncols_sp,
                                 self.v, self.n, self.m, activation=activation)              # [out, tokens]
         return out.T.reshape(*input.shape[:-1], -1)     # strides (.., 1, tokens): a view, nothing moves
+
+
+class _MergedProjections:
+    """Several SrnmSpmm layers that read the same activation (the query / key / value projections of an attention
+    block) as ONE SpMM over the row-wise concatenation of their V:N:M matrices: the format is blocked by rows
+    (values by 16, metadata by 32, column-loc by V), so the arrays simply concatenate.  The first member asked
+    computes all of them; the others take their slice of the result while the activation is unchanged."""
+
+    def __init__(self, layers):
+        first = layers[0]
+        assert all((l.ncols_sp, l.n, l.m, l.v) == (first.ncols_sp, first.n, first.m, first.v) for l in layers)
+        self.v, self.n, self.m, self.cols = first.v, first.n, first.m, first.ncols_sp
+        self.values = torch.cat([l.values.data for l in layers]).contiguous()
+        self.metadata = torch.cat([l.metadata for l in layers]).contiguous()
+        self.columns = torch.cat([l.columns for l in layers]).contiguous()
+        zeros = [torch.zeros(l.nrows_sp, dtype=first.values.dtype, device=first.values.device) for l in layers]
+        self.bias = torch.cat([l.bias.data if l.bias is not None else z for l, z in zip(layers, zeros)]).contiguous()
+        self.starts, self.rows = [], 0
+        for l in layers:
+            self.starts.append(self.rows)
+            self.rows += l.nrows_sp
+        self._last = (None, None, None)          # (key, activation held alive, [tokens, rows] result)
+
+    def output(self, index, nrows, input):
+        flat = torch.flatten(input, start_dim=0, end_dim=-2)
+        key = (flat.data_ptr(), tuple(flat.shape), tuple(flat.stride()), flat._version, flat.device)
+        if self._last[0] != key:
+            rhs = SrnmSpmm._transposed(flat)
+            out = spatha.spmm(self.metadata, self.columns, self.values, rhs, self.bias, self.rows, self.cols, rhs.shape[1],
+                              self.v, self.n, self.m, 0, 0, 32, 4)
+            self._last = (key, flat, out)
+        start = self.starts[index]
+        return self._last[2][:, start:start + nrows].reshape(*input.shape[:-1], nrows)
+
+
+def merge_qkv(model):
+    """One SpMM instead of three for the query / key / value projections of every BertSelfAttention whose projections
+    are SrnmSpmm layers (same numbers: every output row is computed exactly as before)."""
+    from transformers.models.bert.modeling_bert import BertSelfAttention
+
+    for mod in model.modules():
+        if isinstance(mod, BertSelfAttention) and all(isinstance(getattr(mod, k), SrnmSpmm) for k in ("query", "key", "value")):
+            layers = [mod.query, mod.key, mod.value]
+            group = _MergedProjections(layers)
+            for i, l in enumerate(layers):
+                l._group, l._group_index = group, i
+    return model
 
 
 class FusedFeedForwardIn(torch.nn.Module):
@@ -199,6 +251,7 @@ def main(argv=None):
     ap.add_argument("--fuse-ffn", action="store_true",
                     help="first feed-forward layer of every block as one kernel (bias + GELU in the write-out, feature-major "
                          "result handed to the second layer without a transposed copy)")
+    ap.add_argument("--merge-qkv", action="store_true", help="query, key and value projections of a block as one SpMM")
     ap.add_argument("--kernel-gelu", action="store_true",
                     help="with --fuse-ffn: GELU in the kernel's write-out too (default: torch's elementwise pass over the "
                          "feature-major buffer, which keeps the model's output bit-identical to the unfused layers)")
@@ -210,6 +263,8 @@ def main(argv=None):
     sparse_model = linear_to_spmm(sparse_model.to(dev).half(), args.n, args.m, args.v, args.magnitude)
     if args.fuse_ffn:
         fuse_feed_forward(sparse_model, activation_in_kernel=args.kernel_gelu)
+    if args.merge_qkv:
+        merge_qkv(sparse_model)
     ids = torch.randint(0, 30522, (args.batch, args.seq), device=dev)
 
     def run(model):
@@ -223,7 +278,8 @@ def main(argv=None):
     timeit.repeat(lambda: run(sparse_model), repeat=5, number=1)
     t_sparse = report_time("n:m", timeit.repeat(lambda: run(sparse_model), repeat=args.repeats, number=1), 1, args.n, args.m, args.v)
     print("# dense %.2f ms, %d:%d:%d%s %.2f ms, speed-up %.2fx" % (t_dense, args.v, args.n, args.m,
-                                                                    (" (fused feed-forward%s)" % (", activation in the kernel" if args.kernel_gelu else "")) if args.fuse_ffn else "", t_sparse,
+                                                                    ((" (fused feed-forward%s)" % (", activation in the kernel" if args.kernel_gelu else "")) if args.fuse_ffn else "")
+                                                                    + (" (merged q/k/v)" if args.merge_qkv else ""), t_sparse,
                                                                     t_dense / t_sparse))
 
 

@@ -17,6 +17,7 @@ def main(argv=None):
     ap.add_argument("--m", default="8,16,32")
     ap.add_argument("--fuse-ffn", action="store_true", help="passed on to the three harnesses")
     ap.add_argument("--kernel-gelu", action="store_true", help="passed on to the three harnesses")
+    ap.add_argument("--merge-qkv", action="store_true", help="passed on to the BERT harness (GPT-2's c_attn is one layer already)")
     args = ap.parse_args(argv)
     extra = (["--fuse-ffn"] if args.fuse_ffn else []) + (["--kernel-gelu"] if args.kernel_gelu else [])
     print("algo,n,m,v,mean,median,std,len", flush=True)
@@ -24,7 +25,8 @@ def main(argv=None):
     for v in [int(x) for x in args.v.split(",")]:
         for name in args.models.split(","):
             for m in [int(x) for x in args.m.split(",")]:
-                mains[name](["-m", str(m), "-n", "2", "-v", str(v), "--repeats", str(args.repeats)] + extra)
+                mains[name](["-m", str(m), "-n", "2", "-v", str(v), "--repeats", str(args.repeats)] + extra +
+                            (["--merge-qkv"] if args.merge_qkv and name == "bert" else []))
 
 
 if __name__ == "__main__":

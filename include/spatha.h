@@ -103,6 +103,13 @@ int spatha_vnm_decode_f16(const uint16_t* values, const uint32_t* metadata, cons
 int spatha_vnm_select_columns_f32(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
                                   int32_t* columns, int threads);
 
+/* The same selector with its search phase (all C(m,4) column subsets of every V x m block: 35 960 at m = 32) on the
+ * GPU; masks and column offsets are bit-identical to spatha_vnm_select_columns_f32.  All pointers are HOST memory;
+ * the call uploads |A|, runs the search on `stream`, waits for it and finishes on the host (it allocates and frees
+ * device scratch).  Same reference functions as above. */
+int spatha_vnm_select_columns_f32_gpu(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
+                                      int32_t* columns, int threads, void* stream);
+
 /* Layout of the single "metadata + column-loc" device blob the reference
  * uploads: metadata words first, column-loc words at the next multiple of 8
  * words.  Replaces BlockwiseSpMatrix<T>::transform_and_sync_device

@@ -8,6 +8,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <new>
+#include <vector>
 
 #include "../../include/spatha.h"
 #include "spmm_kernels.h"
@@ -216,6 +217,40 @@ int spatha_vnm_file_info(const char* path, spatha_vnm_geometry* geometry, int* v
 
 int spatha_vnm_file_read(const char* path, void* values, uint32_t* metadata, uint32_t* columns) {
     return spatha::file_read(path, values, metadata, columns);
+}
+
+int spatha_vnm_select_columns_f32_gpu(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
+                                      int32_t* columns, int threads, void* stream) {
+    spatha_vnm_geometry geo;
+    int st = spatha::geometry_init(rows, cols, n, m, v, &geo);
+    if (st) return st;
+    if (!dense_abs || !masks || !columns) return SPATHA_ERR_BAD_ARGUMENT;
+    int per_block = 0;
+    const int tasks = spatha::select_task_count(rows, cols, m, v, &per_block);
+    std::vector<spatha::GroupTask> winners((size_t)tasks);
+    if (tasks > 0) {
+        if ((size_t)v * (size_t)m * sizeof(float) > 150u * 1024u) return SPATHA_ERR_TOO_LARGE;   // one V x m block per workgroup in LDS
+        float* d_abs = nullptr;
+        spatha::SelectWinner* d_out = nullptr;
+        std::vector<spatha::SelectWinner> h_out((size_t)tasks);
+        const size_t bytes = (size_t)rows * (size_t)cols * sizeof(float);
+        hipStream_t s = (hipStream_t)stream;
+        hipError_t e = hipMalloc((void**)&d_abs, bytes);
+        if (e == hipSuccess) e = hipMalloc((void**)&d_out, (size_t)tasks * sizeof(spatha::SelectWinner));
+        if (e == hipSuccess) e = hipMemcpyAsync(d_abs, dense_abs, bytes, hipMemcpyHostToDevice, s);
+        if (e == hipSuccess) e = spatha::launch_select_winners(d_abs, rows, cols, m, v, d_out, s);
+        if (e == hipSuccess) e = hipMemcpyAsync(h_out.data(), d_out, (size_t)tasks * sizeof(spatha::SelectWinner), hipMemcpyDeviceToHost, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        if (d_abs) (void)hipFree(d_abs);
+        if (d_out) (void)hipFree(d_out);
+        if (e != hipSuccess) return hip_fail(e);
+        for (int i = 0; i < tasks; i++) {
+            winners[(size_t)i].any = h_out[(size_t)i].any != 0;
+            for (int k = 0; k < 4; k++) winners[(size_t)i].best[k] = h_out[(size_t)i].best[k];
+        }
+    }
+    return spatha::select_columns_with_winners(dense_abs, rows, cols, n, m, v, tasks > 0 ? winners.data() : nullptr, masks,
+                                               columns, threads);
 }
 
 int spatha_vnm_pack_meta_blob(const uint32_t* metadata, int64_t n_metadata, const uint32_t* columns,

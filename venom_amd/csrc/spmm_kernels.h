@@ -82,6 +82,15 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
                        int m, int v, int ksp, int S, int half_tiles, uint16_t* apack, uint32_t* rowtab, hipStream_t stream);
 
+// Search phase of the magnitude selector on the GPU (select_gpu.hip): one entry per (V-row block, group) task,
+// block-major, groups in the order full groups then the tail group (if it has three or more columns).
+struct SelectWinner {
+    int best[4];    // winning column subset, ascending; zeros when no subset has a positive total
+    int any;
+};
+hipError_t launch_select_winners(const float* dense_abs_dev, int rows, int cols, int m, int v, SelectWinner* out_dev,
+                                 hipStream_t stream);
+
 hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, int block_rows, uint16_t* gtab,
                             hipStream_t stream);
 

@@ -192,14 +192,6 @@ int decode(const T* values, const uint32_t* metadata, const uint32_t* columns, i
 // second/third place, the permutation's history is replayed sequentially so
 // that the mask matches bit for bit.
 // ---------------------------------------------------------------------------
-struct GroupTask {
-    int width;      // candidate columns in this group (m, or cols % m in the tail)
-    int take;       // subset size (4, or 3 in the tail of width 3)
-    int best[4];    // winning subset (ascending); all zero when every total is 0
-    bool any;       // a subset had total > 0
-    bool tie;       // the winner's mask depends on the permutation history
-};
-
 inline void top2_of(const float* v, int take, int& i1, int& i2) {
     // indices of the largest and second largest; the lower index wins ties
     i1 = 0;
@@ -248,7 +240,13 @@ void find_winner(const float* base, int ld, int v_rows, GroupTask& t) {
             for (int i = 0; i < take; i++) t.best[i] = pick[i];
         }
     });
+}
+
+// does the winner's mask depend on the permutation history (second and third largest equal in some row)?
+void check_tie(const float* base, int ld, int v_rows, GroupTask& t) {
+    t.tie = false;
     if (!t.any) return;
+    const int take = t.take;
     for (int r = 0; r < v_rows && !t.tie; r++) {
         const float* row = base + (int64_t)r * ld;
         float x[4];
@@ -277,8 +275,20 @@ int decode_f16(const uint16_t* values, const uint32_t* metadata, const uint32_t*
     return decode<uint16_t>(values, metadata, columns, rows, cols, n, m, v, dense, threads);
 }
 
+int select_task_count(int rows, int cols, int m, int v, int* per_block_out) {
+    const int blocks = rows / v, full = cols / m, rem = cols % m;
+    const int per_block = full + ((rem >= 3) ? 1 : 0);       // a tail of three or more columns goes through the search
+    if (per_block_out) *per_block_out = per_block;
+    return blocks * per_block;
+}
+
 int select_columns_f32(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
                        int32_t* columns, int threads) {
+    return select_columns_with_winners(dense_abs, rows, cols, n, m, v, nullptr, masks, columns, threads);
+}
+
+int select_columns_with_winners(const float* dense_abs, int rows, int cols, int n, int m, int v, const GroupTask* winners,
+                                int32_t* masks, int32_t* columns, int threads) {
     spatha_vnm_geometry g;
     int st = geometry_init(rows, cols, n, m, v, &g);
     if (st) return st;
@@ -290,14 +300,22 @@ int select_columns_f32(const float* dense_abs, int rows, int cols, int n, int m,
     std::vector<GroupTask> tasks((size_t)blocks * per_block);
     set_threads(threads);
 
-    // Phase 1: winners, independent per (block, group).
+    // Phase 1: winners, independent per (block, group): searched here, or taken from the caller (the GPU search).
 #pragma omp parallel for schedule(dynamic, 1) collapse(2)
     for (int b = 0; b < blocks; b++)
         for (int gi = 0; gi < per_block; gi++) {
             GroupTask& t = tasks[(size_t)b * per_block + gi];
             if (gi < full) { t.width = m; t.take = 4; }
             else { t.width = rem; t.take = (rem == 3) ? 3 : 4; }
-            find_winner(dense_abs + (int64_t)b * v * cols + (int64_t)gi * m, cols, v, t);
+            const float* base = dense_abs + (int64_t)b * v * cols + (int64_t)gi * m;
+            if (winners) {
+                const GroupTask& w = winners[(size_t)b * per_block + gi];
+                t.any = w.any;
+                for (int i = 0; i < 4; i++) t.best[i] = w.any ? w.best[i] : 0;
+            } else {
+                find_winner(base, cols, v, t);
+            }
+            check_tie(base, cols, v, t);
         }
 
     bool need_replay = false;

@@ -20,6 +20,19 @@ int decode_f32(const float* values, const uint32_t* metadata, const uint32_t* co
 int decode_f16(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols, int n,
                int m, int v, uint16_t* dense, int threads);
 
+// One (V-row block, m-column group) of the magnitude selector.
+struct GroupTask {
+    int width;      // candidate columns in this group (m, or cols % m in the tail)
+    int take;       // subset size (4, or 3 in the tail of width 3)
+    int best[4];    // winning subset (ascending); all zero when every total is 0
+    bool any;       // a subset had total > 0
+    bool tie;       // the winner's mask depends on the permutation history
+};
+// tasks of the search: (rows / v) blocks x per_block groups, block-major
+int select_task_count(int rows, int cols, int m, int v, int* per_block_out);
+// the selector with the winners of the search supplied by the caller (winners == nullptr: searched on the host)
+int select_columns_with_winners(const float* dense_abs, int rows, int cols, int n, int m, int v, const GroupTask* winners,
+                                int32_t* masks, int32_t* columns, int threads);
 int select_columns_f32(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
                        int32_t* columns, int threads);
 

@@ -104,11 +104,15 @@ int spatha_vnm_select_columns_f32(const float* dense_abs, int rows, int cols, in
                                   int32_t* columns, int threads);
 
 /* The same selector with its search phase (all C(m,4) column subsets of every V x m block: 35 960 at m = 32) on the
- * GPU; masks and column offsets are bit-identical to spatha_vnm_select_columns_f32.  All pointers are HOST memory;
- * the call uploads |A|, runs the search on `stream`, waits for it and finishes on the host (it allocates and frees
- * device scratch).  Same reference functions as above. */
+ * GPU.  All pointers are HOST memory; the call uploads |A|, runs the search on `stream`, waits for it and finishes on
+ * the host (it allocates and frees device scratch).  exact_ties != 0: masks and column offsets are bit-identical to
+ * spatha_vnm_select_columns_f32, i.e. to the reference; when a winning subset has two EQUAL magnitudes competing for a
+ * row's second slot, that costs a sequential replay of the reference's whole run (its choice among equals depends on
+ * every comparison made before).  exact_ties == 0: the lower column index wins such a tie (same magnitudes kept, no
+ * replay) - the setting for converting fp16 models, where equal magnitudes are common.  Same reference functions as
+ * above. */
 int spatha_vnm_select_columns_f32_gpu(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
-                                      int32_t* columns, int threads, void* stream);
+                                      int32_t* columns, int threads, int exact_ties, void* stream);
 
 /* Layout of the single "metadata + column-loc" device blob the reference
  * uploads: metadata words first, column-loc words at the next multiple of 8

@@ -61,3 +61,32 @@ def test_gpu_search_on_a_bert_large_ffn_weight(gpu):
     assert gm.sum().item() == 4096 * (1024 // 32) * 2
     print("GPU-assisted selector, 4096 x 1024 at 64:2:32: %.2f s" % t_gpu)
     assert t_gpu < 5.0
+
+
+def test_without_tie_replay_equal_magnitudes_go_to_the_lower_column(gpu):
+    """exact_ties=False: same column offsets, and per row the two largest of the four chosen columns with the lower
+    column winning among equals; identical to the exact result wherever no tie decides."""
+    rng = np.random.default_rng(3)
+    rows, cols, m, v = 128, 128, 8, 64
+    d = rng.integers(0, 4, size=(rows, cols)).astype(np.float32)          # plenty of equal magnitudes
+    exact_masks, exact_cols = F.select_columns(d, 2, m, v, gpu=True)
+    masks, columns = F.select_columns(d, 2, m, v, gpu=True, exact_ties=False)
+    assert np.array_equal(columns, exact_cols)
+    ngroups = cols // m
+    chosen = columns.reshape(rows // v, -1, 4)[:, :ngroups]
+    for r in range(rows):
+        for g in range(ngroups):
+            c = chosen[r // v, g]
+            x = d[r, g * m + c]
+            order = sorted(range(4), key=lambda i: (-x[i], i))[:2]        # largest first, lower index among equals
+            want = np.zeros(m, np.int32)
+            if d[(r // v) * v:(r // v + 1) * v, g * m:(g + 1) * m].any():
+                want[c[order]] = 1
+            assert np.array_equal(masks[r, g * m:(g + 1) * m], want), (r, g)
+            kept, kept_exact = np.sort(d[r, g * m:(g + 1) * m][masks[r, g * m:(g + 1) * m] == 1]), \
+                np.sort(d[r, g * m:(g + 1) * m][exact_masks[r, g * m:(g + 1) * m] == 1])
+            assert np.array_equal(kept, kept_exact)                          # the same magnitudes either way
+    g2 = np.abs(rng.standard_normal((rows, cols))).astype(np.float32)     # no ties: the two settings agree exactly
+    a = F.select_columns(g2, 2, m, v, gpu=True)
+    b = F.select_columns(g2, 2, m, v, gpu=True, exact_ties=False)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])

@@ -40,7 +40,7 @@ SIGNATURES = {
     "spatha_vnm_decode_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int]),
     "spatha_vnm_decode_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int]),
     "spatha_vnm_select_columns_f32": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int]),
-    "spatha_vnm_select_columns_f32_gpu": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
+    "spatha_vnm_select_columns_f32_gpu": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "spatha_vnm_pack_meta_blob": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, POINTER(c_int64), POINTER(c_int64)]),
     "spatha_spmm_plan_create": (c_int, [c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_void_p)]),
     "spatha_spmm_plan_destroy": (c_int, [c_void_p]),

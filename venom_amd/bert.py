@@ -42,7 +42,8 @@ class NMVectorSparsifier:
     def __call__(self, tensor, grad_fmt=None):
         nrows, ncols = tensor.shape
         if self.magnitude:
-            mask, columns = nm_vector_mask_sparsify(tensor, self.n, self.m, self.tileM)
+            # model conversion: equal magnitudes (frequent in fp16 weights) go to the lower column, no history replay
+            mask, columns = nm_vector_mask_sparsify(tensor, self.n, self.m, self.tileM, exact_ties=not tensor.is_cuda)
         else:
             columns = torch.arange(4, dtype=torch.int32).repeat(nrows // self.tileM, ncols // self.m)
             pat = torch.zeros(self.m, dtype=torch.int32)

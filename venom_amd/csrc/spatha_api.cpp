@@ -220,7 +220,7 @@ int spatha_vnm_file_read(const char* path, void* values, uint32_t* metadata, uin
 }
 
 int spatha_vnm_select_columns_f32_gpu(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
-                                      int32_t* columns, int threads, void* stream) {
+                                      int32_t* columns, int threads, int exact_ties, void* stream) {
     spatha_vnm_geometry geo;
     int st = spatha::geometry_init(rows, cols, n, m, v, &geo);
     if (st) return st;
@@ -249,8 +249,8 @@ int spatha_vnm_select_columns_f32_gpu(const float* dense_abs, int rows, int cols
             for (int k = 0; k < 4; k++) winners[(size_t)i].best[k] = h_out[(size_t)i].best[k];
         }
     }
-    return spatha::select_columns_with_winners(dense_abs, rows, cols, n, m, v, tasks > 0 ? winners.data() : nullptr, masks,
-                                               columns, threads);
+    return spatha::select_columns_with_winners(dense_abs, rows, cols, n, m, v, tasks > 0 ? winners.data() : nullptr,
+                                               exact_ties != 0, masks, columns, threads);
 }
 
 int spatha_vnm_pack_meta_blob(const uint32_t* metadata, int64_t n_metadata, const uint32_t* columns,

@@ -284,11 +284,11 @@ int select_task_count(int rows, int cols, int m, int v, int* per_block_out) {
 
 int select_columns_f32(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
                        int32_t* columns, int threads) {
-    return select_columns_with_winners(dense_abs, rows, cols, n, m, v, nullptr, masks, columns, threads);
+    return select_columns_with_winners(dense_abs, rows, cols, n, m, v, nullptr, true, masks, columns, threads);
 }
 
 int select_columns_with_winners(const float* dense_abs, int rows, int cols, int n, int m, int v, const GroupTask* winners,
-                                int32_t* masks, int32_t* columns, int threads) {
+                                bool replay_ties, int32_t* masks, int32_t* columns, int threads) {
     spatha_vnm_geometry g;
     int st = geometry_init(rows, cols, n, m, v, &g);
     if (st) return st;
@@ -318,8 +318,12 @@ int select_columns_with_winners(const float* dense_abs, int rows, int cols, int 
             check_tie(base, cols, v, t);
         }
 
+    // Equal magnitudes in a winner: which of them a row keeps depends, in the reference, on a permutation that every
+    // partial_sort call of the whole run has shaped.  Reproducing it means replaying the run sequentially (the cost of
+    // the complete search on one thread); without the replay the lower column wins, which keeps the same magnitudes.
     bool need_replay = false;
-    for (const GroupTask& t : tasks) need_replay |= t.tie;
+    if (replay_ties)
+        for (const GroupTask& t : tasks) need_replay |= t.tie;
 
     // Phase 2: masks and column offsets.  Without ties the two largest of each
     // row are unique as a set and the mask needs no history.

@@ -31,8 +31,10 @@ struct GroupTask {
 // tasks of the search: (rows / v) blocks x per_block groups, block-major
 int select_task_count(int rows, int cols, int m, int v, int* per_block_out);
 // the selector with the winners of the search supplied by the caller (winners == nullptr: searched on the host)
+// replay_ties: reproduce the reference's choice among EQUAL magnitudes (sequential replay of the whole run when any
+// winner has such a tie); false: the lower column index wins
 int select_columns_with_winners(const float* dense_abs, int rows, int cols, int n, int m, int v, const GroupTask* winners,
-                                int32_t* masks, int32_t* columns, int threads);
+                                bool replay_ties, int32_t* masks, int32_t* columns, int threads);
 int select_columns_f32(const float* dense_abs, int rows, int cols, int n, int m, int v, int32_t* masks,
                        int32_t* columns, int threads);
 

@@ -62,9 +62,11 @@ def decode(values, metadata, columns, rows, cols, n, m, v, threads=0):
     return dense
 
 
-def select_columns(dense_abs, n, m, v, threads=0, gpu=False, stream=None):
+def select_columns(dense_abs, n, m, v, threads=0, gpu=False, stream=None, exact_ties=True):
     """|A| float32 (rows, cols) -> (masks int32 (rows, cols), columns int32).  gpu=True runs the search over the
-    column subsets on the GPU (same result bit for bit; 12 s -> milliseconds for a 4096 x 1024 matrix at m = 32)."""
+    column subsets on the GPU (same result bit for bit; 12 s -> milliseconds for a 4096 x 1024 matrix at m = 32).
+    exact_ties=False (GPU path only): among EQUAL magnitudes the lower column wins instead of the reference's
+    history-dependent choice, which spares the sequential replay that such ties otherwise force."""
     d = np.ascontiguousarray(dense_abs, dtype=np.float32)
     rows, cols = d.shape
     g = geometry(rows, cols, n, m, v)
@@ -72,7 +74,8 @@ def select_columns(dense_abs, n, m, v, threads=0, gpu=False, stream=None):
     columns = np.zeros(g.n_columns, np.int32)
     if gpu:
         _lib.check(_lib.lib().spatha_vnm_select_columns_f32_gpu(_p(d), rows, cols, n, m, v, _p(masks), _p(columns), threads,
-                                                                stream), "spatha_vnm_select_columns_f32_gpu")
+                                                                1 if exact_ties else 0, stream),
+                   "spatha_vnm_select_columns_f32_gpu")
     else:
         _lib.check(_lib.lib().spatha_vnm_select_columns_f32(_p(d), rows, cols, n, m, v, _p(masks), _p(columns), threads),
                    "spatha_vnm_select_columns_f32")

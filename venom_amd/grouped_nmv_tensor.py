@@ -14,11 +14,13 @@ def round_up(x, y):
     return -(-x // y) * y
 
 
-def nm_vector_mask_sparsify(tensor, n, m, tileM, threads=0, gpu=None):
+def nm_vector_mask_sparsify(tensor, n, m, tileM, threads=0, gpu=None, exact_ties=True):
     """Per tileM x m block keep the 4 columns with the largest sum of per-row top-n magnitudes,
     per row the n largest of those.  Returns (masks int32 [rows, cols], columns int32 flat), both
     on the CPU, like the reference.  gpu: search the column subsets on the GPU (default: when the
-    tensor lives there); the result is the same bit for bit."""
+    tensor lives there); the result is the same bit for bit.  exact_ties=False (with gpu): equal magnitudes are
+    resolved towards the lower column instead of through the reference's history-dependent order, which avoids a
+    sequential replay of the whole search whenever such a tie occurs (common for fp16 weights)."""
     if tensor.dim() != 2:
         raise NotImplementedError("Only support layers of dimension 2")
     if gpu is None:
@@ -28,7 +30,7 @@ def nm_vector_mask_sparsify(tensor, n, m, tileM, threads=0, gpu=None):
         dev = tensor.device if tensor.is_cuda else torch.device("cuda:0")
         with torch.cuda.device(dev):
             masks, columns = F.select_columns(mag, n, m, tileM, threads=threads, gpu=True,
-                                              stream=torch.cuda.current_stream(dev).cuda_stream)
+                                              stream=torch.cuda.current_stream(dev).cuda_stream, exact_ties=exact_ties)
     else:
         masks, columns = F.select_columns(mag, n, m, tileM, threads=threads)
     return torch.from_numpy(masks), torch.from_numpy(columns)

@@ -47,7 +47,7 @@ def main():
     ap.add_argument("--v", type=int, default=64)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--extra", action="store_true", help="also time the other BASELINE shapes (reported under 'extra')")
+    ap.add_argument("--extra", action="store_true", help="also time the other benchmark shapes (reported under 'extra')")
     ap.add_argument("--ablation", action="store_true",
                     help="also time the same matrix with identity column-loc (the reference's IDEAL_KERNEL ablation) and, "
                          "if `python -m venom_amd.build --ablation` has been run, the OUT_32B build (4-byte stores of C)")

@@ -14,7 +14,7 @@ from venom_amd import format as F
 
 BENCH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "venom_amd", "lib", "benchmark_spmm")
 
-# README.md:174 of the reference (BASELINE config 1)
+# README.md:174 of the reference (its worked example: 1024 x 4096 x 4096 at 128:2:8)
 CONFIG1 = ("--sparsity-type n-to-m --spmm spatha --gemm cuBlas --precision half --meta-block-size 32 --block-size 4 "
            "--nn_row 2 --mm_row 8 --m 1024 --k 4096 --n 4096 --d 0.5 --bm 128 --bn 64 --bk 32 --wm 32 --wn 64 --wk 32 "
            "--mm 16 --mn 8 --mk 32 --nstage 2 --random --check").split()

@@ -258,7 +258,7 @@ def test_reference_encoded_matrices(gpu, path):
 
 
 def test_config1_gaussian_within_tolerance(gpu):
-    """BASELINE config 1: 1024 x 4096 x 4096, 128:2:8, A ~ N(0,1), B ~ U(-1,1), seed 0."""
+    """The reference README's example shape: 1024 x 4096 x 4096, 128:2:8, A ~ N(0,1), B ~ U(-1,1), seed 0."""
     rows, cols, N, m, v = 1024, 4096, 4096, 8, 128
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=0, value_std=1.0)
     rng = np.random.default_rng(0)
@@ -305,7 +305,7 @@ def test_full_size_checksums(gpu, rows, cols, N, m, v):
 
 @pytest.mark.parametrize("N", [16, 256])
 def test_gpt3_ffn_shape_blocks_within_tolerance(gpu, N):
-    """BASELINE config 4: A 49152 x 12288 in 128:2:16, values ~N(0, 0.02), B ~N(0, 1); N = 16 runs on the skinny
+    """GPT-3 feed-forward shape: A 49152 x 12288 in 128:2:16, values ~N(0, 0.02), B ~N(0, 1); N = 16 runs on the skinny
     kernel.  Three V-row blocks of C are compared with the float64 product of their decoded rows."""
     rows, cols, m, v = 49152, 12288, 16, 128
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=0, value_std=0.02)

@@ -52,6 +52,16 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 
+// Development knobs (time accounting: parts of a kernel switched off, results then wrong on purpose) exist only in
+// builds with -DSPATHA_DEV_PROFILE; in the product they are compile-time false.
+#ifdef SPATHA_DEV_PROFILE
+#define SPATHA_KNOB(bit) (p.debug & (bit))
+#define SPATHA_SKEW_ON(p) ((p).skew > 0)
+#else
+#define SPATHA_KNOB(bit) false
+#define SPATHA_SKEW_ON(p) false
+#endif
+
 // Row-major stores of C: 16 bytes per lane.  Built with -DSPATHA_OUT_32B (the counterpart of the reference's OUT_32B
 // ablation switch, CMakeLists.txt:25-33) the same bytes leave as four 4-byte stores, to measure what the wide
 // stores are worth; assembly, so that the compiler cannot merge them again.
@@ -211,7 +221,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_kernel(SpmmParams p) {
         for (int i = 0; i < B_LOADS; i++) {
             uint32_t row = rows_next[i];
             u32x4 z = {0u, 0u, 0u, 0u};
-            breg[i] = (row != 0xffffffffu && bcol_ok && !(p.debug & 1)) ? *(const u32x4*)(bbase + (int64_t)row * N) : z;
+            breg[i] = (row != 0xffffffffu && bcol_ok && !SPATHA_KNOB(1)) ? *(const u32x4*)(bbase + (int64_t)row * N) : z;
         }
 #pragma unroll
         for (int mb = 0; mb < 4; mb++) areg[mb] = *(const u32x4*)(a_blk + (int64_t)s * APACK_BLOCK + mb * 1024 + lane * 16);
@@ -334,7 +344,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_kernel(SpmmParams p) {
             const int row = 16 * (L & 3) + (L >> 2);
             const int col = n0 + wn * 64 + ch * 8;
             u32x4 v = *(const u32x4*)(st + L * PITCH_C + ch * 16);
-            if (col < N && !(p.debug & 2)) store_c16(p.C + ((int64_t)m0 + wm * 64 + row) * N + col, v);
+            if (col < N && !SPATHA_KNOB(2)) store_c16(p.C + ((int64_t)m0 + wm * 64 + row) * N + col, v);
         }
     }
 }
@@ -553,7 +563,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_pipe_kernel(SpmmParams p) {
 #pragma unroll
         for (int j = 0; j < NB_LOADS; j++) {
             const int inst = wave * NB_LOADS + j;
-            const bool ok = (rows[j] != 0xffffffffu) && (b_col_off[j] >= 0) && !(p.debug & 1);
+            const bool ok = (rows[j] != 0xffffffffu) && (b_col_off[j] >= 0) && !SPATHA_KNOB(1);
             const char* src = (const char*)p.B + (int64_t)rows[j] * N * 2 + b_col_off[j];
             src = ok ? src : zero_src;
             dma_b128(src, stage + inst * 1024);
@@ -644,7 +654,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_pipe_kernel(SpmmParams p) {
                 *(half8_t*)(dst + 8) = hi;
             }
         }
-    } else if (!(p.debug & 4)) {
+    } else if (!SPATHA_KNOB(4)) {
         __syncthreads();                 // every wave is done reading the stages
         char* stg = smem + wave * (64 * PITCH_C);
 #pragma unroll
@@ -664,7 +674,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_pipe_kernel(SpmmParams p) {
             const int row = 16 * (Lr & 3) + (Lr >> 2);
             const int col = n0 + wn * 64 + ch * 8;
             u32x4 v = *(const u32x4*)(stg + Lr * PITCH_C + ch * 16);
-            if (col < N && !(p.debug & 2)) store_c16(p.C + ((int64_t)m0 + wm * 64 + row) * N + col, v);
+            if (col < N && !SPATHA_KNOB(2)) store_c16(p.C + ((int64_t)m0 + wm * 64 + row) * N + col, v);
         }
     }
 }
@@ -1058,7 +1068,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_persist_kernel(SpmmParams p)
 #pragma unroll
         for (int j = 0; j < NB_LOADS; j++) {
             const int col = is_tn * BN + src_chunk[j] * 8;
-            coloff[j] = (col < N && !(p.debug & 1)) ? (uint32_t)col * 2u : 0xF0000000u;
+            coloff[j] = (col < N && !SPATHA_KNOB(1)) ? (uint32_t)col * 2u : 0xF0000000u;
         }
     };
     set_coloff();
@@ -1193,13 +1203,13 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_persist_kernel(SpmmParams p)
                     lo = lo + bias_lo;
                     hi = hi + bias_hi;
                 }
-                if (col < N && !(p.debug & 2)) {
+                if (col < N && !SPATHA_KNOB(2)) {
                     uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
                     *(half8_t*)dst = lo;
                     *(half8_t*)(dst + 8) = hi;
                 }
             }
-        } else if (!(p.debug & 4)) {
+        } else if (!SPATHA_KNOB(4)) {
             // 16-row slabs through a wave-private LDS buffer -> 128-byte row segments
             char* stg = smem + EPI_BASE + wave * (16 * EPI_PITCH);
 #pragma unroll
@@ -1216,7 +1226,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_persist_kernel(SpmmParams p)
                     const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
                     const int col = cn0 + wn * 64 + ch * 8;
                     u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
-                    if (col < N && !(p.debug & 2)) store_c16(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col, v);
+                    if (col < N && !SPATHA_KNOB(2)) store_c16(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col, v);
                 }
                 __builtin_amdgcn_wave_barrier();
             }
@@ -1353,7 +1363,7 @@ __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk&
 #pragma unroll
         for (int j = 0; j < NB_LOADS; j++) {
             const int col = is_tn * BN + src_chunk[j] * 8;
-            coloff[j] = (col < N && !(p.debug & 1)) ? (uint32_t)col * 2u : 0xF0000000u;
+            coloff[j] = (col < N && !SPATHA_KNOB(1)) ? (uint32_t)col * 2u : 0xF0000000u;
         }
     };
     set_coloff();
@@ -1431,7 +1441,7 @@ __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk&
     for (int q = 0; q < q_main; q++) {
         wait_vmcnt<(PA - 1) * LOADS>();
         __syncthreads();
-        if (!(p.debug & 8)) issue_from_ring();
+        if (!SPATHA_KNOB(8)) issue_from_ring();
     }
     // drain: nothing left to issue
     for (int q = q_main; q < Q; q++) {
@@ -1469,7 +1479,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk&
             for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
         for (int c_step = 0; c_step < S; c_step++) {
             __syncthreads();
-            if (!(p.debug & 16)) mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {});
+            if (!SPATHA_KNOB(16)) mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {});
             c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
         }
         const int cm0 = c_tm * BM, cn0 = c_tn * BN;
@@ -1498,13 +1508,13 @@ __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk&
                     lo = lo + bias_lo;
                     hi = hi + bias_hi;
                 }
-                if (col < N && !(p.debug & 2)) {
+                if (col < N && !SPATHA_KNOB(2)) {
                     uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
                     *(half8_t*)dst = lo;
                     *(half8_t*)(dst + 8) = hi;
                 }
             }
-        } else if (!(p.debug & 4)) {
+        } else if (!SPATHA_KNOB(4)) {
             // 16-row slabs through a wave-private LDS buffer -> 128-byte row segments
             char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
 #pragma unroll
@@ -1521,7 +1531,7 @@ __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk&
                     const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
                     const int col = cn0 + wn * 64 + ch * 8;
                     u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
-                    if (col < N && !(p.debug & 2)) store_c16(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col, v);
+                    if (col < N && !SPATHA_KNOB(2)) store_c16(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col, v);
                 }
                 __builtin_amdgcn_wave_barrier();
             }
@@ -1600,7 +1610,7 @@ __device__ __forceinline__ void ws_consumer_deferred(const SpmmParams& p, const 
     const int i_off = B_BYTES + wm * APACK_BLOCK + 4096 + lane * 4;
     const int j16 = lane & 15, ib = lane >> 4;
     char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
-    const bool stores_on = !(p.debug & 2);
+    const bool stores_on = !SPATHA_KNOB(2);
 
     int c_tm = walk.tm0, c_tn = walk.tn0;
     int pm0 = 0, pn0 = 0;           // origin of the tile held in pend
@@ -1630,12 +1640,12 @@ __device__ __forceinline__ void ws_consumer_deferred(const SpmmParams& p, const 
             for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
         for (int c_step = 0; c_step < S; c_step++) {
             __syncthreads();
-            if (!(p.debug & 16)) mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {});
+            if (!SPATHA_KNOB(16)) mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {});
             c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
-            if (have_pend && c_step < 4 && !(p.debug & 4)) flush_part(c_step);
+            if (have_pend && c_step < 4 && !SPATHA_KNOB(4)) flush_part(c_step);
         }
         // a k-loop shorter than four steps leaves parts of the previous tile unwritten
-        if (have_pend && !(p.debug & 4))
+        if (have_pend && !SPATHA_KNOB(4))
             for (int part = S; part < 4; part++) flush_part(part);
         const int cm0 = c_tm * BM, cn0 = c_tn * BN;
         const bool with_bias = (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) && p.bias;
@@ -1664,7 +1674,7 @@ __device__ __forceinline__ void ws_consumer_deferred(const SpmmParams& p, const 
         have_pend = true;
         walk.next(c_tm, c_tn);
     }
-    if (have_pend && !(p.debug & 4))
+    if (have_pend && !SPATHA_KNOB(4))
         for (int part = 0; part < 4; part++) flush_part(part);
 }
 
@@ -1777,7 +1787,7 @@ __device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const Tile
                 for (int b = 0; b < 4; b++) acc[h][a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
         for (int c_step = 0; c_step < S; c_step++) {
             __syncthreads();
-            if (!(p.debug & 16)) mma_stage_tall<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc);
+            if (!SPATHA_KNOB(16)) mma_stage_tall<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc);
             c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
         }
         const int cm0 = c_tm * BM, cn0 = c_tn * BN;
@@ -1785,10 +1795,10 @@ __device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const Tile
         for (int h = 0; h < 2; h++) {
             if (p.fuse) fused_bias_act(acc[h], p.bias, (int64_t)cm0 + h * 64 + ib * 16, p.act);
             if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
-                if (!(p.debug & 4))
+                if (!SPATHA_KNOB(4))
                     store_block_transposed_slab(acc[h], smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH), p.C, p.fuse ? nullptr : p.bias,
-                                                (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !(p.debug & 2));
-            } else if (!(p.debug & 4)) {
+                                                (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !SPATHA_KNOB(2));
+            } else if (!SPATHA_KNOB(4)) {
                 char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
 #pragma unroll
                 for (int mb = 0; mb < 4; mb++) {
@@ -1804,7 +1814,7 @@ __device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const Tile
                         const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
                         const int col = cn0 + wn * 64 + ch * 8;
                         u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
-                        if (col < N && !(p.debug & 2)) store_c16(p.C + ((int64_t)cm0 + h * 64 + row) * N + col, v);
+                        if (col < N && !SPATHA_KNOB(2)) store_c16(p.C + ((int64_t)cm0 + h * 64 + row) * N + col, v);
                     }
                     __builtin_amdgcn_wave_barrier();
                 }
@@ -1825,7 +1835,7 @@ __global__ __launch_bounds__((WN + NP) * 64) void spmm_wst_kernel(SpmmParams p) 
     TileWalk walk;
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
-    if (p.skew > 0) {
+    if (SPATHA_SKEW_ON(p)) {
         const int units = ((blockIdx.x >> 3) & 7) * p.skew;
         for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);
     }
@@ -2023,7 +2033,7 @@ __device__ __forceinline__ void ds_producer(const SpmmParams& p, const TileWalk&
         for (int j = 0; j < NB_LOADS; j++) {
             const int row = (PR * NB_LOADS + j) * 4 + slot_row;             // dense row inside the stage
             const int col = is_tn * BN + (slot_chunk ^ ((row & 7) << 1)) * 8;
-            voff[j] = (col < N && row < dense_rows && !(p.debug & 1)) ? (uint32_t)row * row_bytes_b + (uint32_t)col * 2u
+            voff[j] = (col < N && row < dense_rows && !SPATHA_KNOB(1)) ? (uint32_t)row * row_bytes_b + (uint32_t)col * 2u
                                                                        : 0xF0000000u;
         }
     };
@@ -2060,7 +2070,7 @@ __device__ __forceinline__ void ds_producer(const SpmmParams& p, const TileWalk&
     for (int q = 0; q < q_main; q++) {
         wait_vmcnt<(PA - 1) * LOADS>();
         __syncthreads();
-        if (!(p.debug & 8)) issue_batch();
+        if (!SPATHA_KNOB(8)) issue_batch();
     }
     for (int q = q_main; q < Q; q++) {
         wait_stages<LOADS, PA - 1>(Q - 1 - q);
@@ -2125,7 +2135,7 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
             SPATHA_PROF_MARK(0)
             __syncthreads();
             SPATHA_PROF_MARK(1)
-            if (!(p.debug & 16)) {
+            if (!SPATHA_KNOB(16)) {
                 const char* st = smem + c_stage;
 #pragma unroll
                 for (int h = 0; h < H; h++) {
@@ -2180,12 +2190,12 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
             const bool pre = p.fuse && (p.act != SPATHA_ACT_NONE || OUT_LAYOUT == SPATHA_OUT_TRANSPOSED);
             if (pre) fused_bias_act(acc[h], p.bias, (int64_t)cm0 + h * 64 + ib * 16, p.act);
             if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
-                if (!(p.debug & 4))
+                if (!SPATHA_KNOB(4))
                     store_block_transposed_slab(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, p.fuse ? nullptr : p.bias,
-                                                (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !(p.debug & 2));
-            } else if (!(p.debug & 4)) {
+                                                (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !SPATHA_KNOB(2));
+            } else if (!SPATHA_KNOB(4)) {
                 store_block_row_major_tr<Cfg::NC == 8>(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C,
-                                                        (int64_t)cm0 + h * 64, cn0 + wn * 64, N, lane, !(p.debug & 2),
+                                                        (int64_t)cm0 + h * 64, cn0 + wn * 64, N, lane, !SPATHA_KNOB(2),
                                                         (p.fuse && !pre) ? p.bias : nullptr);
             }
         }
@@ -2421,15 +2431,15 @@ __device__ __forceinline__ void ds_consumer_pp(const SpmmParams& p, const TileWa
                     lo = lo + bias_lo;
                     hi = hi + bias_hi;
                 }
-                if (col < N && !(p.debug & 2)) {
+                if (col < N && !SPATHA_KNOB(2)) {
                     uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
                     *(half8_t*)dst = lo;
                     *(half8_t*)(dst + 8) = hi;
                 }
             }
-        } else if (!(p.debug & 4)) {
+        } else if (!SPATHA_KNOB(4)) {
             store_block_row_major_tr<true>(acc, smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, (int64_t)cm0,
-                                           cn0 + wn * 64, N, lane, !(p.debug & 2));
+                                           cn0 + wn * 64, N, lane, !SPATHA_KNOB(2));
         }
         SPATHA_PROF_MARK(2)
     };
@@ -2461,7 +2471,7 @@ __device__ __forceinline__ void ds_consumer_pp(const SpmmParams& p, const TileWa
             SPATHA_PROF_MARK(1)
             const char* st = smem + c_stage;
             if (!LATE) {
-                if (!(p.debug & 16)) {
+                if (!SPATHA_KNOB(16)) {
                     read_a(st);
                     read_frag(st, 0);
                     read_frag(st, 1);
@@ -2478,7 +2488,7 @@ __device__ __forceinline__ void ds_consumer_pp(const SpmmParams& p, const TileWa
                     SPATHA_MMA4P(3)
                     __builtin_amdgcn_sched_barrier(0);
                 }
-            } else if (!(p.debug & 16)) {
+            } else if (!SPATHA_KNOB(16)) {
                 // registers hold the previous step (all zeros before the first one)
                 SPATHA_MMA4P(0)
                 __builtin_amdgcn_sched_barrier(0);
@@ -2512,7 +2522,7 @@ __device__ __forceinline__ void ds_consumer_pp(const SpmmParams& p, const TileWa
         walk.next(c_tm, c_tn);
     }
     if (LATE) {
-        if (!(p.debug & 16)) {
+        if (!SPATHA_KNOB(16)) {
             SPATHA_MMA4P(0)
             SPATHA_MMA4P(1)
             SPATHA_MMA4P(2)
@@ -2557,7 +2567,7 @@ __global__ __launch_bounds__((NC + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
     TileWalk walk;
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
-    if (p.skew > 0) {
+    if (SPATHA_SKEW_ON(p)) {
         // workgroups of one XCD start up to 7 * skew * 1024 clocks apart (write-out bursts spread over time)
         const int units = ((blockIdx.x >> 3) & 7) * p.skew;
         for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);
@@ -2682,7 +2692,7 @@ __device__ __forceinline__ void dsf_producer(const SpmmParams& p, const TileWalk
         for (int j = 0; j < NB_LOADS; j++) {
             const int row = (PR * NB_LOADS + j) * 4 + slot_row;
             const int col = is_tn * BN + (slot_chunk ^ ((row & 7) << 1)) * 8;
-            voff[j] = (col < N && row < dense_rows && !(p.debug & 1)) ? (uint32_t)row * row_bytes_b + (uint32_t)col * 2u
+            voff[j] = (col < N && row < dense_rows && !SPATHA_KNOB(1)) ? (uint32_t)row * row_bytes_b + (uint32_t)col * 2u
                                                                        : 0xF0000000u;
         }
     };
@@ -2705,7 +2715,7 @@ __device__ __forceinline__ void dsf_producer(const SpmmParams& p, const TileWalk
                 flag_wait(empty_base + st * 4, (uint32_t)Cfg::NC * use);
             }
         }
-        if (!(p.debug & 8)) {
+        if (!SPATHA_KNOB(8)) {
             const uint32_t stage = smem_base + st * STAGE_BYTES;
 #pragma unroll
             for (int j = 0; j < NB_LOADS; j++) bdma_b128(voff[j], rsrc_b, b_soff, stage + (PR * NB_LOADS + j) * 1024);
@@ -2733,7 +2743,7 @@ __device__ __forceinline__ void dsf_producer(const SpmmParams& p, const TileWalk
         }
         if (pending) {
             // everything but the batch just issued has landed: publish the previous batch
-            if (!(p.debug & 8)) wait_vmcnt<LOADS>();
+            if (!SPATHA_KNOB(8)) wait_vmcnt<LOADS>();
             flag_signal(full_base + prev_st * 4, lane);
         }
         pending = true;
@@ -2912,15 +2922,15 @@ __device__ __forceinline__ void dsf_consumer(const SpmmParams& p, const TileWalk
                         lo = lo + bias_lo;
                         hi = hi + bias_hi;
                     }
-                    if (col < N && !(p.debug & 2)) {
+                    if (col < N && !SPATHA_KNOB(2)) {
                         uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
                         *(half8_t*)dst = lo;
                         *(half8_t*)(dst + 8) = hi;
                     }
                 }
-            } else if (!(p.debug & 4)) {
+            } else if (!SPATHA_KNOB(4)) {
                 store_block_row_major_tr<true>(acc, smem + Cfg::EPI_BASE + wave * TR8_SLAB_BYTES, p.C, (int64_t)cm0,
-                                               cn0 + wn * 64, N, lane, !(p.debug & 2));
+                                               cn0 + wn * 64, N, lane, !SPATHA_KNOB(2));
             }
             SPATHA_PROF_MARK(2)
             zero_acc();
@@ -3111,7 +3121,7 @@ __global__ __launch_bounds__(256) void spmm_skinny_kernel(SpmmParams p) {
         half4_t h4;
 #pragma unroll
         for (int r = 0; r < 4; r++) h4[r] = (_Float16)sum[r];
-        if (col >= N || (p.debug & 2)) continue;
+        if (col >= N || SPATHA_KNOB(2)) continue;
         if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
             if (p.bias) h4 = h4 + *(const half4_t*)(p.bias + row0);
             *(half4_t*)(p.C + (int64_t)col * p.rows + row0) = h4;
@@ -3174,7 +3184,7 @@ __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams
     if (walk.my_tiles == 0) return;
     // Workgroups of one XCD start up to 7 * skew apart, so that tiles do not all finish (and
     // hit HBM with their stores) at the same moment on every CU.
-    if (p.skew > 0) {
+    if (SPATHA_SKEW_ON(p)) {
         const int units = ((blockIdx.x >> 3) & 7) * p.skew;
         for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);      // 16 * 64 clocks
     }

@@ -65,6 +65,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 // Row-major stores of C: 16 bytes per lane.  Built with -DSPATHA_OUT_32B (the counterpart of the reference's OUT_32B
 // ablation switch, CMakeLists.txt:25-33) the same bytes leave as four 4-byte stores, to measure what the wide
 // stores are worth; assembly, so that the compiler cannot merge them again.
+template <bool WRITE_THROUGH = false>
 __device__ __forceinline__ void store_c16(uint16_t* dst, u32x4 v) {
 #ifdef SPATHA_OUT_32B
     asm volatile(
@@ -74,7 +75,15 @@ __device__ __forceinline__ void store_c16(uint16_t* dst, u32x4 v) {
         "global_store_dword %0, %4, off offset:12" ::"v"(dst), "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w)
         : "memory");
 #else
-    *(u32x4*)dst = v;
+    // WRITE_THROUGH (sc1): the result goes through to memory instead of staying in the XCD's L2, where it would push
+    // out the operand panels the other workgroups of the XCD are re-reading.  Pays in the dense-staged kernels
+    // (4096 x 1024 x 16384 at 64:2:8: 63.7 -> 62.2 us row-major, 66.3 -> 60.7 us transposed + bias) and in the tall
+    // kernel's transposed write-out (1024 x 4096 x 16384 at 128:2:16: 33 -> 30.4 us), not in the 128 x 128 tiles
+    // (37.7 -> 39.3 us at 128:2:32); the non-temporal hint costs 3 us everywhere.
+    // The s_nop covers the two wait states that the hardware needs between a store of more than 64 bits and a VALU
+    // write of its data registers: the compiler inserts them for its own stores, not after an asm statement.
+    if (WRITE_THROUGH) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
+    else *(u32x4*)dst = v;
 #endif
 }
 
@@ -460,6 +469,15 @@ __device__ __forceinline__ void mma_stage(const char* st, int a_off, int i_off, 
     SPATHA_MMA4(3, bf1)
 }
 
+constexpr int TT_PITCH = 144;                      // 64 rows x 2 B + 16 B pad (keeps 16-byte alignment)
+constexpr int TT_SLAB_BYTES = 8 * TT_PITCH;        // per wave
+// Transposed write-out (C^T[N][rows], + bias) of one wave's 64 x 64 block through an LDS slab of 8 columns x 64 rows,
+// so that every store instruction covers whole 128-byte lines (defined further down).
+template <bool WRITE_THROUGH = false>
+__device__ __forceinline__ void store_block_transposed_slab(const float4_t (&acc)[4][4], char* stg, uint16_t* C,
+                                                            const uint16_t* bias, int64_t row0, int col0, int rows_total, int N,
+                                                            int lane, bool stores_on);
+
 // ---------------------------------------------------------------------------
 // Pipelined SpMM kernel.  Everything the k-loop consumes -- the gathered B rows, the packed
 // A operands and their index words -- is copied global -> LDS by the DMA path
@@ -483,11 +501,13 @@ __device__ __forceinline__ void mma_stage(const char* st, int a_off, int i_off, 
 //                               index of row rho with 2*(rho % 8) on the GLOBAL side of the copy
 //   [.., + WM*APACK_BLOCK)      per 64-row wave tile: 4 KiB A operands + 512 B index words
 // ---------------------------------------------------------------------------
+// (s_nop: one wait state between the write of m0 and the LDS-DMA instruction that reads it; the compiler does not
+// look inside an asm statement for that.)
 __device__ __forceinline__ void dma_b128(const void* gptr, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "m0");
 }
 __device__ __forceinline__ void dma_b32(const void* gptr, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(gptr) : "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(gptr) : "m0");
 }
 template <int N_>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -627,33 +647,9 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_pipe_kernel(SpmmParams p) {
     if (p.fuse) fused_bias_act(acc, p.bias, (int64_t)m0 + wm * 64 + ib * 16, p.act);
     const uint16_t* bias = p.fuse ? nullptr : p.bias;
     if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
-        const int64_t row0 = (int64_t)m0 + wm * 64 + ib * 16;
-        half8_t bias_lo, bias_hi;
-        if (bias) {
-            bias_lo = *(const half8_t*)(bias + row0);
-            bias_hi = *(const half8_t*)(bias + row0 + 8);
-        }
-#pragma unroll
-        for (int nb = 0; nb < 4; nb++) {
-            const int col = n0 + wn * 64 + nb * 16 + j;
-            half8_t lo, hi;
-#pragma unroll
-            for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
-                    hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
-                }
-            if (bias) {
-                lo = lo + bias_lo;
-                hi = hi + bias_hi;
-            }
-            if (col < N) {
-                uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
-                *(half8_t*)dst = lo;
-                *(half8_t*)(dst + 8) = hi;
-            }
-        }
+        __syncthreads();                 // every wave is done reading the stages: their memory becomes the slabs
+        store_block_transposed_slab<true>(acc, smem + wave * TT_SLAB_BYTES, p.C, bias, (int64_t)m0 + wm * 64, n0 + wn * 64,
+                                          p.rows, N, lane, true);
     } else if (!SPATHA_KNOB(4)) {
         __syncthreads();                 // every wave is done reading the stages
         char* stg = smem + wave * (64 * PITCH_C);
@@ -964,12 +960,12 @@ __device__ __forceinline__ i32x4 make_buffer(const void* base, uint32_t bytes) {
     return r;
 }
 __device__ __forceinline__ void bdma_b128(uint32_t voff, i32x4 rsrc, uint32_t soff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc),
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc),
                  "s"(soff)
                  : "m0");
 }
 __device__ __forceinline__ void bdma_b32(uint32_t voff, i32x4 rsrc, uint32_t soff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc),
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc),
                  "s"(soff)
                  : "m0");
 }
@@ -1486,34 +1482,8 @@ __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk&
         if (p.fuse) fused_bias_act(acc, p.bias, (int64_t)cm0 + wm * 64 + ib * 16, p.act);
         const uint16_t* bias = p.fuse ? nullptr : p.bias;
         if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
-            // the lane owns 16 consecutive matrix rows of one output column: 32 contiguous bytes
-            const int64_t row0 = (int64_t)cm0 + wm * 64 + ib * 16;
-            half8_t bias_lo, bias_hi;
-            if (bias) {
-                bias_lo = *(const half8_t*)(bias + row0);
-                bias_hi = *(const half8_t*)(bias + row0 + 8);
-            }
-#pragma unroll
-            for (int nb = 0; nb < 4; nb++) {
-                const int col = cn0 + wn * 64 + nb * 16 + j16;
-                half8_t lo, hi;
-#pragma unroll
-                for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
-                        hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
-                    }
-                if (bias) {
-                    lo = lo + bias_lo;
-                    hi = hi + bias_hi;
-                }
-                if (col < N && !SPATHA_KNOB(2)) {
-                    uint16_t* dst = p.C + (int64_t)col * p.rows + row0;
-                    *(half8_t*)dst = lo;
-                    *(half8_t*)(dst + 8) = hi;
-                }
-            }
+            store_block_transposed_slab<true>(acc, smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH), p.C, bias,
+                                              (int64_t)cm0 + wm * 64, cn0 + wn * 64, p.rows, N, lane, !SPATHA_KNOB(2));
         } else if (!SPATHA_KNOB(4)) {
             // 16-row slabs through a wave-private LDS buffer -> 128-byte row segments
             char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
@@ -1681,8 +1651,7 @@ __device__ __forceinline__ void ws_consumer_deferred(const SpmmParams& p, const 
 // Transposed write-out (C^T[N][rows], + bias) of one wave's 64 x 64 block through an LDS slab of 8 columns x 64 rows.
 // Straight from the accumulators a lane could only store 16-byte pieces 32 bytes apart; through the slab every
 // store instruction writes 8 output rows (columns of C) x 128 contiguous bytes.
-constexpr int TT_PITCH = 144;                      // 64 rows x 2 B + 16 B pad (keeps 16-byte alignment)
-constexpr int TT_SLAB_BYTES = 8 * TT_PITCH;        // per wave
+template <bool WRITE_THROUGH>
 __device__ __forceinline__ void store_block_transposed_slab(const float4_t (&acc)[4][4], char* stg, uint16_t* C,
                                                             const uint16_t* bias, int64_t row0, int col0, int rows_total, int N,
                                                             int lane, bool stores_on) {
@@ -1712,7 +1681,7 @@ __device__ __forceinline__ void store_block_transposed_slab(const float4_t (&acc
             const u32x4 v = *(const u32x4*)(stg + rn * TT_PITCH + rc * 16);
             __builtin_amdgcn_wave_barrier();
             const int col = col0 + nb * 16 + hf * 8 + rn;
-            if (col < N && stores_on) *(u32x4*)(C + (int64_t)col * rows_total + row0 + rc * 8) = v;
+            if (col < N && stores_on) store_c16<WRITE_THROUGH>(C + (int64_t)col * rows_total + row0 + rc * 8, v);
         }
     }
 }
@@ -1796,7 +1765,7 @@ __device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const Tile
             if (p.fuse) fused_bias_act(acc[h], p.bias, (int64_t)cm0 + h * 64 + ib * 16, p.act);
             if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
                 if (!SPATHA_KNOB(4))
-                    store_block_transposed_slab(acc[h], smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH), p.C, p.fuse ? nullptr : p.bias,
+                    store_block_transposed_slab<true>(acc[h], smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH), p.C, p.fuse ? nullptr : p.bias,
                                                 (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !SPATHA_KNOB(2));
             } else if (!SPATHA_KNOB(4)) {
                 char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
@@ -1959,7 +1928,7 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
         short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff));
         short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff + 4 * PITCH));
         __builtin_amdgcn_wave_barrier();
-        if (ph > 0 && live) store_c16(C + (row0 + held_row) * N + out_col, held);
+        if (ph > 0 && live) store_c16<true>(C + (row0 + held_row) * N + out_col, held);
         held.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
         held.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
         held.z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
@@ -1967,7 +1936,7 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
         const int q = 8 * sidx + q_lo;
         held_row = 16 * (q >> 2) + 4 * mb + (q & 3);
     }
-    if (live) store_c16(C + (row0 + held_row) * N + out_col, held);
+    if (live) store_c16<true>(C + (row0 + held_row) * N + out_col, held);
     __builtin_amdgcn_wave_barrier();
 }
 
@@ -2191,7 +2160,7 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
             if (pre) fused_bias_act(acc[h], p.bias, (int64_t)cm0 + h * 64 + ib * 16, p.act);
             if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
                 if (!SPATHA_KNOB(4))
-                    store_block_transposed_slab(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, p.fuse ? nullptr : p.bias,
+                    store_block_transposed_slab<true>(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, p.fuse ? nullptr : p.bias,
                                                 (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !SPATHA_KNOB(2));
             } else if (!SPATHA_KNOB(4)) {
                 store_block_row_major_tr<Cfg::NC == 8>(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C,
@@ -2332,7 +2301,7 @@ __device__ __forceinline__ void ds_consumer_half(const SpmmParams& p, const Tile
         const bool pre = p.fuse && (p.act != SPATHA_ACT_NONE || OUT_LAYOUT == SPATHA_OUT_TRANSPOSED);
         if (pre) fused_bias_act(acc, p.bias, (int64_t)cm0 + ib * 16, p.act);
         if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
-            store_block_transposed_slab(acc, smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, p.fuse ? nullptr : p.bias,
+            store_block_transposed_slab<true>(acc, smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, p.fuse ? nullptr : p.bias,
                                         (int64_t)cm0, cn0 + wn * 64, p.rows, N, lane, true);
         else
             store_block_row_major_tr<true>(acc, smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, (int64_t)cm0, cn0 + wn * 64, N,

@@ -26,7 +26,7 @@ SMFMAC_PEAK_TFLOPS = 5033.0    # fp16 MFMA with 2:4 structured sparsity (dense f
 # HBM-side bytes per launch of the default workload's kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # scaled by a plain 256 MiB copy (summary under profiles/, named for the kernel); keyed by kernel name and shape.
 MEASURED_TRAFFIC_BYTES = {
-    ("smfmac16x16x64_warpspec_densestage_tile256x128_3stage_8consumers", 4096, 1024, 16384, 8, 64): 225_088_000,
+    ("smfmac16x16x64_warpspec_densestage_tile256x128_3stage_8consumers", 4096, 1024, 16384, 8, 64): 194_615_000,
 }
 
 

@@ -100,16 +100,30 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
             if (variant_ok(plan, N, order[i], fused)) return order[i];
         return -1;
     }
+    // Dense-staged 256 x 128 tiles: with at most 768 of them the two-phase-group form leads the eight-consumer form by
+    // 2-5 % (BERT-base / BERT-large layer shapes at N = 2048 .. 8192), beyond that it falls behind; it has no fused
+    // write-out and is measured for row-major output only.
+    const int64_t ds_tiles = (int64_t)(plan->geo.rows / 256) * ((N + 127) / 128);
+    const int ds_variant = (ds_tiles <= 768 && !fused && out_layout == SPATHA_OUT_ROW_MAJOR &&
+                            variant_ok(plan, N, SPMM_VARIANT_DS256x128_S3_PP, fused))
+                               ? SPMM_VARIANT_DS256x128_S3_PP
+                               : SPMM_VARIANT_DS256x128_S3_C8;
     if (v % 128 == 0) {
         const int64_t wide_tiles = (int64_t)(plan->geo.rows / 128) * ((N + 255) / 256);
         order[0] = wide_tiles >= 512 ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x128_S3;
         order[1] = SPMM_VARIANT_W128x128_S3;
-        // measured on the BERT-large shapes (N = 16384): plain 2:4 runs 6-8 % faster with dense-staged 256 x 128
-        // tiles, m >= 16 3-5 % faster with two 128 x 128 workgroups per CU (two stages each)
-        if (wide_tiles >= 512 && plan->geo.m <= 4) order[0] = SPMM_VARIANT_DS256x128_S3_C8;
-        if (wide_tiles >= 512 && plan->geo.m >= 16 && plan->S <= 16) {      // (long k-loops: the tall tile stays ahead)
+        // measured on the BERT-large shapes (N = 16384): m >= 16 runs 3-5 % faster with two 128 x 128 workgroups per CU
+        // (two stages each); with fewer tiles (N <= 8192) the tall tile leads by up to 30 %
+        if (wide_tiles >= 2048 && plan->geo.m >= 16 && plan->S <= 16) {      // (long k-loops: the tall tile stays ahead)
             order[1] = order[0];
             order[0] = SPMM_VARIANT_W128x128_S2;
+        }
+        // m <= 8: dense staging leads the gathered tiles by 5-35 % as soon as its 256 x 128 tiles fill three quarters of
+        // the CUs (BERT layer shapes, N = 2048 .. 16384); with fewer tiles the 128 x 128 tile's finer split wins
+        if (plan->geo.m <= 8 && plan->geo.rows % 256 == 0 && ds_tiles >= 192 && plan->S <= 64 &&
+            out_layout == SPATHA_OUT_ROW_MAJOR) {
+            order[1] = order[0];
+            order[0] = ds_variant;
         }
         if (out_layout == SPATHA_OUT_TRANSPOSED) {
             // measured with transposed output + bias on the BERT-large layer shapes (N = 16384): the kernels that write
@@ -133,11 +147,15 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         order[3] = SPMM_VARIANT_128x128;
     } else if (v % 64 == 0) {
         // m <= 8: staging the dense B rows once for four 64-row blocks halves the L2 -> LDS traffic
-        order[0] = SPMM_VARIANT_DS256x128_S3_C8;
-        // m > 8: gathered 64 x 256 tiles; with many k-steps per tile the persistent pipeline (which keeps loading
-        // across tile boundaries) is 1.6x faster than the per-tile one, with few it is a few percent slower
-        const bool long_k = plan->S >= 24;
-        const bool ws_short = plan->geo.m >= 32 && out_layout != SPATHA_OUT_TRANSPOSED;   // transposed: the pipeline leads by 6-8 %
+        order[0] = ds_variant;
+        // m > 8: gathered 64 x 256 tiles.  Per-tile pipeline with two stages (two workgroups per CU) unless there is
+        // work for many rounds: then, with many k-steps per tile, the persistent pipeline (which keeps loading across
+        // tile boundaries) is 1.6x faster, and for m >= 32 with row-major output the producer/consumer kernel leads by
+        // 5-10 % (transposed: the pipeline leads by 6-8 %).  With one tile per CU or less the persistent kernel's third
+        // stage still gives long k-loops 5-15 %.
+        const int64_t tiles = (int64_t)(plan->geo.rows / 64) * ((N + 255) / 256);
+        const bool long_k = plan->S >= 24 && (tiles >= 2048 || tiles <= 256);
+        const bool ws_short = plan->geo.m >= 32 && out_layout != SPATHA_OUT_TRANSPOSED && tiles >= 2048;
         order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : (ws_short ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_P64x256_S2);
         order[2] = long_k ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_R64x256_S3;
         order[3] = SPMM_VARIANT_64x256;

@@ -157,3 +157,31 @@ def test_out_32b_ablation_build_computes_the_same_numbers(gpu):
                        env=dict(os.environ, SPATHA_LIBRARY=alt), stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
                        timeout=300)
     assert r.returncode == 0 and "smoke ok" in r.stdout, r.stderr[-2000:]
+
+
+def test_sweep_script_issues_the_reference_command_lines():
+    """run_spmm_spatha builds, per point, the command line of benchmark/run_spmm_spatha.sh:135 (with --check)."""
+    from venom_amd import run_spmm_spatha as sweep
+    cmd = sweep.command(4096, 1024, 8192, 64, 7)
+    assert cmd[0] == BENCH
+    for flag, value in (("--sparsity-type", "n-to-m"), ("--spmm", "spatha"), ("--gemm", "cuBlas"), ("--precision", "half"),
+                        ("--meta-block-size", "32"), ("--block-size", "4"), ("--nn_row", "2"), ("--mm_row", "7"),
+                        ("--m", "4096"), ("--k", "1024"), ("--n", "8192"), ("--bm", "64")):
+        assert cmd[cmd.index(flag) + 1] == value
+    assert "--check" in cmd and "--variant" not in cmd
+    assert sweep.command(64, 64, 64, 64, 4, variant=5)[-2:] == ["--variant", "5"]
+    assert sweep.HEADER.split(",")[:24] == [c if c != "mm_row" else "mm_col" for c in REFERENCE_COLUMNS]   # run_spmm_spatha.sh:8
+    assert len(sweep.HEADER.split(",")) == len(REFERENCE_COLUMNS) + len(APPENDED_COLUMNS)
+    assert (768, 3072) in sweep.LAYERS and (4096, 1024) in sweep.LAYERS and sweep.M_VALUES == [4, 7, 8, 10, 20, 40, 100]
+
+
+@pytest.mark.gpu
+def test_sweep_script_runs_and_every_point_passes_the_check(gpu, tmp_path):
+    from venom_amd import run_spmm_spatha as sweep
+    out = str(tmp_path / "sweep.csv")
+    assert sweep.main(["--out", out, "--tokens", "2048", "--v", "64,128", "--m", "7,20"]) == 0
+    lines = open(out).read().splitlines()
+    assert lines[0] == sweep.HEADER and len(lines) == 1 + 2 * 2 * len(sweep.LAYERS)
+    for ln in lines[1:]:
+        row = dict(zip(sweep.HEADER.split(","), ln.split(",")))
+        assert row["error"] == "0" and row["arch"] == "gfx950" and float(row["spmm_time"]) > 0

@@ -185,3 +185,26 @@ def test_sweep_script_runs_and_every_point_passes_the_check(gpu, tmp_path):
     for ln in lines[1:]:
         row = dict(zip(sweep.HEADER.split(","), ln.split(",")))
         assert row["error"] == "0" and row["arch"] == "gfx950" and float(row["spmm_time"]) > 0
+
+
+def test_ablation_script_covers_the_reference_points():
+    """run_ablation: the shapes of benchmark/run_ablation1.sh:12-28 (V = 128, M in 10, 20, 40, 100) and of
+    run_ablation2.sh:8 (V in 32, 64, 128; M in 7 .. 100), rows under the reference's header."""
+    from venom_amd import run_ablation as ab
+    p1, p2 = ab.points(1), ab.points(2)
+    assert len(p1) == 16 * 4 and {p[1] for p in p1} == {768 * i for i in range(1, 17)} and {p[3] for p in p1} == {128}
+    assert len(p2) == 18 and {p[:3] for p in p2} == {(1024, 4096, 4096)} and {p[3] for p in p2} == {32, 64, 128}
+    assert ab.points(2, limit=2) == p2[:2]
+    assert ab.HEADER.split(",")[:24] == REFERENCE_COLUMNS
+    row = ab.csv_row(4, {"rows": 1024, "cols": 4096, "N": 4096, "m": 8, "v": 64, "ms": 0.025, "kernel": "k"}, 0).split(",")
+    assert len(row) == len(ab.HEADER.split(",")) and row[0] == "4" and row[8] == "8" and row[10] == "64" and row[23] == "0"
+
+
+@pytest.mark.gpu
+def test_ablation_script_runs_both_builds_and_they_agree(gpu, tmp_path):
+    from venom_amd import run_ablation as ab
+    assert ab.main(["--which", "2", "--limit", "3", "--out-dir", str(tmp_path)]) == 0
+    lines = open(str(tmp_path / "ablation2.csv")).read().splitlines()
+    assert lines[0] == ab.HEADER and len(lines) == 1 + 2 * 3
+    assert [ln.split(",")[0] for ln in lines[1:]] == ["2"] * 3 + ["4"] * 3
+    assert all(ln.split(",")[23] == "0" for ln in lines[1:])

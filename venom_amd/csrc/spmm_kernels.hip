@@ -1881,11 +1881,19 @@ constexpr int TR_PITCH = 40;                       // 16 rows x 2 B + 8 B pad
 constexpr int TR_SLAB_BYTES = 64 * TR_PITCH;       // per wave, all 16 slab rows at once
 constexpr int TR8_PITCH = 16;                      // 8 rows x 2 B
 constexpr int TR8_SLAB_BYTES = 64 * TR8_PITCH;     // per wave, 8 slab rows at a time (ROWS8: half the lanes write)
-template <bool ROWS8>
+// BIAS_VIA_SLAB (needs ROWS8 and 128 spare bytes behind the slab): the block's 64 bias values are fetched once, ahead of
+// the first store, and the phases read them from LDS; a bias load inside a phase would make that phase wait on the
+// vector-memory counter, i.e. for every store issued so far.
+template <bool ROWS8, bool BIAS_VIA_SLAB = false>
 __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4][4], char* stg, uint16_t* C, int64_t row0,
                                                          int col0, int N, int lane, bool stores_on,
                                                          const uint16_t* bias = nullptr) {
+    static_assert(!BIAS_VIA_SLAB || ROWS8, "the spare bytes sit behind the 8-row slab");
     constexpr int PITCH = ROWS8 ? TR8_PITCH : TR_PITCH;
+    if (BIAS_VIA_SLAB && bias) {
+        if (lane < 32) *(uint32_t*)(stg + TR8_SLAB_BYTES + lane * 4) = *(const uint32_t*)(bias + row0 + lane * 2);
+        __builtin_amdgcn_wave_barrier();
+    }
     const int j16 = lane & 15, ib = lane >> 4;     // as accumulator lane: column j16, rows 4*ib + r
     const int li = lane & 15, kb = lane >> 4;
     // as chunk supplier: source row e = li/4, chunk k = li%4
@@ -1909,7 +1917,8 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
 #pragma unroll
                 for (int r = 0; r < 4; r++) h4[nb][r] = (_Float16)acc[mb][nb][r];
             if (bias) {          // fp16 addition on the rounded product, rows row0 + 16*ib + 4*mb + r
-                const half4_t bv = *(const half4_t*)(bias + row0 + 16 * ib + 4 * mb);
+                const half4_t bv = BIAS_VIA_SLAB ? *(const half4_t*)(stg + TR8_SLAB_BYTES + (16 * ib + 4 * mb) * 2)
+                                                 : *(const half4_t*)(bias + row0 + 16 * ib + 4 * mb);
 #pragma unroll
                 for (int nb = 0; nb < 4; nb++) h4[nb] = h4[nb] + bv;
             }
@@ -1967,6 +1976,7 @@ struct DsCfg {
     static constexpr int STAGE_BYTES = B_BYTES + 4 * APACK_BLOCK;
     static constexpr int PA = NS - 1;
     static constexpr int SLAB_BYTES = NC == 4 ? TR_SLAB_BYTES : (TR8_SLAB_BYTES > TT_SLAB_BYTES ? TR8_SLAB_BYTES : TT_SLAB_BYTES);
+    static_assert(NC == 4 || SLAB_BYTES >= TR8_SLAB_BYTES + 128, "room for the block's bias values behind the 8-row slab");
     static constexpr int EPI_BYTES = NC * SLAB_BYTES;
     static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
     static constexpr int LDS_BYTES = NS * STAGE_BYTES + EPI_BYTES;
@@ -2099,8 +2109,10 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
                 ns = 0;
                 if (c_tile + 1 < walk.my_tiles) walk.next(n_tm, n_tn);
             }
+            if (!SPATHA_KNOB(32) || ns == 0) {      // (development knob 32: table entries only ahead of a tile's stores)
 #pragma unroll
-            for (int h = 0; h < H; h++) g_next[h] = *gtab_ptr(n_tm, h, ns);
+                for (int h = 0; h < H; h++) g_next[h] = *gtab_ptr(n_tm, h, ns);
+            }
             SPATHA_PROF_MARK(0)
             __syncthreads();
             SPATHA_PROF_MARK(1)
@@ -2163,9 +2175,14 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
                     store_block_transposed_slab<true>(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C, p.fuse ? nullptr : p.bias,
                                                 (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !SPATHA_KNOB(2));
             } else if (!SPATHA_KNOB(4)) {
-                store_block_row_major_tr<Cfg::NC == 8>(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C,
-                                                        (int64_t)cm0 + h * 64, cn0 + wn * 64, N, lane, !SPATHA_KNOB(2),
-                                                        (p.fuse && !pre) ? p.bias : nullptr);
+                // two copies, so that the plain path carries nothing of the bias path
+                if (p.fuse && !pre && p.bias)
+                    store_block_row_major_tr<Cfg::NC == 8, Cfg::NC == 8>(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C,
+                                                                         (int64_t)cm0 + h * 64, cn0 + wn * 64, N, lane,
+                                                                         !SPATHA_KNOB(2), p.bias);
+                else
+                    store_block_row_major_tr<Cfg::NC == 8>(acc[h], smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES, p.C,
+                                                           (int64_t)cm0 + h * 64, cn0 + wn * 64, N, lane, !SPATHA_KNOB(2), nullptr);
             }
         }
         SPATHA_PROF_MARK(2)

@@ -119,8 +119,9 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
             order[0] = SPMM_VARIANT_W128x128_S2;
         }
         // m <= 8: dense staging leads the gathered tiles by 5-35 % as soon as its 256 x 128 tiles fill three quarters of
-        // the CUs (BERT layer shapes, N = 2048 .. 16384); with fewer tiles the 128 x 128 tile's finer split wins
-        if (plan->geo.m <= 8 && plan->geo.rows % 256 == 0 && ds_tiles >= 192 && plan->S <= 64 &&
+        // the CUs (BERT layer shapes, N = 2048 .. 16384; from 160 tiles on the GPT-2-large ones); with fewer tiles the 128 x 128
+        // tile's finer split wins
+        if (plan->geo.m <= 8 && plan->geo.rows % 256 == 0 && ds_tiles >= 160 && plan->S <= 64 &&
             out_layout == SPATHA_OUT_ROW_MAJOR) {
             order[1] = order[0];
             order[0] = ds_variant;
@@ -129,33 +130,35 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
             // measured with transposed output + bias on the BERT-large layer shapes (N = 16384): the kernels that write
             // through the 8-column slab (dense-staged, tall) lead by 10-25 % once there is enough work per tile column
             if (plan->geo.m <= 8) {
-                // short k-loops only: with many k-steps per tile the gathered 128 x 256 tile moves fewer bytes per
-                // output element (GPT-3 block at 128:2:8: 6.95 ms against 8.26 ms with dense staging)
-                if (plan->S <= 16) {
+                // not for long k-loops: with many k-steps per tile the gathered 128 x 256 tile moves fewer bytes per
+                // output element (GPT-3 block at 128:2:8, 96 k-steps: 6.95 ms against 8.26 ms with dense staging; GPT-2-large
+                // FFN-down, 40 k-steps: dense staging 20 % ahead)
+                if (plan->S <= 40) {
                     order[1] = order[0];
                     order[0] = SPMM_VARIANT_DS256x128_S3_C8;
                 }
-            } else if (wide_tiles >= 1024 || plan->S >= 8) {
-                order[0] = SPMM_VARIANT_T128x256_S3;
-                order[1] = SPMM_VARIANT_W128x128_S3;
             } else {
-                order[0] = SPMM_VARIANT_W128x128_S3;
+                // m >= 16: the producer/consumer kernel on 128 x 256 tiles (64 x 64 consumer blocks) leads the tall tile
+                // and the 128 x 128 tile by 5-15 % on the BERT-large and GPT-2-large layer shapes (N = 4096, 16384)
+                order[0] = SPMM_VARIANT_W128x256_S3;
                 order[1] = SPMM_VARIANT_T128x256_S3;
+                order[2] = SPMM_VARIANT_W128x128_S3;
             }
         }
-        order[2] = SPMM_VARIANT_P128x128_S3;
+        if (order[2] == 0) order[2] = SPMM_VARIANT_P128x128_S3;
         order[3] = SPMM_VARIANT_128x128;
     } else if (v % 64 == 0) {
         // m <= 8: staging the dense B rows once for four 64-row blocks halves the L2 -> LDS traffic
         order[0] = ds_variant;
         // m > 8: gathered 64 x 256 tiles.  Per-tile pipeline with two stages (two workgroups per CU) unless there is
-        // work for many rounds: then, with many k-steps per tile, the persistent pipeline (which keeps loading across
-        // tile boundaries) is 1.6x faster, and for m >= 32 with row-major output the producer/consumer kernel leads by
+        // work for many rounds: then, with 32 or more k-steps per tile, the persistent pipeline (which keeps loading
+        // across tile boundaries) leads (GPT-3 layers at 64:2:16; at 64:2:32, 24 k-steps, the per-tile pipeline is
+        // 10-20 % ahead), and for m >= 32 with few k-steps and row-major output the producer/consumer kernel leads by
         // 5-10 % (transposed: the pipeline leads by 6-8 %).  With one tile per CU or less the persistent kernel's third
         // stage still gives long k-loops 5-15 %.
         const int64_t tiles = (int64_t)(plan->geo.rows / 64) * ((N + 255) / 256);
-        const bool long_k = plan->S >= 24 && (tiles >= 2048 || tiles <= 256);
-        const bool ws_short = plan->geo.m >= 32 && out_layout != SPATHA_OUT_TRANSPOSED && tiles >= 2048;
+        const bool long_k = plan->S >= 32 && (tiles >= 2048 || tiles <= 256);
+        const bool ws_short = plan->geo.m >= 32 && out_layout != SPATHA_OUT_TRANSPOSED && tiles >= 2048 && plan->S <= 8;
         order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : (ws_short ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_P64x256_S2);
         order[2] = long_k ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_R64x256_S3;
         order[3] = SPMM_VARIANT_64x256;

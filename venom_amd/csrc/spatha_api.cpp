@@ -110,13 +110,20 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
                                : SPMM_VARIANT_DS256x128_S3_C8;
     if (v % 128 == 0) {
         const int64_t wide_tiles = (int64_t)(plan->geo.rows / 128) * ((N + 255) / 256);
-        order[0] = wide_tiles >= 512 ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x128_S3;
-        order[1] = SPMM_VARIANT_W128x128_S3;
-        // measured on the BERT-large shapes (N = 16384): m >= 16 runs 3-5 % faster with two 128 x 128 workgroups per CU
-        // (two stages each); with fewer tiles (N <= 8192) the tall tile leads by up to 30 %
-        if (wide_tiles >= 2048 && plan->geo.m >= 16 && plan->S <= 16) {      // (long k-loops: the tall tile stays ahead)
-            order[1] = order[0];
-            order[0] = SPMM_VARIANT_W128x128_S2;
+        // 128 x 256 tiles once there is work for two rounds of them, or for four with few k-steps per tile (measured on
+        // the BERT-large layer shapes, N = 16384: 1024 x 1024 at 128:2:16, 512 wide tiles of 4 k-steps, runs 19 % faster on
+        // 128 x 128 tiles; 1024 x 4096, 512 tiles of 16 k-steps, 3 % slower).  m >= 16: the producer/consumer kernel with
+        // 64 x 64 consumer blocks leads the tall-consumer form by 1-13 % up to 16 k-steps per tile (BERT-large, GPT-2-large
+        // layers) and trails it by 1-3 % on long k-loops (GPT-3 layers).
+        const bool wide = wide_tiles >= 512 && (wide_tiles >= 1024 || plan->S >= 8);
+        const bool ws_wide = plan->geo.m >= 16 && plan->S <= 16;
+        if (wide) {
+            order[0] = ws_wide ? SPMM_VARIANT_W128x256_S3 : SPMM_VARIANT_T128x256_S3;
+            order[1] = ws_wide ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x256_S3;
+            order[2] = SPMM_VARIANT_W128x128_S3;
+        } else {
+            order[0] = SPMM_VARIANT_W128x128_S3;
+            order[1] = SPMM_VARIANT_P128x128_S3;
         }
         // m <= 8: dense staging leads the gathered tiles by 5-35 % as soon as its 256 x 128 tiles fill three quarters of
         // the CUs (BERT layer shapes, N = 2048 .. 16384; from 160 tiles on the GPT-2-large ones); with fewer tiles the 128 x 128
@@ -138,10 +145,10 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
                     order[0] = SPMM_VARIANT_DS256x128_S3_C8;
                 }
             } else {
-                // m >= 16: the producer/consumer kernel on 128 x 256 tiles (64 x 64 consumer blocks) leads the tall tile
-                // and the 128 x 128 tile by 5-15 % on the BERT-large and GPT-2-large layer shapes (N = 4096, 16384)
-                order[0] = SPMM_VARIANT_W128x256_S3;
-                order[1] = SPMM_VARIANT_T128x256_S3;
+                // m >= 16: 128 x 256 tiles at any tile count (5-15 % ahead of 128 x 128 on the BERT-large and GPT-2-large
+                // layer shapes, N = 4096 and 16384)
+                order[0] = ws_wide ? SPMM_VARIANT_W128x256_S3 : SPMM_VARIANT_T128x256_S3;
+                order[1] = ws_wide ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x256_S3;
                 order[2] = SPMM_VARIANT_W128x128_S3;
             }
         }

@@ -1949,6 +1949,108 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
     __builtin_amdgcn_wave_barrier();
 }
 
+// The same two write-outs with four slabs per wave (stg: 4 slabs, then 128 bytes for the block's bias values): four
+// phases' LDS writes and transposing / row reads are in flight before the first store waits for its data, so a 64 x 64
+// block costs two LDS round trips instead of eight.
+template <bool WITH_BIAS>
+__device__ __forceinline__ void store_block_row_major_tr4(const float4_t (&acc)[4][4], char* stg, uint16_t* C, int64_t row0,
+                                                          int col0, int N, int lane, bool stores_on, const uint16_t* bias) {
+    constexpr int PITCH = TR8_PITCH, SLAB = TR8_SLAB_BYTES;
+    const int j16 = lane & 15, ib = lane >> 4;
+    const int li = lane & 15, kb = lane >> 4;
+    const int rd_off = (8 * (2 * kb + ((li & 3) >> 1)) + (li >> 2)) * PITCH + (li & 1) * 8;
+    const int q_lo = 4 * ((li >> 2) & 1) + (li & 3);
+    const int out_col = col0 + 8 * (2 * kb + (li >> 3));
+    const bool live = out_col < N && stores_on;
+    char* bias_lds = stg + 4 * TT_SLAB_BYTES;
+    if (WITH_BIAS) {
+        if (lane < 32) *(uint32_t*)(bias_lds + lane * 4) = *(const uint32_t*)(bias + row0 + lane * 2);
+        __builtin_amdgcn_wave_barrier();
+    }
+#pragma unroll
+    for (int grp = 0; grp < 2; grp++) {
+#pragma unroll
+        for (int mb2 = 0; mb2 < 2; mb2++) {
+            const int mb = grp * 2 + mb2;
+            half4_t h4[4];
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) h4[nb][r] = (_Float16)acc[mb][nb][r];
+            if (WITH_BIAS) {     // fp16 addition on the rounded product, rows row0 + 16*ib + 4*mb + r
+                const half4_t bv = *(const half4_t*)(bias_lds + (16 * ib + 4 * mb) * 2);
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++) h4[nb] = h4[nb] + bv;
+            }
+            // slab 2*mb2 + sidx takes the rows of lane groups ib = 2*sidx, 2*sidx + 1
+            char* slab = stg + (mb2 * 2 + (ib >> 1)) * SLAB;
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++) *(half4_t*)(slab + (nb * 16 + j16) * PITCH + (ib & 1) * 8) = h4[nb];
+        }
+        __builtin_amdgcn_wave_barrier();
+        short4_t lo[4], hi[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            lo[k] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + k * SLAB + rd_off));
+            hi[k] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + k * SLAB + rd_off + 4 * PITCH));
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int mb = grp * 2 + (k >> 1), sidx = k & 1;
+            const int q = 8 * sidx + q_lo;
+            const int row = 16 * (q >> 2) + 4 * mb + (q & 3);
+            u32x4 v;
+            v.x = (uint32_t)(uint16_t)lo[k][0] | ((uint32_t)(uint16_t)lo[k][1] << 16);
+            v.y = (uint32_t)(uint16_t)lo[k][2] | ((uint32_t)(uint16_t)lo[k][3] << 16);
+            v.z = (uint32_t)(uint16_t)hi[k][0] | ((uint32_t)(uint16_t)hi[k][1] << 16);
+            v.w = (uint32_t)(uint16_t)hi[k][2] | ((uint32_t)(uint16_t)hi[k][3] << 16);
+            if (live) store_c16<true>(C + (row0 + row) * N + out_col, v);
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+}
+
+__device__ __forceinline__ void store_block_transposed_slab4(const float4_t (&acc)[4][4], char* stg, uint16_t* C,
+                                                             const uint16_t* bias, int64_t row0, int col0, int rows_total, int N,
+                                                             int lane, bool stores_on) {
+    const int j16 = lane & 15, ib = lane >> 4;     // as accumulator lane: column j16 of a 16-column block, rows 16*ib + 4*mb + r
+    const int rn = lane >> 3, rc = lane & 7;       // as reader: slab column rn, 16-byte chunk rc (rows 8*rc .. 8*rc + 7)
+    half4_t b4[4];
+    if (bias) {
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) b4[mb] = *(const half4_t*)(bias + row0 + 16 * ib + 4 * mb);
+    }
+#pragma unroll
+    for (int grp = 0; grp < 2; grp++) {
+#pragma unroll
+        for (int nb2 = 0; nb2 < 2; nb2++) {
+            const int nb = grp * 2 + nb2;
+            // slab 2*nb2 + hf takes the columns j16 = 8*hf .. 8*hf + 7 of block nb
+            char* slab = stg + (nb2 * 2 + (j16 >> 3)) * TT_SLAB_BYTES;
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) {
+                half4_t h4;
+#pragma unroll
+                for (int r = 0; r < 4; r++) h4[r] = (_Float16)acc[mb][nb][r];
+                if (bias) h4 = h4 + b4[mb];
+                *(half4_t*)(slab + (j16 & 7) * TT_PITCH + (16 * ib + 4 * mb) * 2) = h4;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        u32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = *(const u32x4*)(stg + k * TT_SLAB_BYTES + rn * TT_PITCH + rc * 16);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int col = col0 + (grp * 2 + (k >> 1)) * 16 + (k & 1) * 8 + rn;
+            if (col < N && stores_on) store_c16<true>(C + (int64_t)col * rows_total + row0 + rc * 8, v[k]);
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+}
+
 // ---------------------------------------------------------------------------
 // Dense-staged kernel for m <= 8 (tile 256 x 128 = four 64-row blocks; pays off most at V = 64).
 //
@@ -1964,8 +2066,13 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
 // 64*(w%2) .. +63; with eight, rows 64*(w/2) .. +63 (two waves per SIMD hide each other's LDS
 // latency and barrier waits).  Producers need no row table: B rows are consecutive.
 // ---------------------------------------------------------------------------
-template <int M, int NS, int NP, int NC_>
+// STAGE_EPI: the consumers write a tile out through the memory of the stage they consumed last (a workgroup barrier at
+// the end of every tile, which the producers join, makes it theirs until the next step barrier): room for four slabs
+// per wave, so that a 64 x 64 block leaves in two LDS round trips instead of eight.
+constexpr int WAVE_EPI_BYTES = 4 * TT_SLAB_BYTES + 128;      // four slabs of the larger kind + the block's bias values
+template <int M, int NS, int NP, int NC_, bool STAGE_EPI_ = false>
 struct DsCfg {
+    static constexpr bool STAGE_EPI = STAGE_EPI_;
     static constexpr int NC = NC_;                 // consumer waves: 4 (128 x 64 each) or 8 (64 x 64 each)
     static constexpr int H = 8 / NC;               // 64-row blocks per consumer wave
     static_assert(NC == 4 || NC == 8, "consumer waves");
@@ -1981,6 +2088,7 @@ struct DsCfg {
     static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
     static constexpr int LDS_BYTES = NS * STAGE_BYTES + EPI_BYTES;
     static constexpr int THREADS = (NC + NP) * 64;
+    static_assert(!STAGE_EPI || (NC == 8 && NC * WAVE_EPI_BYTES <= STAGE_BYTES), "the write-out slabs must fit one stage");
 };
 
 template <class Cfg, int M, int NP, int PR>
@@ -2046,14 +2154,25 @@ __device__ __forceinline__ void ds_producer(const SpmmParams& p, const TileWalk&
     for (int t = 0; t < PA; t++)
         if (t < Q) issue_batch();
     const int q_main = Q - PA > 0 ? Q - PA : 0;
+    // STAGE_EPI: the barrier the consumers hold after the last step of every tile, before they take that step's stage
+    // for their write-out (the refill of that stage is issued after the NEXT step barrier, which they reach afterwards)
+    int bar_step = 0;
+    auto tile_end_barrier = [&]() {
+        if (Cfg::STAGE_EPI && ++bar_step == S) {
+            bar_step = 0;
+            __syncthreads();
+        }
+    };
     for (int q = 0; q < q_main; q++) {
         wait_vmcnt<(PA - 1) * LOADS>();
         __syncthreads();
         if (!SPATHA_KNOB(8)) issue_batch();
+        tile_end_barrier();
     }
     for (int q = q_main; q < Q; q++) {
         wait_stages<LOADS, PA - 1>(Q - 1 - q);
         __syncthreads();
+        tile_end_barrier();
     }
 }
 
@@ -2082,7 +2201,7 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
     int c_tm = walk.tm0, c_tn = walk.tn0;
     int n_tm = c_tm, n_tn = c_tn;       // tile of the NEXT step's table entries
     SPATHA_PROF_DECL
-    uint32_t c_stage = 0;
+    uint32_t c_stage = 0, epi_stage = 0;
     u32x2 g_next[H];
     // LDS offsets of this step's four fragments (per 64-row block): computed at the end of the previous step,
     // behind its matrix instructions, so that the first reads can issue right after the barrier
@@ -2159,12 +2278,29 @@ __device__ __forceinline__ void ds_consumer(const SpmmParams& p, const TileWalk&
 #undef SPATHA_MMA4H
                 }
             }
+            epi_stage = c_stage;
             c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
 #pragma unroll
             for (int h = 0; h < H; h++) set_base(h, g_next[h]);
         }
         const int cm0 = c_tm * BM + rb0 * 64, cn0 = c_tn * BN;
         SPATHA_PROF_MARK(0)
+        if constexpr (Cfg::STAGE_EPI) {
+            __syncthreads();            // every consumer is done with the last stage: it is the write-out's until the next step barrier
+            SPATHA_PROF_MARK(1)
+            char* stg = smem + epi_stage + wave * WAVE_EPI_BYTES;
+            const bool pre = p.fuse && (p.act != SPATHA_ACT_NONE || OUT_LAYOUT == SPATHA_OUT_TRANSPOSED);
+            if (pre) fused_bias_act(acc[0], p.bias, (int64_t)cm0 + ib * 16, p.act);
+            if (!SPATHA_KNOB(4)) {
+                if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
+                    store_block_transposed_slab4(acc[0], stg, p.C, p.fuse ? nullptr : p.bias, (int64_t)cm0, cn0 + wn * 64, p.rows, N,
+                                                 lane, !SPATHA_KNOB(2));
+                else if (p.fuse && !pre && p.bias)
+                    store_block_row_major_tr4<true>(acc[0], stg, p.C, (int64_t)cm0, cn0 + wn * 64, N, lane, !SPATHA_KNOB(2), p.bias);
+                else
+                    store_block_row_major_tr4<false>(acc[0], stg, p.C, (int64_t)cm0, cn0 + wn * 64, N, lane, !SPATHA_KNOB(2), nullptr);
+            }
+        } else
 #pragma unroll
         for (int h = 0; h < H; h++) {
             // a bias alone rides in the row-major write-out itself (packed fp16 additions); anything else goes first
@@ -2545,7 +2681,7 @@ __global__ __launch_bounds__((8 + NP) * 64) void spmm_dspp_kernel(SpmmParams p) 
 
 template <int M, int NS, int NP, int NC, int OUT_LAYOUT, bool HALF = false>
 __global__ __launch_bounds__((NC + NP) * 64) void spmm_ds_kernel(SpmmParams p) {
-    using Cfg = DsCfg<M, NS, NP, NC>;
+    using Cfg = DsCfg<M, NS, NP, NC, (NC == 8 && !HALF)>;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
     const int tid = threadIdx.x, lane = tid & 63;

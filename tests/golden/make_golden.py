@@ -11,7 +11,7 @@ convention of the reference, not something mathematics fixes, and the selector's
 choice among equal-magnitude candidates depends on the persistent permutation
 state of its std::partial_sort calls.  Neither can be pinned by an invariant.
 
-Usage:  cd _work/golden_cache && python ../../tests/golden/make_golden.py
+Usage:  cd <an empty scratch directory> && python <repository>/tests/golden/make_golden.py
 (the reference JIT-compiles its embedded C++ into ./.compile_cache of the cwd).
 """
 import os

@@ -210,6 +210,16 @@ int spatha_dense_gemm_f16(const uint16_t* A_dev, const uint16_t* B_dev, int rows
  * (end2end/bert_pytorch.py:85-87, called from SrnmSpmm.forward :126-136). */
 int spatha_transpose_f16(const uint16_t* in_dev, int rows, int cols, uint16_t* out_dev, void* stream);
 
+/* out[tokens x hidden] = LayerNorm(x + residual) over the last dimension, fp16 in and out, fp32 arithmetic
+ * (the sum is rounded to fp16 first, as the separate addition would; biased variance; gamma, beta of length hidden).
+ * residual_dev may be NULL (plain layer norm).  hidden % 8 == 0 and hidden <= 4096 (SPATHA_ERR_UNSUPPORTED beyond);
+ * all pointers 16-byte aligned; out may alias x or residual.
+ * One kernel for the `LayerNorm(dropout(dense(h)) + input)` tail of the stock BertSelfOutput / BertOutput modules
+ * that the reference's harness runs after its attention-output and FFN-down SpMMs (the model of
+ * end2end/bert_pytorch.py:170-171; the SpMM layers it swaps in are :108-167). */
+int spatha_add_layernorm_f16(const uint16_t* x_dev, const uint16_t* residual_dev, const uint16_t* gamma_dev,
+                             const uint16_t* beta_dev, float eps, int tokens, int hidden, uint16_t* out_dev, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -205,3 +205,67 @@ def test_merged_qkv_projection_gives_the_same_bits(gpu):
     for got, layer in ((q, plain.encoder.layer[0].attention.self.query), (k, plain.encoder.layer[0].attention.self.key),
                        (v, plain.encoder.layer[0].attention.self.value)):
         assert torch.equal(got, layer(x))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tokens,hidden,with_residual", [(16384, 1024, True), (300, 1024, False), (64, 1280, True),
+                                                          (7, 4096, True), (5, 8, True), (33, 72, False)])
+def test_add_layernorm_matches_torch_addition_and_layer_norm(gpu, tokens, hidden, with_residual):
+    """One kernel against the two it replaces.  The sum is rounded to fp16 in both; the statistics are accumulated in a
+    different order (per-lane partial sums here, Welford there), so the fp32 results differ in the last bits and a few
+    outputs land on the neighbouring fp16 value: at least 99 % equal, none more than one fp16 step apart
+    (relative 2^-10) or, near zero, 1e-3 absolute."""
+    from venom_amd import spatha
+
+    g = torch.Generator(device=gpu)
+    g.manual_seed(tokens * 31 + hidden)
+    x = (torch.randn((tokens, hidden), generator=g, device=gpu) * 1.5 + 0.3).half()
+    r = torch.randn((tokens, hidden), generator=g, device=gpu).half() if with_residual else None
+    w = (1.0 + 0.1 * torch.randn(hidden, generator=g, device=gpu)).half()
+    b = (0.1 * torch.randn(hidden, generator=g, device=gpu)).half()
+    got = spatha.add_layernorm(x, r, w, b, 1e-12)
+    want = torch.nn.functional.layer_norm(x + r if with_residual else x, (hidden,), w, b, 1e-12)
+    assert got.shape == want.shape and got.dtype == torch.float16
+    assert (got == want).float().mean().item() >= 0.99
+    diff = (got.float() - want.float()).abs()
+    assert bool((diff <= torch.maximum(want.float().abs() * 2.0 ** -10, torch.tensor(1e-3, device=gpu))).all())
+    # a 3-d activation is taken as [tokens, hidden] rows
+    if tokens % 4 == 0:
+        got3 = spatha.add_layernorm(x.view(4, tokens // 4, hidden), None if r is None else r.view(4, tokens // 4, hidden), w, b, 1e-12)
+        assert torch.equal(got3.view(tokens, hidden), got)
+
+
+@pytest.mark.gpu
+def test_add_layernorm_rejects_what_the_kernel_does_not_take(gpu):
+    from venom_amd import _lib, spatha
+
+    x = torch.zeros((4, 12), device=gpu).half()           # hidden not a multiple of 8
+    w = torch.ones(12, device=gpu).half()
+    with pytest.raises(_lib.SpathaError):
+        spatha.add_layernorm(x, None, w, w, 1e-5)
+    x = torch.zeros((2, 8192), device=gpu).half()         # more than a lane's registers hold
+    w = torch.ones(8192, device=gpu).half()
+    with pytest.raises(_lib.SpathaError):
+        spatha.add_layernorm(x, None, w, w, 1e-5)
+    with pytest.raises(ValueError):
+        spatha.add_layernorm(torch.zeros((2, 16), device=gpu).half(), torch.zeros((2, 8), device=gpu).half(),
+                             torch.ones(16, device=gpu).half(), torch.ones(16, device=gpu).half(), 1e-5)
+
+
+@pytest.mark.gpu
+def test_fused_projection_norm_tracks_the_stock_modules(gpu):
+    from venom_amd.bert import FusedProjectionNorm, build_bert_large, fuse_add_layernorm, linear_to_spmm
+
+    torch.set_grad_enabled(False)
+    torch.manual_seed(3)
+    stock = linear_to_spmm(build_bert_large(layers=2).to(gpu).half(), 2, 8, 64)
+    torch.manual_seed(3)
+    fused = fuse_add_layernorm(linear_to_spmm(build_bert_large(layers=2).to(gpu).half(), 2, 8, 64))
+    assert isinstance(fused.encoder.layer[0].output, FusedProjectionNorm)
+    assert isinstance(fused.encoder.layer[1].attention.output, FusedProjectionNorm)
+    ids = torch.randint(0, 30522, (2, 64), device=gpu)
+    a, b = stock(ids).last_hidden_state.float(), fused(ids).last_hidden_state.float()
+    assert (a - b).abs().max().item() <= 2e-2 and ((a - b).abs() <= 2e-3).float().mean().item() >= 0.99
+    fused.train()                                            # in training the stock sequence runs (dropout is live)
+    assert fused.encoder.layer[0].output(torch.zeros((1, 8, 4096), device=gpu).half(),
+                                         torch.zeros((1, 8, 1024), device=gpu).half()).shape == (1, 8, 1024)

@@ -211,6 +211,37 @@ def fuse_feed_forward(model, activation_in_kernel=False):
     return model
 
 
+class FusedProjectionNorm(torch.nn.Module):
+    """Stands in for transformers' BertSelfOutput / BertOutput: the projection, then LayerNorm(projection + input) as ONE
+    kernel (`spatha.add_layernorm`) instead of an addition and a normalisation.  Independent of the weight format: the
+    projection may be an nn.Linear or an SrnmSpmm.  In training, or for tensors the kernel does not take, the stock
+    sequence runs."""
+
+    def __init__(self, mod):
+        super().__init__()
+        self.dense, self.LayerNorm, self.dropout = mod.dense, mod.LayerNorm, mod.dropout
+        self.train(mod.training)
+
+    def forward(self, hidden_states, input_tensor):
+        h = self.dense(hidden_states)
+        ln = self.LayerNorm
+        if self.training or not h.is_cuda or h.dtype != torch.float16 or h.shape[-1] % 8 or h.shape[-1] > 4096 \
+                or ln.weight is None or ln.bias is None:
+            return ln(self.dropout(h) + input_tensor)
+        return spatha.add_layernorm(h.contiguous(), input_tensor.contiguous(), ln.weight, ln.bias, ln.eps)
+
+
+def fuse_add_layernorm(model):
+    """Replaces, in place, every BertSelfOutput / BertOutput by FusedProjectionNorm (same parameters)."""
+    from transformers.models.bert.modeling_bert import BertOutput, BertSelfOutput
+
+    for mod in model.modules():
+        for name, child in list(mod.named_children()):
+            if isinstance(child, (BertSelfOutput, BertOutput)):
+                setattr(mod, name, FusedProjectionNorm(child))
+    return model
+
+
 def linear_to_spmm(mod, n, m, v, magnitude=False, prefix="", only=("encoder.layer",)):
     """Replaces, in place, every nn.Linear whose qualified name contains one of `only`."""
     for name, child in list(mod.named_children()):
@@ -253,6 +284,9 @@ def main(argv=None):
                     help="first feed-forward layer of every block as one kernel (bias + GELU in the write-out, feature-major "
                          "result handed to the second layer without a transposed copy)")
     ap.add_argument("--merge-qkv", action="store_true", help="query, key and value projections of a block as one SpMM")
+    ap.add_argument("--fuse-ln", action="store_true",
+                    help="residual addition + LayerNorm after the attention-output and FFN-down projections as one kernel, "
+                         "in BOTH models (the fusion does not depend on the weight format)")
     ap.add_argument("--kernel-gelu", action="store_true",
                     help="with --fuse-ffn: GELU in the kernel's write-out too (default: torch's elementwise pass over the "
                          "feature-major buffer, which keeps the model's output bit-identical to the unfused layers)")
@@ -266,6 +300,9 @@ def main(argv=None):
         fuse_feed_forward(sparse_model, activation_in_kernel=args.kernel_gelu)
     if args.merge_qkv:
         merge_qkv(sparse_model)
+    if args.fuse_ln:
+        fuse_add_layernorm(dense_model)
+        fuse_add_layernorm(sparse_model)
     ids = torch.randint(0, 30522, (args.batch, args.seq), device=dev)
 
     def run(model):
@@ -280,7 +317,8 @@ def main(argv=None):
     t_sparse = report_time("n:m", timeit.repeat(lambda: run(sparse_model), repeat=args.repeats, number=1), 1, args.n, args.m, args.v)
     print("# dense %.2f ms, %d:%d:%d%s %.2f ms, speed-up %.2fx" % (t_dense, args.v, args.n, args.m,
                                                                     ((" (fused feed-forward%s)" % (", activation in the kernel" if args.kernel_gelu else "")) if args.fuse_ffn else "")
-                                                                    + (" (merged q/k/v)" if args.merge_qkv else ""), t_sparse,
+                                                                    + (" (merged q/k/v)" if args.merge_qkv else "")
+                                                                    + (" (fused add + LayerNorm in both)" if args.fuse_ln else ""), t_sparse,
                                                                     t_dense / t_sparse))
 
 

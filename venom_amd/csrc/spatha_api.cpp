@@ -458,4 +458,16 @@ int spatha_transpose_f16(const uint16_t* in_dev, int rows, int cols, uint16_t* o
     return e == hipSuccess ? SPATHA_OK : hip_fail(e);
 }
 
+int spatha_add_layernorm_f16(const uint16_t* x_dev, const uint16_t* residual_dev, const uint16_t* gamma_dev,
+                             const uint16_t* beta_dev, float eps, int tokens, int hidden, uint16_t* out_dev, void* stream) {
+    if (!x_dev || !gamma_dev || !beta_dev || !out_dev || tokens <= 0 || hidden <= 0) return SPATHA_ERR_BAD_ARGUMENT;
+    if (hidden % 8 != 0) return SPATHA_ERR_BAD_SHAPE;
+    if (hidden > 4096) return SPATHA_ERR_UNSUPPORTED;           // a lane keeps hidden / 64 values in registers
+    if (((uintptr_t)x_dev | (uintptr_t)residual_dev | (uintptr_t)gamma_dev | (uintptr_t)beta_dev | (uintptr_t)out_dev) & 15u)
+        return SPATHA_ERR_BAD_ARGUMENT;
+    hipError_t e = spatha::launch_add_layernorm_f16(x_dev, residual_dev, gamma_dev, beta_dev, eps, tokens, hidden, out_dev,
+                                                    (hipStream_t)stream);
+    return e == hipSuccess ? SPATHA_OK : hip_fail(e);
+}
+
 }  // extern "C"

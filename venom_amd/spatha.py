@@ -148,6 +148,30 @@ def transpose(x):
     return out
 
 
+def add_layernorm(x, residual, weight, bias, eps):
+    """LayerNorm(x + residual) over the last dimension in one kernel (residual may be None): fp16 tensors on the GPU,
+    x and residual contiguous and of the same shape, weight and bias of length x.shape[-1] (a multiple of 8, at most
+    4096).  Same arithmetic as torch's addition followed by torch.nn.functional.layer_norm on fp16 tensors."""
+    _check_dev(x, torch.float16, "x")
+    hidden = x.shape[-1]
+    if residual is not None:
+        _check_dev(residual, torch.float16, "residual")
+        if residual.shape != x.shape:
+            raise ValueError("residual must have the shape of x")
+    _check_dev(weight, torch.float16, "weight")
+    _check_dev(bias, torch.float16, "bias")
+    if weight.numel() != hidden or bias.numel() != hidden:
+        raise ValueError("weight and bias must have x.shape[-1] elements")
+    out = torch.empty_like(x)
+    if x.numel():
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.lib().spatha_add_layernorm_f16(x.data_ptr(), residual.data_ptr() if residual is not None else None,
+                                                           weight.data_ptr(), bias.data_ptr(), float(eps),
+                                                           x.numel() // hidden, hidden, out.data_ptr(), _stream_ptr(x.device)),
+                       "spatha_add_layernorm_f16")
+    return out
+
+
 def spmm(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_cols, B_num_cols, vec_length, n, m,
          nnz=0, seed=0, mbrow=32, brow=4):
     """out[B_num_cols, A_num_rows] = (A_vnm @ rhs_matrix).T + bias, fp16.

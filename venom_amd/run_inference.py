@@ -3,7 +3,7 @@ each dense and with its linear layers in V:2:M for M in {8, 16, 32} and V in {64
 (`algo,n,m,v,mean,median,std,len`; algo 0 = BERT, 1 = GPT-2, 2 = GPT-3 block) followed by one `#` summary line
 per run.
 
-    python -m venom_amd.run_inference [--repeats 10] [--models bert,gpt2,gpt3]"""
+    python -m venom_amd.run_inference [--repeats 10] [--models bert,gpt2,gpt3] [--fuse-ffn [--kernel-gelu]] [--merge-qkv] [--fuse-ln]"""
 import argparse
 
 from . import bert, gpt2, gpt3
@@ -18,6 +18,7 @@ def main(argv=None):
     ap.add_argument("--fuse-ffn", action="store_true", help="passed on to the three harnesses")
     ap.add_argument("--kernel-gelu", action="store_true", help="passed on to the three harnesses")
     ap.add_argument("--merge-qkv", action="store_true", help="passed on to the BERT harness (GPT-2's c_attn is one layer already)")
+    ap.add_argument("--fuse-ln", action="store_true", help="passed on to the BERT harness (residual addition + LayerNorm as one kernel)")
     args = ap.parse_args(argv)
     extra = (["--fuse-ffn"] if args.fuse_ffn else []) + (["--kernel-gelu"] if args.kernel_gelu else [])
     print("algo,n,m,v,mean,median,std,len", flush=True)
@@ -26,7 +27,8 @@ def main(argv=None):
         for name in args.models.split(","):
             for m in [int(x) for x in args.m.split(",")]:
                 mains[name](["-m", str(m), "-n", "2", "-v", str(v), "--repeats", str(args.repeats)] + extra +
-                            (["--merge-qkv"] if args.merge_qkv and name == "bert" else []))
+                            (["--merge-qkv"] if args.merge_qkv and name == "bert" else []) +
+                            (["--fuse-ln"] if args.fuse_ln and name == "bert" else []))
 
 
 if __name__ == "__main__":

@@ -167,6 +167,11 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         const bool long_k = plan->S >= 32 && (tiles >= 2048 || tiles <= 256);
         const bool ws_short = plan->geo.m >= 32 && out_layout != SPATHA_OUT_TRANSPOSED && tiles >= 2048 && plan->S <= 8;
         order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : (ws_short ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_P64x256_S2);
+        // 16 <= m < 32, many tiles, few k-steps, plain row-major output: the producer/consumer kernel with the write-out
+        // deferred into the next tile's steps leads the pipeline by 5-8 % (3072 / 4096 x 1024 x 16384 at 64:2:16)
+        if (!long_k && !ws_short && !fused && out_layout == SPATHA_OUT_ROW_MAJOR && plan->geo.m >= 16 && tiles >= 3072 &&
+            plan->S <= 8 && variant_ok(plan, N, SPMM_VARIANT_D64x256_S3, fused))
+            order[1] = SPMM_VARIANT_D64x256_S3;
         order[2] = long_k ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_R64x256_S3;
         order[3] = SPMM_VARIANT_64x256;
     } else {

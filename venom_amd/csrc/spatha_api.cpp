@@ -24,7 +24,7 @@ struct spatha_spmm_plan {
     void* zeros;           // 1 KiB of zeros on the device
     uint16_t* gtab;        // gather table of the dense-staged kernels (m <= 8, rows % 256 == 0), or null
     uint16_t* gtab_tiles;  // tile-major copy for the flag-synchronised kernel
-    size_t gtab_tiles_bytes;
+    size_t gtab_tiles_bytes, gtab_bytes;
     size_t apack_bytes, rowtab_bytes;
 };
 
@@ -64,8 +64,12 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = f
         variant == SPMM_VARIANT_DSF256x128_S3) {
         // four 64-row blocks per tile; all 16*m dense rows of a k-step must fit one stage
         if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 256 != 0 || !plan->gtab) return false;
-    } else if (plan->geo.v % bm != 0) {
+    } else if (variant != SPMM_VARIANT_DU512x128_S4 && plan->geo.v % bm != 0) {
         return false;
+    }
+    if (variant == SPMM_VARIANT_DU512x128_S4) {
+        if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 512 != 0 || !plan->gtab || plan->half_tiles) return false;
+        if (plan->gtab_bytes >= 0xE0000000ull) return false;
     }
     if (variant == SPMM_VARIANT_SKINNY && N > 64) return false;
     if (spmm_variant_lds(variant, plan->S) > 160 * 1024) return false;      // row table kept in LDS
@@ -310,7 +314,7 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     plan->geo = geo;
     plan->S = (geo.ksp + 31) / 32;
     plan->half_tiles = (v % 64 != 0);      // V = 32, 96, ...: a wave tile spans two V blocks
-    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr; plan->gtab_tiles = nullptr; plan->gtab_tiles_bytes = 0;
+    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr; plan->gtab_tiles = nullptr; plan->gtab_tiles_bytes = 0; plan->gtab_bytes = 0;
     e = hipGetDevice(&plan->device);
     if (e != hipSuccess) { delete plan; return hip_fail(e); }
     const size_t a_bytes = (size_t)(rows / 64) * plan->S * spatha::APACK_BLOCK;
@@ -330,6 +334,7 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
         // gather table of the dense-staged kernels: one entry per 64-row block, or per 32-row block when V % 64 != 0
         const int block_rows = plan->half_tiles ? 32 : 64;
         const size_t g_bytes = (size_t)(rows / block_rows) * plan->S * 64 * 2;
+        plan->gtab_bytes = g_bytes;
         if ((e = hipMalloc((void**)&plan->gtab, g_bytes)) != hipSuccess ||
             (e = spatha::launch_pack_gtab(columns_dev, rows, m, v, geo.ksp, plan->S, block_rows, plan->gtab,
                                           (hipStream_t)stream)) != hipSuccess) {
@@ -381,6 +386,7 @@ static int run_spmm(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
     p.apack = plan->apack; p.rowtab = plan->rowtab;
     p.B = B_dev; p.bias = bias_dev; p.C = out_dev; p.zeros = plan->zeros; p.gtab = plan->gtab;
     p.gtab_tiles = plan->gtab_tiles; p.gtab_tiles_bytes = (uint32_t)plan->gtab_tiles_bytes;
+    p.gtab_bytes = (uint32_t)plan->gtab_bytes;
     p.rows = plan->geo.rows; p.cols = plan->geo.cols; p.N = N; p.S = plan->S; p.v = plan->geo.v; p.m = plan->geo.m;
     const int bm = spatha::spmm_variant_bm(var), bn = spatha::spmm_variant_bn(var);
     p.tiles_m = plan->geo.rows / bm;

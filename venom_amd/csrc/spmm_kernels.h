@@ -16,6 +16,7 @@ struct SpmmParams {
     const uint16_t* gtab;     // dense-staged kernels: LDS offset per (64-row block, step, lane class, fragment), or null
     const uint16_t* gtab_tiles;  // the same table, tile-major (512 B per 256-row tile and step), or null
     uint32_t gtab_tiles_bytes;
+    uint32_t gtab_bytes;      // size of gtab (buffer descriptor of the unified dense-staged kernel)
     const uint16_t* B;        // cols x N, row-major
     const uint16_t* bias;     // rows, or null
     const void* zeros;        // >= 1 KiB of zero bytes (source of zero-filled B rows)
@@ -69,7 +70,8 @@ enum {
     SPMM_VARIANT_H64x128_S3 = 34,
     SPMM_VARIANT_H64x128_S2 = 35,
     SPMM_VARIANT_DSH256x128_S3_C8 = 36, // V % 64 != 0, m <= 8: dense-staged B, two gather-table entries per consumer wave
-    SPMM_VARIANT_COUNT = 37
+    SPMM_VARIANT_DU512x128_S4 = 37,     // m <= 8, rows % 512 == 0: eight unified 64 x 128 waves, A operands in registers, only B staged
+    SPMM_VARIANT_COUNT = 38
 };
 
 const char* spmm_variant_name(int variant);

@@ -2736,6 +2736,249 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------------------
+// Dense-staged kernel with unified waves and the A operands in registers (m <= 8, rows % 512 == 0): tile 512 x 128.
+//
+// The producer/consumer kernels above move 150 KB per k-step through LDS for a 256 x 128 tile (50 KB of DMA writes,
+// 36.8 KB of A operand reads, 64 KB of transposing B reads) and fetch 50 KB from L2; both rates are at their limit.
+// Here each of the eight waves owns 64 rows x 128 columns (128 accumulator registers), so the packed A operands of a
+// row block are used by exactly one wave and go straight from L2 into its registers, one k-step ahead; only the dense
+// B stage (32 KB) lives in LDS, four stages deep, shared by eight 64-row blocks.  Per 256 x 128 of output and step
+// that is 34.4 KB from L2 and 80 KB through LDS.  Every wave issues an eighth of each stage's DMA itself.
+// Vector-memory bookkeeping: register loads and LDS-DMA loads retire in order on one counter; a step issues the
+// gather-table entry and the A operands of the next step (7 loads), then its share of the stage three steps ahead
+// (4 loads), and waits for "all but the 4 youngest" before it ends.
+// ---------------------------------------------------------------------------
+struct DuCfg {
+    static constexpr int BM = 512, BN = 128, NS = 4, PA = 3, M = 8;
+    static constexpr int ROW_BYTES = BN * 2;
+    static constexpr int STAGE_BYTES = 16 * M * ROW_BYTES;
+    static constexpr int SLAB_BYTES = TT_SLAB_BYTES;
+    static_assert(SLAB_BYTES >= TR8_SLAB_BYTES + 128, "slab");
+    static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES + 8 * SLAB_BYTES;
+    static constexpr int THREADS = 512;
+};
+
+__device__ __forceinline__ u32x4 bload_b128(uint32_t voff, i32x4 rsrc, uint32_t soff) {
+    u32x4 r;
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    return r;
+}
+__device__ __forceinline__ uint32_t bload_b32(uint32_t voff, i32x4 rsrc, uint32_t soff) {
+    uint32_t r;
+    asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "=v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    return r;
+}
+__device__ __forceinline__ u32x2 bload_b64(uint32_t voff, i32x4 rsrc, uint32_t soff) {
+    u32x2 r;
+    asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "=v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    return r;
+}
+
+template <int OUT_LAYOUT>
+__global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
+    using Cfg = DuCfg;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, PA = Cfg::PA, STAGE_BYTES = Cfg::STAGE_BYTES;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TileWalk walk;
+    walk.init(p.tiles_m, p.tiles_n);
+    if (walk.my_tiles == 0) return;
+    const int S = p.S, N = p.N;
+    const int Q = walk.my_tiles * S;
+    const i32x4 rsrc_b = make_buffer(p.B, p.b_bytes);
+    const i32x4 rsrc_a = make_buffer(p.apack, p.apack_bytes);
+    const i32x4 rsrc_g = make_buffer(p.gtab, p.gtab_bytes);
+
+    // ---- this wave's share of the B stages (as a producer) ----
+    const uint32_t row_bytes_b = (uint32_t)N * 2u;
+    const int dense_rows = 16 * p.m;
+    const uint32_t step_bytes_b = (uint32_t)dense_rows * row_bytes_b;
+    const int slot_row = lane >> 4, slot_chunk = lane & 15;
+    int is_tm = walk.tm0, is_tn = walk.tn0, is_step = 0;
+    uint32_t is_stage = 0, b_soff = 0;
+    uint32_t voff[4];
+    auto set_voff = [&]() {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int row = (wave * 4 + j) * 4 + slot_row;
+            const int col = is_tn * BN + (slot_chunk ^ ((row & 7) << 1)) * 8;
+            voff[j] = (col < N && row < dense_rows) ? (uint32_t)row * row_bytes_b + (uint32_t)col * 2u : 0xF0000000u;
+        }
+    };
+    set_voff();
+    auto issue_stage = [&]() {
+        const uint32_t stage = smem_base + is_stage;
+#pragma unroll
+        for (int j = 0; j < 4; j++) bdma_b128(voff[j], rsrc_b, b_soff, stage + (wave * 4 + j) * 1024);
+        is_stage = (is_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : is_stage + STAGE_BYTES;
+        b_soff += step_bytes_b;
+        if (++is_step == S) {
+            is_step = 0;
+            b_soff = 0;
+            walk.next(is_tm, is_tn);
+            set_voff();
+        }
+    };
+
+    // ---- operands (as a consumer) ----
+    const int li = lane & 15, kb = lane >> 4;
+    const uint32_t col_xor = (uint32_t)(((li & 3) >> 1) << 4);
+    const uint32_t col_or = (uint32_t)(li & 1) * 8u;
+    const int lane_class = kb * 4 + (li >> 2);
+    const uint32_t lane16 = lane * 16, lane4 = lane * 4, gvoff = lane_class * 8;
+    u32x4 ax[4], ay[4];
+    uint32_t ix0, ix1, iy0, iy1;
+    u32x2 gy;
+    uint32_t base[4];
+    auto set_base = [&](u32x2 g) {
+        base[0] = ((g.x & 0xffffu) ^ col_xor) | col_or;
+        base[1] = ((g.x >> 16) ^ col_xor) | col_or;
+        base[2] = ((g.y & 0xffffu) ^ col_xor) | col_or;
+        base[3] = ((g.y >> 16) ^ col_xor) | col_or;
+    };
+    auto load_next = [&](int tm, int step) {      // gather-table entry and A operands of (tile row tm, step) -> set y
+        const uint32_t blk = (uint32_t)((tm * 8 + wave) * S + step);
+        gy = bload_b64(gvoff, rsrc_g, blk * 128u);
+        const uint32_t soff = blk * (uint32_t)APACK_BLOCK;
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) ay[mb] = bload_b128(lane16, rsrc_a, soff + mb * 1024);
+        iy0 = bload_b32(lane4, rsrc_a, soff + 4096);
+        iy1 = bload_b32(lane4, rsrc_a, soff + 4096 + 256);
+    };
+    float4_t acc[2][4][4];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int a = 0; a < 4; a++)
+#pragma unroll
+                for (int b = 0; b < 4; b++) acc[h][a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    };
+
+    // ---- prologue: three stages and the first operand set in flight ----
+#pragma unroll
+    for (int t = 0; t < PA; t++)
+        if (t < Q) issue_stage();
+    int issued = Q < PA ? Q : PA;
+    load_next(walk.tm0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(ay[0]), "+v"(ay[1]), "+v"(ay[2]), "+v"(ay[3]), "+v"(iy0), "+v"(iy1), "+v"(gy));
+#pragma unroll
+    for (int mb = 0; mb < 4; mb++) ax[mb] = ay[mb];
+    ix0 = iy0;
+    ix1 = iy1;
+    set_base(gy);
+    zero_acc();
+
+    int c_tm = walk.tm0, c_tn = walk.tn0, c_step = 0;
+    int n_tm = c_tm, n_tn = c_tn, tiles_left = walk.my_tiles;
+    uint32_t c_stage = 0;
+    for (int q = 0; q < Q; q++) {
+        __syncthreads();        // stage q has landed for every wave; stage q - 1 is free
+        int ns = c_step + 1;
+        if (ns == S) {
+            ns = 0;
+            if (tiles_left > 1) walk.next(n_tm, n_tn);
+        }
+        load_next(n_tm, ns);    // (one past the end: the last block again, never used)
+        const bool more = issued < Q;
+        if (more) {
+            issue_stage();
+            ++issued;
+        }
+        const char* st = smem + c_stage;
+        {
+            half8_t a_cur[4];
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) a_cur[mb] = __builtin_bit_cast(half8_t, ax[mb]);
+            auto read_frag = [&](int nb8) {
+                half16_t bf;
+#pragma unroll
+                for (int fb = 0; fb < 4; fb++) {
+                    short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, st + (base[fb] ^ (uint32_t)(nb8 << 5))));
+                    half4_t h4 = __builtin_bit_cast(half4_t, t4);
+                    bf[fb * 4 + 0] = h4[0];
+                    bf[fb * 4 + 1] = h4[1];
+                    bf[fb * 4 + 2] = h4[2];
+                    bf[fb * 4 + 3] = h4[3];
+                }
+                return bf;
+            };
+#define SPATHA_MMA4U(NB8, BF)                                                                                          \
+    acc[(NB8) >> 2][0][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[0], BF, acc[(NB8) >> 2][0][(NB8)&3], (int)ix0, 0, 0); \
+    acc[(NB8) >> 2][1][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], BF, acc[(NB8) >> 2][1][(NB8)&3], (int)ix0, 0, 1); \
+    acc[(NB8) >> 2][2][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], BF, acc[(NB8) >> 2][2][(NB8)&3], (int)ix1, 0, 0); \
+    acc[(NB8) >> 2][3][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], BF, acc[(NB8) >> 2][3][(NB8)&3], (int)ix1, 0, 1);
+            half16_t bf0 = read_frag(0);
+            half16_t bf1 = read_frag(1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int nb8 = 0; nb8 < 8; nb8 += 2) {
+                SPATHA_MMA4U(nb8, bf0)
+                __builtin_amdgcn_sched_barrier(0);
+                if (nb8 + 2 < 8) bf0 = read_frag(nb8 + 2);
+                __builtin_amdgcn_sched_barrier(0);
+                SPATHA_MMA4U(nb8 + 1, bf1)
+                __builtin_amdgcn_sched_barrier(0);
+                if (nb8 + 3 < 8) bf1 = read_frag(nb8 + 3);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#undef SPATHA_MMA4U
+        }
+        c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+        // the next step's operands (and with them everything older) must be in; only this step's DMA may still fly
+        if (more) asm volatile("s_waitcnt vmcnt(4)" : "+v"(ay[0]), "+v"(ay[1]), "+v"(ay[2]), "+v"(ay[3]), "+v"(iy0), "+v"(iy1), "+v"(gy));
+        else asm volatile("s_waitcnt vmcnt(0)" : "+v"(ay[0]), "+v"(ay[1]), "+v"(ay[2]), "+v"(ay[3]), "+v"(iy0), "+v"(iy1), "+v"(gy));
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) ax[mb] = ay[mb];
+        ix0 = iy0;
+        ix1 = iy1;
+        set_base(gy);
+        if (++c_step == S) {
+            c_step = 0;
+            const int cm0 = c_tm * BM + wave * 64, cn0 = c_tn * BN;
+            char* stg = smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES;
+#pragma unroll
+            for (int wn = 0; wn < 2; wn++) {
+                if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
+                    store_block_transposed_slab<true>(acc[wn], stg, p.C, p.bias, (int64_t)cm0, cn0 + wn * 64, p.rows, N, lane, true);
+                else
+                    store_block_row_major_tr<true>(acc[wn], stg, p.C, (int64_t)cm0, cn0 + wn * 64, N, lane, true);
+            }
+            zero_acc();
+            walk.next(c_tm, c_tn);
+            --tiles_left;
+        }
+    }
+}
+
+template <int OUT_LAYOUT>
+static hipError_t launch_du(const SpmmParams& p, hipStream_t stream) {
+    constexpr int lds = DuCfg::LDS_BYTES;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static int cus = 0;
+    void (*kern)(SpmmParams) = spmm_du_kernel<OUT_LAYOUT>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        int dev = 0;
+        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int tiles = p.tiles_m * p.tiles_n;
+    int grid = (cus / 8) * 8;
+    const int need = ((tiles + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    if (grid < 8) grid = 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(DuCfg::THREADS), lds, stream, p);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
 // Dense-staged kernel without workgroup barriers in the main loop ("flag-synchronised").
 //
 // A step of the barrier-synchronised kernels above costs the matrix pipes several hundred idle
@@ -3412,6 +3655,7 @@ const char* spmm_variant_name(int variant) {
         case SPMM_VARIANT_H64x128_S3: return "smfmac16x16x64_halftile_ldsdirect_tile64x128_3stage";
         case SPMM_VARIANT_H64x128_S2: return "smfmac16x16x64_halftile_ldsdirect_tile64x128_2stage";
         case SPMM_VARIANT_DSH256x128_S3_C8: return "smfmac16x16x64_halftile_densestage_tile256x128_3stage_8consumers";
+        case SPMM_VARIANT_DU512x128_S4: return "smfmac16x16x64_unified_densestage_aregs_tile512x128_4stage";
         default: return nullptr;
     }
 }
@@ -3453,6 +3697,7 @@ int spmm_variant_lds(int variant, int S) {
         case SPMM_VARIANT_H64x128_S3: return half_stage_bytes<2, 3>() + S * 256;
         case SPMM_VARIANT_H64x128_S2: return half_stage_bytes<2, 2>() + S * 256;
         case SPMM_VARIANT_DSH256x128_S3_C8: return DsCfg<8, 3, 4, 8>::LDS_BYTES;
+        case SPMM_VARIANT_DU512x128_S4: return DuCfg::LDS_BYTES;
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_64x256: return 1;
         default: return 0;
     }
@@ -3469,6 +3714,7 @@ int spmm_variant_bm(int variant) {
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4:
         case SPMM_VARIANT_SKINNY: case SPMM_VARIANT_H64x256_S2: case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2: return 64;
         case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3: case SPMM_VARIANT_DSH256x128_S3_C8: return 256;
+        case SPMM_VARIANT_DU512x128_S4: return 512;
         default: return 0;
     }
 }
@@ -3479,7 +3725,8 @@ int spmm_variant_bn(int variant) {
         case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x128_S2:
         case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5:
         case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3:
-        case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2: case SPMM_VARIANT_DSH256x128_S3_C8: return 128;
+        case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2: case SPMM_VARIANT_DSH256x128_S3_C8:
+        case SPMM_VARIANT_DU512x128_S4: return 128;
         case SPMM_VARIANT_SKINNY: return 64;
         case SPMM_VARIANT_H64x256_S2: return 256;
         case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D64x256_S3: case SPMM_VARIANT_T128x256_S3:
@@ -3569,6 +3816,9 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
     if (variant == SPMM_VARIANT_DSH256x128_S3_C8)
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ds<8, 3, 4, 8, SPATHA_OUT_TRANSPOSED, false, true>(p, stream)
                                                    : launch_ds<8, 3, 4, 8, SPATHA_OUT_ROW_MAJOR, false, true>(p, stream);
+    if (variant == SPMM_VARIANT_DU512x128_S4)
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_du<SPATHA_OUT_TRANSPOSED>(p, stream)
+                                                   : launch_du<SPATHA_OUT_ROW_MAJOR>(p, stream);
     if (variant == SPMM_VARIANT_DSF256x128_S3)
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_dsf<8, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
                                                    : launch_dsf<8, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);

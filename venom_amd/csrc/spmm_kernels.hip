@@ -2748,6 +2748,9 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
 // gather-table entry and the A operands of the next step (7 loads), then its share of the stage three steps ahead
 // (4 loads), and waits for "all but the 4 youngest" before it ends.
 // ---------------------------------------------------------------------------
+#ifndef DU_EXP
+#define DU_EXP 0
+#endif
 struct DuCfg {
     static constexpr int BM = 512, BN = 128, NS = 4, PA = 3, M = 8;
     static constexpr int ROW_BYTES = BN * 2;
@@ -2809,10 +2812,13 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
         }
     };
     set_voff();
-    auto issue_stage = [&]() {
-        const uint32_t stage = smem_base + is_stage;
+    uint32_t dma_stage = 0, dma_soff = 0;         // target and source offset of the stage being issued
+    uint32_t dma_voff[4];
+    auto stage_begin = [&]() {                    // fixes the addresses of the next stage and advances the cursor
+        dma_stage = smem_base + is_stage + wave * 4096;
+        dma_soff = b_soff;
 #pragma unroll
-        for (int j = 0; j < 4; j++) bdma_b128(voff[j], rsrc_b, b_soff, stage + (wave * 4 + j) * 1024);
+        for (int j = 0; j < 4; j++) dma_voff[j] = voff[j];
         is_stage = (is_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : is_stage + STAGE_BYTES;
         b_soff += step_bytes_b;
         if (++is_step == S) {
@@ -2822,6 +2828,12 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
             set_voff();
         }
     };
+    auto stage_op = [&](int j) { bdma_b128(dma_voff[j], rsrc_b, dma_soff, dma_stage + j * 1024); };
+    auto issue_stage = [&]() {
+        stage_begin();
+#pragma unroll
+        for (int j = 0; j < 4; j++) stage_op(j);
+    };
 
     // ---- operands (as a consumer) ----
     const int li = lane & 15, kb = lane >> 4;
@@ -2829,9 +2841,14 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
     const uint32_t col_or = (uint32_t)(li & 1) * 8u;
     const int lane_class = kb * 4 + (li >> 2);
     const uint32_t lane16 = lane * 16, lane4 = lane * 4, gvoff = lane_class * 8;
-    u32x4 ax[4], ay[4];
-    uint32_t ix0, ix1, iy0, iy1;
-    u32x2 gy;
+    // operand sets: x is the one the matrix instructions read; l0 / l1 are the landing sets of the loads, which run two
+    // k-steps ahead (an L2 round trip under load is longer than one step)
+    struct ASet {
+        u32x4 a[4];
+        uint32_t i0, i1;
+        u32x2 g;
+    };
+    ASet x, l0, l1;
     uint32_t base[4];
     auto set_base = [&](u32x2 g) {
         base[0] = ((g.x & 0xffffu) ^ col_xor) | col_or;
@@ -2839,14 +2856,40 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
         base[2] = ((g.y & 0xffffu) ^ col_xor) | col_or;
         base[3] = ((g.y >> 16) ^ col_xor) | col_or;
     };
-    auto load_next = [&](int tm, int step) {      // gather-table entry and A operands of (tile row tm, step) -> set y
-        const uint32_t blk = (uint32_t)((tm * 8 + wave) * S + step);
-        gy = bload_b64(gvoff, rsrc_g, blk * 128u);
-        const uint32_t soff = blk * (uint32_t)APACK_BLOCK;
+    // loader cursor: (tile row, step) of the next operand set to fetch; stops at the last step of the last tile
+    int ld_tm = walk.tm0, ld_tn = walk.tn0, ld_step = 0, ld_left = Q;
+    uint32_t ld_soff = 0, ld_goff = 0;
+    auto load_begin = [&]() {                     // fixes the addresses of the next operand set and advances the cursor
+        const uint32_t blk = (uint32_t)((ld_tm * 8 + wave) * S + ld_step);
+        ld_goff = blk * 128u;
+        ld_soff = blk * (uint32_t)APACK_BLOCK;
+        if (ld_left > 1) {          // (past the end the last block is fetched again and never used)
+            --ld_left;
+            if (++ld_step == S) {
+                ld_step = 0;
+                walk.next(ld_tm, ld_tn);
+            }
+        }
+    };
+    auto load_op = [&](ASet& y, int k) {          // the set's seven loads, in issue order
+        if (k == 0) y.g = bload_b64(gvoff, rsrc_g, ld_goff);
+        else if (k <= 4) y.a[k - 1] = bload_b128(lane16, rsrc_a, ld_soff + (k - 1) * 1024);
+        else if (k == 5) y.i0 = bload_b32(lane4, rsrc_a, ld_soff + 4096);
+        else y.i1 = bload_b32(lane4, rsrc_a, ld_soff + 4096 + 256);
+    };
+    auto load_set = [&](ASet& y) {
+        load_begin();
 #pragma unroll
-        for (int mb = 0; mb < 4; mb++) ay[mb] = bload_b128(lane16, rsrc_a, soff + mb * 1024);
-        iy0 = bload_b32(lane4, rsrc_a, soff + 4096);
-        iy1 = bload_b32(lane4, rsrc_a, soff + 4096 + 256);
+        for (int k = 0; k < 7; k++) load_op(y, k);
+    };
+#define SPATHA_DU_WAIT(CNT, Y) \
+    asm volatile("s_waitcnt vmcnt(" #CNT ")" : "+v"(Y.a[0]), "+v"(Y.a[1]), "+v"(Y.a[2]), "+v"(Y.a[3]), "+v"(Y.i0), "+v"(Y.i1), "+v"(Y.g))
+    auto take = [&](const ASet& y) {
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) x.a[mb] = y.a[mb];
+        x.i0 = y.i0;
+        x.i1 = y.i1;
+        set_base(y.g);
     };
     float4_t acc[2][4][4];
     auto zero_acc = [&]() {
@@ -2858,41 +2901,38 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
                 for (int b = 0; b < 4; b++) acc[h][a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
     };
 
-    // ---- prologue: three stages and the first operand set in flight ----
+    // ---- prologue: three stages and the first two operand sets in flight ----
 #pragma unroll
     for (int t = 0; t < PA; t++)
         if (t < Q) issue_stage();
     int issued = Q < PA ? Q : PA;
-    load_next(walk.tm0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(ay[0]), "+v"(ay[1]), "+v"(ay[2]), "+v"(ay[3]), "+v"(iy0), "+v"(iy1), "+v"(gy));
-#pragma unroll
-    for (int mb = 0; mb < 4; mb++) ax[mb] = ay[mb];
-    ix0 = iy0;
-    ix1 = iy1;
-    set_base(gy);
+    load_set(l0);
+    load_set(l1);
+    SPATHA_DU_WAIT(0, l0);
+    SPATHA_DU_WAIT(0, l1);
+    take(l0);
     zero_acc();
 
     int c_tm = walk.tm0, c_tn = walk.tn0, c_step = 0;
-    int n_tm = c_tm, n_tn = c_tn, tiles_left = walk.my_tiles;
     uint32_t c_stage = 0;
-    for (int q = 0; q < Q; q++) {
+    // one k-step: `land` receives the operands of step q + 2, `next` holds those of step q + 1
+    auto do_step = [&](ASet& land, ASet& next) {
         __syncthreads();        // stage q has landed for every wave; stage q - 1 is free
-        int ns = c_step + 1;
-        if (ns == S) {
-            ns = 0;
-            if (tiles_left > 1) walk.next(n_tm, n_tn);
-        }
-        load_next(n_tm, ns);    // (one past the end: the last block again, never used)
+        // The step's eleven vector-memory instructions (operands of step q + 2, then this wave's share of stage q + 3)
+        // are issued between the groups of matrix instructions: with the memory pipeline at its limit an issue can
+        // block for a long time, and the matrix pipe should have work queued meanwhile.
+        load_begin();
         const bool more = issued < Q;
         if (more) {
-            issue_stage();
+            stage_begin();
             ++issued;
         }
         const char* st = smem + c_stage;
         {
             half8_t a_cur[4];
 #pragma unroll
-            for (int mb = 0; mb < 4; mb++) a_cur[mb] = __builtin_bit_cast(half8_t, ax[mb]);
+            for (int mb = 0; mb < 4; mb++) a_cur[mb] = __builtin_bit_cast(half8_t, x.a[mb]);
+            const uint32_t ix0 = x.i0, ix1 = x.i1;
             auto read_frag = [&](int nb8) {
                 half16_t bf;
 #pragma unroll
@@ -2911,47 +2951,66 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
     acc[(NB8) >> 2][1][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], BF, acc[(NB8) >> 2][1][(NB8)&3], (int)ix0, 0, 1); \
     acc[(NB8) >> 2][2][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], BF, acc[(NB8) >> 2][2][(NB8)&3], (int)ix1, 0, 0); \
     acc[(NB8) >> 2][3][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], BF, acc[(NB8) >> 2][3][(NB8)&3], (int)ix1, 0, 1);
-            half16_t bf0 = read_frag(0);
-            half16_t bf1 = read_frag(1);
+            constexpr int DEPTH = 2;        // fragments in flight (three or four measure the same)
+            half16_t bf[DEPTH];
+#pragma unroll
+            for (int k = 0; k < DEPTH; k++) bf[k] = read_frag(k);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int nb8 = 0; nb8 < 8; nb8 += 2) {
-                SPATHA_MMA4U(nb8, bf0)
+            for (int nb8 = 0; nb8 < 8; nb8++) {
+                if (DU_EXP & 2) { asm volatile("" ::"v"(bf[nb8 % DEPTH])); if (nb8 == 0) { SPATHA_MMA4U(0, bf[0]) } }
+                else { SPATHA_MMA4U(nb8, bf[nb8 % DEPTH]) }
                 __builtin_amdgcn_sched_barrier(0);
-                if (nb8 + 2 < 8) bf0 = read_frag(nb8 + 2);
+                if (nb8 == 0) { load_op(land, 0); load_op(land, 1); }
+                else if (nb8 == 1) { load_op(land, 2); load_op(land, 3); }
+                else if (nb8 == 2) { load_op(land, 4); load_op(land, 5); }
+                else if (nb8 == 3) { load_op(land, 6); }
+                else if (more && !(DU_EXP & 1)) stage_op(nb8 - 4);
                 __builtin_amdgcn_sched_barrier(0);
-                SPATHA_MMA4U(nb8 + 1, bf1)
-                __builtin_amdgcn_sched_barrier(0);
-                if (nb8 + 3 < 8) bf1 = read_frag(nb8 + 3);
+                if (nb8 + DEPTH < 8 && !(DU_EXP & 4)) bf[nb8 % DEPTH] = read_frag(nb8 + DEPTH);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #undef SPATHA_MMA4U
         }
         c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
-        // the next step's operands (and with them everything older) must be in; only this step's DMA may still fly
-        if (more) asm volatile("s_waitcnt vmcnt(4)" : "+v"(ay[0]), "+v"(ay[1]), "+v"(ay[2]), "+v"(ay[3]), "+v"(iy0), "+v"(iy1), "+v"(gy));
-        else asm volatile("s_waitcnt vmcnt(0)" : "+v"(ay[0]), "+v"(ay[1]), "+v"(ay[2]), "+v"(ay[3]), "+v"(iy0), "+v"(iy1), "+v"(gy));
-#pragma unroll
-        for (int mb = 0; mb < 4; mb++) ax[mb] = ay[mb];
-        ix0 = iy0;
-        ix1 = iy1;
-        set_base(gy);
+        // the operands of step q + 1 were issued a step ago; younger than them: that step's DMA (4), this step's operand
+        // loads (7) and DMA (4).  Near the end fewer are in flight: wait for all.
+        if (DU_EXP & 1) SPATHA_DU_WAIT(7, next);
+        else if (more) SPATHA_DU_WAIT(15, next);
+        else SPATHA_DU_WAIT(0, next);
+        take(next);
         if (++c_step == S) {
             c_step = 0;
             const int cm0 = c_tm * BM + wave * 64, cn0 = c_tn * BN;
             char* stg = smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES;
+#ifndef DU_NOWRITE
+#define DU_NOWRITE 0
+#endif
 #pragma unroll
             for (int wn = 0; wn < 2; wn++) {
-                if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
+                if (DU_NOWRITE) {
+                    float ss = 0.f;
+#pragma unroll
+                    for (int a = 0; a < 4; a++)
+#pragma unroll
+                        for (int b = 0; b < 4; b++)
+#pragma unroll
+                            for (int r = 0; r < 4; r++) ss += acc[wn][a][b][r];
+                    if (ss == 123.456f) p.C[lane] = 1;
+                } else if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
                     store_block_transposed_slab<true>(acc[wn], stg, p.C, p.bias, (int64_t)cm0, cn0 + wn * 64, p.rows, N, lane, true);
                 else
                     store_block_row_major_tr<true>(acc[wn], stg, p.C, (int64_t)cm0, cn0 + wn * 64, N, lane, true);
             }
             zero_acc();
             walk.next(c_tm, c_tn);
-            --tiles_left;
         }
+    };
+    for (int q = 0; q < Q; q += 2) {
+        do_step(l0, l1);
+        if (q + 1 < Q) do_step(l1, l0);
     }
+#undef SPATHA_DU_WAIT
 }
 
 template <int OUT_LAYOUT>

@@ -27,6 +27,7 @@ SMFMAC_PEAK_TFLOPS = 5033.0    # fp16 MFMA with 2:4 structured sparsity (dense f
 # scaled by a plain 256 MiB copy (summary under profiles/, named for the kernel); keyed by kernel name and shape.
 MEASURED_TRAFFIC_BYTES = {
     ("smfmac16x16x64_warpspec_densestage_tile256x128_3stage_8consumers", 4096, 1024, 16384, 8, 64): 194_615_000,
+    ("smfmac16x16x64_unified_densestage_aregs_tile512x128_4stage", 4096, 1024, 16384, 8, 64): 199_275_000,
 }
 
 

@@ -19,6 +19,7 @@ struct spatha_spmm_plan {
     int S;                 // k-steps of 64 compressed B rows
     int half_tiles;        // V % 64 != 0: operands packed in the order of the half-tile kernels
     int device;
+    int cus;               // compute units of that device
     uint16_t* apack;
     uint32_t* rowtab;
     void* zeros;           // 1 KiB of zeros on the device
@@ -181,6 +182,18 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
     } else {
         return -1;
     }
+    // Unified 512 x 128 kernel (m <= 8, rows % 512 == 0, no fused write-out): 3-13 % ahead of the producer/consumer forms
+    // of the dense-staged kernel when its tiles fill whole rounds of the CUs (BERT-large layer shapes at N = 16384,
+    // V = 64 and 128, m = 8 and 4: 256, 768, 1024 tiles), 10-20 % behind at 320 or 384 tiles (1.25 / 1.5 rounds) and up to
+    // 2x behind with fewer tiles than CUs; transposed output with 256 tiles of 8 k-steps measures 2-3 % behind.
+    if (!fused && plan->geo.m <= 8 && variant_ok(plan, N, SPMM_VARIANT_DU512x128_S4, fused)) {
+        const int64_t du_tiles = (int64_t)(plan->geo.rows / 512) * ((N + 127) / 128);
+        const int64_t cus = plan->cus > 0 ? plan->cus : 256;
+        const int64_t rounds = (du_tiles + cus - 1) / cus;
+        const bool whole_rounds = du_tiles >= cus && du_tiles * 10 >= rounds * cus * 9;
+        const bool layout_ok = out_layout == SPATHA_OUT_ROW_MAJOR || du_tiles >= 2 * cus || plan->S >= 16;
+        if (whole_rounds && layout_ok) return SPMM_VARIANT_DU512x128_S4;
+    }
     for (int i = 0; i < 4; i++)
         if (variant_ok(plan, N, order[i], fused)) return order[i];
     return -1;
@@ -317,6 +330,8 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr; plan->gtab_tiles = nullptr; plan->gtab_tiles_bytes = 0; plan->gtab_bytes = 0;
     e = hipGetDevice(&plan->device);
     if (e != hipSuccess) { delete plan; return hip_fail(e); }
+    plan->cus = 0;
+    if (hipDeviceGetAttribute(&plan->cus, hipDeviceAttributeMultiprocessorCount, plan->device) != hipSuccess) plan->cus = 0;
     const size_t a_bytes = (size_t)(rows / 64) * plan->S * spatha::APACK_BLOCK;
     const size_t r_bytes = (size_t)(rows / v) * plan->S * 64 * 4;
     plan->apack_bytes = a_bytes; plan->rowtab_bytes = r_bytes;

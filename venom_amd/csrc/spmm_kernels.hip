@@ -2917,7 +2917,7 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
     uint32_t c_stage = 0;
     // one k-step: `land` receives the operands of step q + 2, `next` holds those of step q + 1
     auto do_step = [&](ASet& land, ASet& next) {
-        __syncthreads();        // stage q has landed for every wave; stage q - 1 is free
+        if (!(DU_EXP & 8)) __syncthreads();        // stage q has landed for every wave; stage q - 1 is free
         // The step's eleven vector-memory instructions (operands of step q + 2, then this wave's share of stage q + 3)
         // are issued between the groups of matrix instructions: with the memory pipeline at its limit an issue can
         // block for a long time, and the matrix pipe should have work queued meanwhile.
@@ -2951,7 +2951,10 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
     acc[(NB8) >> 2][1][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], BF, acc[(NB8) >> 2][1][(NB8)&3], (int)ix0, 0, 1); \
     acc[(NB8) >> 2][2][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], BF, acc[(NB8) >> 2][2][(NB8)&3], (int)ix1, 0, 0); \
     acc[(NB8) >> 2][3][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], BF, acc[(NB8) >> 2][3][(NB8)&3], (int)ix1, 0, 1);
-            constexpr int DEPTH = 2;        // fragments in flight (three or four measure the same)
+#ifndef DU_DEPTH
+#define DU_DEPTH 2
+#endif
+            constexpr int DEPTH = DU_DEPTH;        // fragments in flight (three or four measure the same)
             half16_t bf[DEPTH];
 #pragma unroll
             for (int k = 0; k < DEPTH; k++) bf[k] = read_frag(k);

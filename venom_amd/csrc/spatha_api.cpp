@@ -42,7 +42,7 @@ bool variant_has_fused_writeout(int variant) {
     using namespace spatha;
     return (variant >= SPMM_VARIANT_P128x128_S4 && variant <= SPMM_VARIANT_W64x256_S3) ||      // pipelined, persistent, wave-specialised
            (variant >= SPMM_VARIANT_T128x256_S3 && variant <= SPMM_VARIANT_DS256x128_S3_C8) ||
-           variant == SPMM_VARIANT_DSH256x128_S3_C8;
+           variant == SPMM_VARIANT_DSH256x128_S3_C8 || variant == SPMM_VARIANT_DU512x128_S4;
 }
 
 bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = false) {

@@ -2748,9 +2748,6 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
 // gather-table entry and the A operands of the next step (7 loads), then its share of the stage three steps ahead
 // (4 loads), and waits for "all but the 4 youngest" before it ends.
 // ---------------------------------------------------------------------------
-#ifndef DU_EXP
-#define DU_EXP 0
-#endif
 struct DuCfg {
     static constexpr int BM = 512, BN = 128, NS = 4, PA = 3, M = 8;
     static constexpr int ROW_BYTES = BN * 2;
@@ -2778,7 +2775,9 @@ __device__ __forceinline__ u32x2 bload_b64(uint32_t voff, i32x4 rsrc, uint32_t s
     return r;
 }
 
-template <int OUT_LAYOUT>
+// FUSE: the instantiation that can apply bias / activation ahead of the write-out (kept apart: its temporaries would
+// otherwise push the plain kernel over the register budget)
+template <int OUT_LAYOUT, bool FUSE>
 __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
     using Cfg = DuCfg;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, PA = Cfg::PA, STAGE_BYTES = Cfg::STAGE_BYTES;
@@ -2917,7 +2916,7 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
     uint32_t c_stage = 0;
     // one k-step: `land` receives the operands of step q + 2, `next` holds those of step q + 1
     auto do_step = [&](ASet& land, ASet& next) {
-        if (!(DU_EXP & 8)) __syncthreads();        // stage q has landed for every wave; stage q - 1 is free
+        __syncthreads();        // stage q has landed for every wave; stage q - 1 is free
         // The step's eleven vector-memory instructions (operands of step q + 2, then this wave's share of stage q + 3)
         // are issued between the groups of matrix instructions: with the memory pipeline at its limit an issue can
         // block for a long time, and the matrix pipe should have work queued meanwhile.
@@ -2951,26 +2950,22 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
     acc[(NB8) >> 2][1][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[1], BF, acc[(NB8) >> 2][1][(NB8)&3], (int)ix0, 0, 1); \
     acc[(NB8) >> 2][2][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[2], BF, acc[(NB8) >> 2][2][(NB8)&3], (int)ix1, 0, 0); \
     acc[(NB8) >> 2][3][(NB8)&3] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[3], BF, acc[(NB8) >> 2][3][(NB8)&3], (int)ix1, 0, 1);
-#ifndef DU_DEPTH
-#define DU_DEPTH 2
-#endif
-            constexpr int DEPTH = DU_DEPTH;        // fragments in flight (three or four measure the same)
+            constexpr int DEPTH = 2;        // fragments in flight (three or four measure the same)
             half16_t bf[DEPTH];
 #pragma unroll
             for (int k = 0; k < DEPTH; k++) bf[k] = read_frag(k);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int nb8 = 0; nb8 < 8; nb8++) {
-                if (DU_EXP & 2) { asm volatile("" ::"v"(bf[nb8 % DEPTH])); if (nb8 == 0) { SPATHA_MMA4U(0, bf[0]) } }
-                else { SPATHA_MMA4U(nb8, bf[nb8 % DEPTH]) }
+                SPATHA_MMA4U(nb8, bf[nb8 % DEPTH])
                 __builtin_amdgcn_sched_barrier(0);
                 if (nb8 == 0) { load_op(land, 0); load_op(land, 1); }
                 else if (nb8 == 1) { load_op(land, 2); load_op(land, 3); }
                 else if (nb8 == 2) { load_op(land, 4); load_op(land, 5); }
                 else if (nb8 == 3) { load_op(land, 6); }
-                else if (more && !(DU_EXP & 1)) stage_op(nb8 - 4);
+                else if (more) stage_op(nb8 - 4);
                 __builtin_amdgcn_sched_barrier(0);
-                if (nb8 + DEPTH < 8 && !(DU_EXP & 4)) bf[nb8 % DEPTH] = read_frag(nb8 + DEPTH);
+                if (nb8 + DEPTH < 8) bf[nb8 % DEPTH] = read_frag(nb8 + DEPTH);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #undef SPATHA_MMA4U
@@ -2978,30 +2973,24 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
         c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
         // the operands of step q + 1 were issued a step ago; younger than them: that step's DMA (4), this step's operand
         // loads (7) and DMA (4).  Near the end fewer are in flight: wait for all.
-        if (DU_EXP & 1) SPATHA_DU_WAIT(7, next);
-        else if (more) SPATHA_DU_WAIT(15, next);
+        if (more) SPATHA_DU_WAIT(15, next);
         else SPATHA_DU_WAIT(0, next);
         take(next);
         if (++c_step == S) {
             c_step = 0;
             const int cm0 = c_tm * BM + wave * 64, cn0 = c_tn * BN;
             char* stg = smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES;
-#ifndef DU_NOWRITE
-#define DU_NOWRITE 0
-#endif
+            const int ib = lane >> 4;
+            // a bias alone rides in the row-major write-out itself (packed fp16 additions); anything else goes first
+            const bool pre = FUSE && (p.act != SPATHA_ACT_NONE || OUT_LAYOUT == SPATHA_OUT_TRANSPOSED);
 #pragma unroll
             for (int wn = 0; wn < 2; wn++) {
-                if (DU_NOWRITE) {
-                    float ss = 0.f;
-#pragma unroll
-                    for (int a = 0; a < 4; a++)
-#pragma unroll
-                        for (int b = 0; b < 4; b++)
-#pragma unroll
-                            for (int r = 0; r < 4; r++) ss += acc[wn][a][b][r];
-                    if (ss == 123.456f) p.C[lane] = 1;
-                } else if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
-                    store_block_transposed_slab<true>(acc[wn], stg, p.C, p.bias, (int64_t)cm0, cn0 + wn * 64, p.rows, N, lane, true);
+                if (FUSE && pre) fused_bias_act(acc[wn], p.bias, (int64_t)cm0 + ib * 16, p.act);
+                if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
+                    store_block_transposed_slab<true>(acc[wn], stg, p.C, FUSE ? nullptr : p.bias, (int64_t)cm0, cn0 + wn * 64, p.rows,
+                                                      N, lane, true);
+                else if (FUSE && !pre && p.bias)
+                    store_block_row_major_tr<true, true>(acc[wn], stg, p.C, (int64_t)cm0, cn0 + wn * 64, N, lane, true, p.bias);
                 else
                     store_block_row_major_tr<true>(acc[wn], stg, p.C, (int64_t)cm0, cn0 + wn * 64, N, lane, true);
             }
@@ -3016,12 +3005,12 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
 #undef SPATHA_DU_WAIT
 }
 
-template <int OUT_LAYOUT>
+template <int OUT_LAYOUT, bool FUSE>
 static hipError_t launch_du(const SpmmParams& p, hipStream_t stream) {
     constexpr int lds = DuCfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static int cus = 0;
-    void (*kern)(SpmmParams) = spmm_du_kernel<OUT_LAYOUT>;
+    void (*kern)(SpmmParams) = spmm_du_kernel<OUT_LAYOUT, FUSE>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -3879,8 +3868,9 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ds<8, 3, 4, 8, SPATHA_OUT_TRANSPOSED, false, true>(p, stream)
                                                    : launch_ds<8, 3, 4, 8, SPATHA_OUT_ROW_MAJOR, false, true>(p, stream);
     if (variant == SPMM_VARIANT_DU512x128_S4)
-        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_du<SPATHA_OUT_TRANSPOSED>(p, stream)
-                                                   : launch_du<SPATHA_OUT_ROW_MAJOR>(p, stream);
+        return out_layout == SPATHA_OUT_TRANSPOSED
+                   ? (p.fuse ? launch_du<SPATHA_OUT_TRANSPOSED, true>(p, stream) : launch_du<SPATHA_OUT_TRANSPOSED, false>(p, stream))
+                   : (p.fuse ? launch_du<SPATHA_OUT_ROW_MAJOR, true>(p, stream) : launch_du<SPATHA_OUT_ROW_MAJOR, false>(p, stream));
     if (variant == SPMM_VARIANT_DSF256x128_S3)
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_dsf<8, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
                                                    : launch_dsf<8, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);

@@ -42,6 +42,7 @@ CASES = [
     (384, 416, 520, 8, 192),      # V = 192 (multiple of 64 only)
     (256, 100, 72, 8, 64),        # 256-row tiles (dense-staged kernels), cols % m != 0
     (512, 1000, 392, 8, 64),
+    (1024, 200, 264, 8, 64),      # two 512-row tiles, three column tiles, K tail (unified 512 x 128 kernel among others)
     (256, 64, 8, 4, 64),          # dense-staged, plain 2:4
     (512, 325, 136, 5, 128),      # dense-staged, m = 5, V = 128, cols % m == 0 but Ksp padded
     (768, 450, 264, 7, 192),      # dense-staged, m = 7, V = 192, two-column tail
@@ -126,7 +127,7 @@ def test_half_tile_gaussian_within_tolerance(gpu):
     B = rng.uniform(-1, 1, size=(cols, N)).astype(np.float16)
     exact = oracle.decode(vals, meta, columns, rows, cols, 2, m, v).astype(np.float64) @ B.astype(np.float64)
     plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
-    for variant in (0, spatha.num_variants() - 2):
+    for variant in (0, 35, 36):        # automatic, gathered and dense-staged half-tile kernels
         got = plan.run(_dev(B, gpu), variant=variant).cpu().numpy().astype(np.float64)
         assert (np.abs(got - exact) / np.maximum(np.abs(exact), 1.0)).max() <= REL_TOL
 
@@ -232,6 +233,24 @@ def test_dense_staged_kernel_is_selected_for_v64(gpu):
     assert "densestage" not in _plan(vals, meta, columns, rows, cols, 16, v, gpu).kernel_name(N, 0, 0)
     vals, meta, columns = F.synthetic_vnm(128, cols, 2, m, v, seed=2, integer_values=True)
     assert "densestage" not in _plan(vals, meta, columns, 128, cols, m, v, gpu).kernel_name(N, 0, 0)
+
+
+def test_unified_kernel_is_selected_when_its_tiles_fill_whole_rounds(gpu):
+    """The 512 x 128 kernel (A operands in registers) is the automatic choice when its tiles fill whole rounds of the
+    CUs, and only then; it needs rows % 512 == 0 and m <= 8."""
+    rows, cols, m, v = 4096, 1024, 8, 64
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=3, integer_values=True)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    n_whole = 128 * cus // (rows // 512)            # exactly one tile per CU
+    assert "unified" in plan.kernel_name(n_whole, 0, 0)
+    assert "unified" in plan.kernel_name(4 * n_whole, 0, 0) and "unified" in plan.kernel_name(4 * n_whole, 1, 0)
+    assert "unified" not in plan.kernel_name(n_whole // 2, 0, 0)          # half of the CUs would idle
+    assert "unified" not in plan.kernel_name(n_whole + n_whole // 2, 0, 0)  # 1.5 rounds
+    # explicit request on a small problem: allowed (and bit-exact, see the variant loops above); 256-row matrices are not
+    assert plan.kernel_name(256, 0, 37) is not None
+    vals, meta, columns = F.synthetic_vnm(256, cols, 2, m, v, seed=3, integer_values=True)
+    assert _plan(vals, meta, columns, 256, cols, m, v, gpu).kernel_name(256, 0, 37) is None
 
 
 @pytest.mark.parametrize("path", [p for p in golden_cases() if "vnm_z_" not in p],

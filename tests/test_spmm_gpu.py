@@ -43,6 +43,9 @@ CASES = [
     (256, 100, 72, 8, 64),        # 256-row tiles (dense-staged kernels), cols % m != 0
     (512, 1000, 392, 8, 64),
     (1024, 200, 264, 8, 64),      # two 512-row tiles, three column tiles, K tail (unified 512 x 128 kernel among others)
+    (512, 650, 136, 10, 64),      # unified kernel for 8 < m <= 16: five k-steps through two 64 KB stages, K tail, ragged N
+    (1024, 2048, 264, 16, 128),   # ... m = 16, eight k-steps, two tile rows
+    (1536, 768, 136, 12, 192),    # ... m = 12, V = 192, three tile rows
     (256, 64, 8, 4, 64),          # dense-staged, plain 2:4
     (512, 325, 136, 5, 128),      # dense-staged, m = 5, V = 128, cols % m == 0 but Ksp padded
     (768, 450, 264, 7, 192),      # dense-staged, m = 7, V = 192, two-column tail
@@ -246,6 +249,10 @@ def test_unified_kernel_is_selected_when_its_tiles_fill_whole_rounds(gpu):
     assert "unified" in plan.kernel_name(n_whole, 0, 0)
     assert "unified" in plan.kernel_name(4 * n_whole, 0, 0) and "unified" in plan.kernel_name(4 * n_whole, 1, 0)
     assert "unified" not in plan.kernel_name(n_whole // 2, 0, 0)          # half of the CUs would idle
+    vals16, meta16, columns16 = F.synthetic_vnm(rows, cols, 2, 16, v, seed=3, integer_values=True)
+    plan16 = _plan(vals16, meta16, columns16, rows, cols, 16, v, gpu)
+    assert "unified" in plan16.kernel_name(n_whole, 0, 0) and "m16" in plan16.kernel_name(4 * n_whole, 1, 0)
+    assert "unified" not in plan16.kernel_name(n_whole // 2, 0, 0)
     assert "unified" not in plan.kernel_name(n_whole + n_whole // 2, 0, 0)  # 1.5 rounds
     # explicit request on a small problem: allowed (and bit-exact, see the variant loops above); 256-row matrices are not
     assert plan.kernel_name(256, 0, 37) is not None

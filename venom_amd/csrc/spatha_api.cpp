@@ -65,11 +65,17 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = f
         variant == SPMM_VARIANT_DSF256x128_S3) {
         // four 64-row blocks per tile; all 16*m dense rows of a k-step must fit one stage
         if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 256 != 0 || !plan->gtab) return false;
-    } else if (variant != SPMM_VARIANT_DU512x128_S4 && plan->geo.v % bm != 0) {
+    } else if (variant != SPMM_VARIANT_DU512x128_S4 && variant != SPMM_VARIANT_DU512x128_M16 && plan->geo.v % bm != 0) {
         return false;
     }
     if (variant == SPMM_VARIANT_DU512x128_S4) {
         if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 512 != 0 || !plan->gtab || plan->half_tiles) return false;
+        if (plan->gtab_bytes >= 0xE0000000ull) return false;
+    }
+    if (variant == SPMM_VARIANT_DU512x128_M16) {
+        if (plan->geo.v % 64 != 0 || plan->geo.m <= 8 || plan->geo.m > 16 || plan->geo.rows % 512 != 0 || !plan->gtab ||
+            plan->half_tiles || fused)
+            return false;
         if (plan->gtab_bytes >= 0xE0000000ull) return false;
     }
     if (variant == SPMM_VARIANT_SKINNY && N > 64) return false;
@@ -193,6 +199,15 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         const bool whole_rounds = du_tiles >= cus && du_tiles * 10 >= rounds * cus * 9;
         const bool layout_ok = out_layout == SPATHA_OUT_ROW_MAJOR || du_tiles >= 2 * cus || plan->S >= 16;
         if (whole_rounds && layout_ok) return SPMM_VARIANT_DU512x128_S4;
+    }
+    // Its form for 8 < m <= 16 (64 KB stages, two of them): V a multiple of 64 only - 7-26 % ahead of the gathered
+    // 64 x 256 tiles on the BERT-large layer shapes at N = 16384 (64:2:16 and 64:2:10, both layouts); with V % 128 == 0
+    // the gathered 128 x 256 tiles share their B rows over 128 rows and are equal or up to 15 % ahead.
+    if (!fused && plan->geo.m > 8 && plan->geo.v % 128 != 0 && variant_ok(plan, N, SPMM_VARIANT_DU512x128_M16, fused)) {
+        const int64_t du_tiles = (int64_t)(plan->geo.rows / 512) * ((N + 127) / 128);
+        const int64_t cus = plan->cus > 0 ? plan->cus : 256;
+        const int64_t rounds = (du_tiles + cus - 1) / cus;
+        if (du_tiles >= cus && du_tiles * 10 >= rounds * cus * 9) return SPMM_VARIANT_DU512x128_M16;
     }
     for (int i = 0; i < 4; i++)
         if (variant_ok(plan, N, order[i], fused)) return order[i];
@@ -345,7 +360,7 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     e = spatha::launch_pack(values_dev, metadata_dev, columns_dev, rows, cols, m, v, geo.ksp, plan->S, plan->half_tiles,
                             plan->apack, plan->rowtab, (hipStream_t)stream);
     if (e != hipSuccess) { spatha_spmm_plan_destroy(plan); return hip_fail(e); }
-    if (m <= 8 && rows % 256 == 0) {
+    if ((m <= 8 && rows % 256 == 0) || (m <= 16 && rows % 512 == 0 && !plan->half_tiles)) {
         // gather table of the dense-staged kernels: one entry per 64-row block, or per 32-row block when V % 64 != 0
         const int block_rows = plan->half_tiles ? 32 : 64;
         const size_t g_bytes = (size_t)(rows / block_rows) * plan->S * 64 * 2;

@@ -71,7 +71,8 @@ enum {
     SPMM_VARIANT_H64x128_S2 = 35,
     SPMM_VARIANT_DSH256x128_S3_C8 = 36, // V % 64 != 0, m <= 8: dense-staged B, two gather-table entries per consumer wave
     SPMM_VARIANT_DU512x128_S4 = 37,     // m <= 8, rows % 512 == 0: eight unified 64 x 128 waves, A operands in registers, only B staged
-    SPMM_VARIANT_COUNT = 38
+    SPMM_VARIANT_DU512x128_M16 = 38,    // the same for 8 < m <= 16: 64 KB stages, two of them
+    SPMM_VARIANT_COUNT = 39
 };
 
 const char* spmm_variant_name(int variant);

@@ -2744,12 +2744,17 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
 // row block are used by exactly one wave and go straight from L2 into its registers, one k-step ahead; only the dense
 // B stage (32 KB) lives in LDS, four stages deep, shared by eight 64-row blocks.  Per 256 x 128 of output and step
 // that is 34.4 KB from L2 and 80 KB through LDS.  Every wave issues an eighth of each stage's DMA itself.
-// Vector-memory bookkeeping: register loads and LDS-DMA loads retire in order on one counter; a step issues the
-// gather-table entry and the A operands of the next step (7 loads), then its share of the stage three steps ahead
-// (4 loads), and waits for "all but the 4 youngest" before it ends.
+// Vector-memory bookkeeping: register loads and LDS-DMA loads share one counter; a step issues the gather-table entry
+// and the A operands two steps ahead (7 register loads), then its share of the stage three steps ahead (4 DMA loads),
+// and ends on a wait that leaves at most 7 operations in flight (see there).
 // ---------------------------------------------------------------------------
+// M_ = 8: 32 KB stages, four of them; M_ = 16 (m <= 16): 64 KB stages, two of them - the stage for step q + 1 is issued
+// at the head of step q and has that step to land.
+template <int M_>
 struct DuCfg {
-    static constexpr int BM = 512, BN = 128, NS = 4, PA = 3, M = 8;
+    static_assert(M_ == 8 || M_ == 16, "dense rows per group a stage is sized for");
+    static constexpr int BM = 512, BN = 128, M = M_, NS = M_ == 8 ? 4 : 2, PA = NS - 1;
+    static constexpr int NB = M_ / 2;              // DMA instructions per wave and stage (4 rows x 256 B each)
     static constexpr int ROW_BYTES = BN * 2;
     static constexpr int STAGE_BYTES = 16 * M * ROW_BYTES;
     static constexpr int SLAB_BYTES = TT_SLAB_BYTES;
@@ -2777,9 +2782,10 @@ __device__ __forceinline__ u32x2 bload_b64(uint32_t voff, i32x4 rsrc, uint32_t s
 
 // FUSE: the instantiation that can apply bias / activation ahead of the write-out (kept apart: its temporaries would
 // otherwise push the plain kernel over the register budget)
-template <int OUT_LAYOUT, bool FUSE>
+template <int OUT_LAYOUT, bool FUSE, int M_>
 __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
-    using Cfg = DuCfg;
+    using Cfg = DuCfg<M_>;
+    constexpr int NB = Cfg::NB;
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::NS, PA = Cfg::PA, STAGE_BYTES = Cfg::STAGE_BYTES;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
@@ -2801,23 +2807,23 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
     const int slot_row = lane >> 4, slot_chunk = lane & 15;
     int is_tm = walk.tm0, is_tn = walk.tn0, is_step = 0;
     uint32_t is_stage = 0, b_soff = 0;
-    uint32_t voff[4];
+    uint32_t voff[NB];
     auto set_voff = [&]() {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int row = (wave * 4 + j) * 4 + slot_row;
+        for (int j = 0; j < NB; j++) {
+            const int row = (wave * NB + j) * 4 + slot_row;
             const int col = is_tn * BN + (slot_chunk ^ ((row & 7) << 1)) * 8;
             voff[j] = (col < N && row < dense_rows) ? (uint32_t)row * row_bytes_b + (uint32_t)col * 2u : 0xF0000000u;
         }
     };
     set_voff();
     uint32_t dma_stage = 0, dma_soff = 0;         // target and source offset of the stage being issued
-    uint32_t dma_voff[4];
+    uint32_t dma_voff[NB];
     auto stage_begin = [&]() {                    // fixes the addresses of the next stage and advances the cursor
-        dma_stage = smem_base + is_stage + wave * 4096;
+        dma_stage = smem_base + is_stage + wave * (NB * 1024);
         dma_soff = b_soff;
 #pragma unroll
-        for (int j = 0; j < 4; j++) dma_voff[j] = voff[j];
+        for (int j = 0; j < NB; j++) dma_voff[j] = voff[j];
         is_stage = (is_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : is_stage + STAGE_BYTES;
         b_soff += step_bytes_b;
         if (++is_step == S) {
@@ -2831,7 +2837,7 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
     auto issue_stage = [&]() {
         stage_begin();
 #pragma unroll
-        for (int j = 0; j < 4; j++) stage_op(j);
+        for (int j = 0; j < NB; j++) stage_op(j);
     };
 
     // ---- operands (as a consumer) ----
@@ -2959,11 +2965,18 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
             for (int nb8 = 0; nb8 < 8; nb8++) {
                 SPATHA_MMA4U(nb8, bf[nb8 % DEPTH])
                 __builtin_amdgcn_sched_barrier(0);
-                if (nb8 == 0) { load_op(land, 0); load_op(land, 1); }
-                else if (nb8 == 1) { load_op(land, 2); load_op(land, 3); }
-                else if (nb8 == 2) { load_op(land, 4); load_op(land, 5); }
-                else if (nb8 == 3) { load_op(land, 6); }
-                else if (more) stage_op(nb8 - 4);
+                if constexpr (M_ == 8) {
+                    if (nb8 == 0) { load_op(land, 0); load_op(land, 1); }
+                    else if (nb8 == 1) { load_op(land, 2); load_op(land, 3); }
+                    else if (nb8 == 2) { load_op(land, 4); load_op(land, 5); }
+                    else if (nb8 == 3) { load_op(land, 6); }
+                    else if (more) stage_op(nb8 - 4);
+                } else {
+                    // two stages: the DMA of the next step's stage goes first, the operand loads behind it
+                    if (nb8 < 4) { if (more) { stage_op(2 * nb8); stage_op(2 * nb8 + 1); } }
+                    else if (nb8 < 7) { load_op(land, 2 * (nb8 - 4)); load_op(land, 2 * (nb8 - 4) + 1); }
+                    else load_op(land, 6);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 if (nb8 + DEPTH < 8) bf[nb8 % DEPTH] = read_frag(nb8 + DEPTH);
                 __builtin_amdgcn_sched_barrier(0);
@@ -2973,7 +2986,13 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
         c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
         // the operands of step q + 1 were issued a step ago; younger than them: that step's DMA (4), this step's operand
         // loads (7) and DMA (4).  Near the end fewer are in flight: wait for all.
-        if (more) SPATHA_DU_WAIT(15, next);
+        // LDS-DMA loads and register loads each retire in order, but not with respect to each other (measured: a wait
+        // that leaves the 7 youngest operations, all register loads, in flight returned before older DMA loads had
+        // landed).  With at most 7 operations left, at most the 7 youngest of EACH kind are: the operand set of step
+        // q + 1 (7 younger register loads) and the DMA of stage q + 1 (8 younger DMA loads) are in.  The two-stage form
+        // needs the DMA it issued in this very step and can only wait for everything.
+        // Near the end no younger DMA is in flight any more: wait for everything there as well.
+        if (M_ == 8 && more) SPATHA_DU_WAIT(7, next);
         else SPATHA_DU_WAIT(0, next);
         take(next);
         if (++c_step == S) {
@@ -3005,12 +3024,12 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
 #undef SPATHA_DU_WAIT
 }
 
-template <int OUT_LAYOUT, bool FUSE>
+template <int OUT_LAYOUT, bool FUSE, int M_ = 8>
 static hipError_t launch_du(const SpmmParams& p, hipStream_t stream) {
-    constexpr int lds = DuCfg::LDS_BYTES;
+    constexpr int lds = DuCfg<M_>::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static int cus = 0;
-    void (*kern)(SpmmParams) = spmm_du_kernel<OUT_LAYOUT, FUSE>;
+    void (*kern)(SpmmParams) = spmm_du_kernel<OUT_LAYOUT, FUSE, M_>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -3025,7 +3044,7 @@ static hipError_t launch_du(const SpmmParams& p, hipStream_t stream) {
     const int need = ((tiles + 7) / 8) * 8;
     if (grid > need) grid = need;
     if (grid < 8) grid = 8;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(DuCfg::THREADS), lds, stream, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(DuCfg<M_>::THREADS), lds, stream, p);
     return hipGetLastError();
 }
 
@@ -3707,6 +3726,7 @@ const char* spmm_variant_name(int variant) {
         case SPMM_VARIANT_H64x128_S2: return "smfmac16x16x64_halftile_ldsdirect_tile64x128_2stage";
         case SPMM_VARIANT_DSH256x128_S3_C8: return "smfmac16x16x64_halftile_densestage_tile256x128_3stage_8consumers";
         case SPMM_VARIANT_DU512x128_S4: return "smfmac16x16x64_unified_densestage_aregs_tile512x128_4stage";
+        case SPMM_VARIANT_DU512x128_M16: return "smfmac16x16x64_unified_densestage_aregs_tile512x128_m16_2stage";
         default: return nullptr;
     }
 }
@@ -3748,7 +3768,8 @@ int spmm_variant_lds(int variant, int S) {
         case SPMM_VARIANT_H64x128_S3: return half_stage_bytes<2, 3>() + S * 256;
         case SPMM_VARIANT_H64x128_S2: return half_stage_bytes<2, 2>() + S * 256;
         case SPMM_VARIANT_DSH256x128_S3_C8: return DsCfg<8, 3, 4, 8>::LDS_BYTES;
-        case SPMM_VARIANT_DU512x128_S4: return DuCfg::LDS_BYTES;
+        case SPMM_VARIANT_DU512x128_S4: return DuCfg<8>::LDS_BYTES;
+        case SPMM_VARIANT_DU512x128_M16: return DuCfg<16>::LDS_BYTES;
         case SPMM_VARIANT_128x128: case SPMM_VARIANT_64x256: return 1;
         default: return 0;
     }
@@ -3765,7 +3786,7 @@ int spmm_variant_bm(int variant) {
         case SPMM_VARIANT_64x256: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_P64x256_S3: case SPMM_VARIANT_P64x256_S4:
         case SPMM_VARIANT_SKINNY: case SPMM_VARIANT_H64x256_S2: case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2: return 64;
         case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3: case SPMM_VARIANT_DSH256x128_S3_C8: return 256;
-        case SPMM_VARIANT_DU512x128_S4: return 512;
+        case SPMM_VARIANT_DU512x128_S4: case SPMM_VARIANT_DU512x128_M16: return 512;
         default: return 0;
     }
 }
@@ -3777,7 +3798,7 @@ int spmm_variant_bn(int variant) {
         case SPMM_VARIANT_D128x128_S3: case SPMM_VARIANT_D128x128_S5: case SPMM_VARIANT_T128x128_S4: case SPMM_VARIANT_T128x128_S5:
         case SPMM_VARIANT_DS256x128_S3: case SPMM_VARIANT_DS256x128_S2: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DS256x128_S3_PP: case SPMM_VARIANT_DSF256x128_S3:
         case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2: case SPMM_VARIANT_DSH256x128_S3_C8:
-        case SPMM_VARIANT_DU512x128_S4: return 128;
+        case SPMM_VARIANT_DU512x128_S4: case SPMM_VARIANT_DU512x128_M16: return 128;
         case SPMM_VARIANT_SKINNY: return 64;
         case SPMM_VARIANT_H64x256_S2: return 256;
         case SPMM_VARIANT_D128x256_S3: case SPMM_VARIANT_D64x256_S3: case SPMM_VARIANT_T128x256_S3:
@@ -3871,6 +3892,9 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
         return out_layout == SPATHA_OUT_TRANSPOSED
                    ? (p.fuse ? launch_du<SPATHA_OUT_TRANSPOSED, true>(p, stream) : launch_du<SPATHA_OUT_TRANSPOSED, false>(p, stream))
                    : (p.fuse ? launch_du<SPATHA_OUT_ROW_MAJOR, true>(p, stream) : launch_du<SPATHA_OUT_ROW_MAJOR, false>(p, stream));
+    if (variant == SPMM_VARIANT_DU512x128_M16)
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_du<SPATHA_OUT_TRANSPOSED, false, 16>(p, stream)
+                                                   : launch_du<SPATHA_OUT_ROW_MAJOR, false, 16>(p, stream);
     if (variant == SPMM_VARIANT_DSF256x128_S3)
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_dsf<8, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
                                                    : launch_dsf<8, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);

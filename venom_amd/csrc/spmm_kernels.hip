@@ -2984,8 +2984,6 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
 #undef SPATHA_MMA4U
         }
         c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
-        // the operands of step q + 1 were issued a step ago; younger than them: that step's DMA (4), this step's operand
-        // loads (7) and DMA (4).  Near the end fewer are in flight: wait for all.
         // LDS-DMA loads and register loads each retire in order, but not with respect to each other (measured: a wait
         // that leaves the 7 youngest operations, all register loads, in flight returned before older DMA loads had
         // landed).  With at most 7 operations left, at most the 7 youngest of EACH kind are: the operand set of step

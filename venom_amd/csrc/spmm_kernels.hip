@@ -2764,20 +2764,16 @@ struct DuCfg {
     static constexpr int THREADS = 512;
 };
 
-__device__ __forceinline__ u32x4 bload_b128(uint32_t voff, i32x4 rsrc, uint32_t soff) {
-    u32x4 r;
-    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
-    return r;
+// Loads into registers that complete asynchronously: the destination is the caller's variable itself ("+v"), so that no
+// copy of a not-yet-arrived value can be placed behind the instruction; the caller's wait names the same variables.
+__device__ __forceinline__ void bload_b128(u32x4& r, uint32_t voff, i32x4 rsrc, uint32_t soff) {
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
-__device__ __forceinline__ uint32_t bload_b32(uint32_t voff, i32x4 rsrc, uint32_t soff) {
-    uint32_t r;
-    asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "=v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
-    return r;
+__device__ __forceinline__ void bload_b32(uint32_t& r, uint32_t voff, i32x4 rsrc, uint32_t soff) {
+    asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
-__device__ __forceinline__ u32x2 bload_b64(uint32_t voff, i32x4 rsrc, uint32_t soff) {
-    u32x2 r;
-    asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "=v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
-    return r;
+__device__ __forceinline__ void bload_b64(u32x2& r, uint32_t voff, i32x4 rsrc, uint32_t soff) {
+    asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "+v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
 // FUSE: the instantiation that can apply bias / activation ahead of the write-out (kept apart: its temporaries would
@@ -2853,7 +2849,7 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
         uint32_t i0, i1;
         u32x2 g;
     };
-    ASet x, l0, l1;
+    ASet x, l0 = {}, l1 = {};
     uint32_t base[4];
     auto set_base = [&](u32x2 g) {
         base[0] = ((g.x & 0xffffu) ^ col_xor) | col_or;
@@ -2877,10 +2873,10 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
         }
     };
     auto load_op = [&](ASet& y, int k) {          // the set's seven loads, in issue order
-        if (k == 0) y.g = bload_b64(gvoff, rsrc_g, ld_goff);
-        else if (k <= 4) y.a[k - 1] = bload_b128(lane16, rsrc_a, ld_soff + (k - 1) * 1024);
-        else if (k == 5) y.i0 = bload_b32(lane4, rsrc_a, ld_soff + 4096);
-        else y.i1 = bload_b32(lane4, rsrc_a, ld_soff + 4096 + 256);
+        if (k == 0) bload_b64(y.g, gvoff, rsrc_g, ld_goff);
+        else if (k <= 4) bload_b128(y.a[k - 1], lane16, rsrc_a, ld_soff + (k - 1) * 1024);
+        else if (k == 5) bload_b32(y.i0, lane4, rsrc_a, ld_soff + 4096);
+        else bload_b32(y.i1, lane4, rsrc_a, ld_soff + 4096 + 256);
     };
     auto load_set = [&](ASet& y) {
         load_begin();

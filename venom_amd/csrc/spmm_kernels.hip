@@ -2736,13 +2736,13 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------------------
-// Dense-staged kernel with unified waves and the A operands in registers (m <= 8, rows % 512 == 0): tile 512 x 128.
+// Dense-staged kernel with unified waves and the A operands in registers (m <= 16, rows % 512 == 0): tile 512 x 128.
 //
 // The producer/consumer kernels above move 150 KB per k-step through LDS for a 256 x 128 tile (50 KB of DMA writes,
 // 36.8 KB of A operand reads, 64 KB of transposing B reads) and fetch 50 KB from L2; both rates are at their limit.
 // Here each of the eight waves owns 64 rows x 128 columns (128 accumulator registers), so the packed A operands of a
-// row block are used by exactly one wave and go straight from L2 into its registers, one k-step ahead; only the dense
-// B stage (32 KB) lives in LDS, four stages deep, shared by eight 64-row blocks.  Per 256 x 128 of output and step
+// row block are used by exactly one wave and go straight from L2 into its registers, two k-steps ahead; only the dense
+// B stage (32 KB for m <= 8) lives in LDS, four stages deep, shared by eight 64-row blocks.  Per 256 x 128 of output and step
 // that is 34.4 KB from L2 and 80 KB through LDS.  Every wave issues an eighth of each stage's DMA itself.
 // Vector-memory bookkeeping: register loads and LDS-DMA loads share one counter; a step issues the gather-table entry
 // and the A operands two steps ahead (7 register loads), then its share of the stage three steps ahead (4 DMA loads),

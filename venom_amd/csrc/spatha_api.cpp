@@ -115,7 +115,8 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
     // 2-5 % (BERT-base / BERT-large layer shapes at N = 2048 .. 8192), beyond that it falls behind; it has no fused
     // write-out and is measured for row-major output only.
     const int64_t ds_tiles = (int64_t)(plan->geo.rows / 256) * ((N + 127) / 128);
-    const int ds_variant = (ds_tiles <= 768 && !fused && out_layout == SPATHA_OUT_ROW_MAJOR &&
+    // (not for long k-loops: 12288 x 12288 x 2048 at 64:2:8, 96 k-steps, 255 us against 239 us)
+    const int ds_variant = (ds_tiles <= 768 && plan->S <= 32 && !fused && out_layout == SPATHA_OUT_ROW_MAJOR &&
                             variant_ok(plan, N, SPMM_VARIANT_DS256x128_S3_PP, fused))
                                ? SPMM_VARIANT_DS256x128_S3_PP
                                : SPMM_VARIANT_DS256x128_S3_C8;
@@ -207,7 +208,10 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         const int64_t du_tiles = (int64_t)(plan->geo.rows / 512) * ((N + 127) / 128);
         const int64_t cus = plan->cus > 0 ? plan->cus : 256;
         const int64_t rounds = (du_tiles + cus - 1) / cus;
-        if (du_tiles >= cus && du_tiles * 10 >= rounds * cus * 9) return SPMM_VARIANT_DU512x128_M16;
+        // long k-loops (GPT-3 projections at 64:2:16, 48 k-steps and more): ahead of every gathered form at 1.5 rounds too
+        // (12288 x 12288 x 2048: 177 us against 188 us for the best of them and 262 us for the per-tile pipeline)
+        const bool whole_rounds = du_tiles * 10 >= rounds * cus * 9;
+        if (du_tiles >= cus && (whole_rounds || plan->S >= 32)) return SPMM_VARIANT_DU512x128_M16;
     }
     for (int i = 0; i < 4; i++)
         if (variant_ok(plan, N, order[i], fused)) return order[i];

@@ -23,11 +23,15 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 SMFMAC_PEAK_TFLOPS = 5033.0    # fp16 MFMA with 2:4 structured sparsity (dense fp16 peak 2516.6 x 2)
 
 
-# HBM-side bytes per launch of the default workload's kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# scaled by a plain 256 MiB copy (summary under profiles/, named for the kernel); keyed by kernel name and shape.
-MEASURED_TRAFFIC_BYTES = {
-    ("smfmac16x16x64_warpspec_densestage_tile256x128_3stage_8consumers", 4096, 1024, 16384, 8, 64): 194_615_000,
-    ("smfmac16x16x64_unified_densestage_aregs_tile512x128_4stage", 4096, 1024, 16384, 8, 64): 199_275_000,
+# HBM-side bytes per launch of the default workload's kernel.  NOT measured by this script: the figure comes from two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by what the same counter reads for a
+# plain 256 MiB device copy (--copy-calibration); the summary that holds it is named beside it and printed as
+# roofline.traffic_source.  Keyed by kernel name and shape; any other kernel or shape reports null.
+MEASURED_TRAFFIC = {
+    ("smfmac16x16x64_warpspec_densestage_tile256x128_3stage_8consumers", 4096, 1024, 16384, 8, 64):
+        (194_615_000, "profiles/spmm_ds_kernel_tile256x128_ffn_up_64-2-8.md"),
+    ("smfmac16x16x64_unified_densestage_aregs_tile512x128_4stage", 4096, 1024, 16384, 8, 64):
+        (199_275_000, "profiles/spmm_du_kernel_tile512x128_ffn_up_64-2-8.md"),
 }
 
 
@@ -40,7 +44,13 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=500, help="untimed launches (the GPU needs ~50 ms of work to settle its clocks)")
+    ap.add_argument("--warmup", type=int, default=20, help="untimed launches right before the timed ones")
+    ap.add_argument("--settle-ms", type=float, default=200.0,
+                    help="before the warm-up launches, keep launching the kernel for this many milliseconds: the GPU's clock "
+                         "needs ~50-100 ms of work to settle, whatever --warmup says (reported as settle_ms, separate from warmup)")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the two compute-bound workloads (2:4 FFN-up, GPT-3 FFN at 2048 tokens) that the default run "
+                         "reports under 'extra'")
     ap.add_argument("--rows", type=int, default=4096)
     ap.add_argument("--cols", type=int, default=1024)
     ap.add_argument("--n", type=int, default=16384, help="columns of B (tokens)")
@@ -48,7 +58,7 @@ def main():
     ap.add_argument("--v", type=int, default=64)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--extra", action="store_true", help="also time the other benchmark shapes (reported under 'extra')")
+    ap.add_argument("--extra", action="store_true", help="also time the other BERT-large layer shapes (appended to 'extra')")
     ap.add_argument("--ablation", action="store_true",
                     help="also time the same matrix with identity column-loc (the reference's IDEAL_KERNEL ablation) and, "
                          "if `python -m venom_amd.build --ablation` has been run, the OUT_32B build (4-byte stores of C)")
@@ -70,7 +80,7 @@ def main():
         alt = os.path.join(ROOT, "venom_amd", "lib", "libspatha_out32b.so")
         if os.path.exists(alt):
             import subprocess
-            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu-baseline", "--steps", str(args.steps),
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu-baseline", "--no-extra", "--steps", str(args.steps),
                                 "--warmup", str(args.warmup), "--variant", str(args.variant)],
                                env=dict(os.environ, SPATHA_LIBRARY=alt), stdout=subprocess.PIPE, text=True)
             if r.returncode == 0 and r.stdout.strip():
@@ -100,12 +110,18 @@ def main():
         C = torch.empty((rows, N), dtype=torch.float16, device=dev)
         return dict(vals=vals, meta=meta, columns=columns, geo=g, plan=plan, B=B, C=C)
 
-    def timed(w, steps, warmup, variant=0):
+    def timed(w, steps, warmup, variant=0, settle_ms=None):
         """Wall clock around `steps` launches bracketed by synchronize, plus HIP events on the
         launch stream over the same region (average kernel duration)."""
         plan, B, C = w["plan"], w["B"], w["C"]
         stream = torch.cuda.current_stream(dev)
         sp = ctypes.c_void_p(stream.cuda_stream)
+        settle_ms = args.settle_ms if settle_ms is None else settle_ms
+        t_settle = time.perf_counter()
+        while (time.perf_counter() - t_settle) * 1e3 < settle_ms:       # time based: the clock settles on work done, not on a count
+            for _ in range(20):
+                _lib.check(L.spatha_spmm_run(plan._handle, B.data_ptr(), B.shape[1], None, C.data_ptr(), 0, variant, sp), "run")
+            torch.cuda.synchronize()
         for _ in range(warmup):
             _lib.check(L.spatha_spmm_run(plan._handle, B.data_ptr(), B.shape[1], None, C.data_ptr(), 0, variant, sp), "run")
         torch.cuda.synchronize()
@@ -138,6 +154,7 @@ def main():
     tflops = flops_dense / (ms_wall * 1e-3) / 1e12
     achieved_gbs = nbytes / (ms_kernel * 1e-3) / 1e9
 
+    traffic, traffic_source = MEASURED_TRAFFIC.get((w["plan"].kernel_name(N, 0, args.variant), rows, cols, N, m, v), (None, None))
     out = {
         "metric": "dense-equiv TFLOPS of the V:N:M SpMM at 64:2:8, BERT-large FFN",
         "value": round(tflops, 2),
@@ -145,6 +162,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_ms": args.settle_ms,
         "ms_per_step": round(ms_wall, 6),
         "us_per_spmm": round(ms_wall * 1e3, 3),
         "higher_is_better": True,
@@ -157,22 +175,39 @@ def main():
         "pct_smfmac_peak": round(100.0 * flops_smfmac / (ms_kernel * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((w["plan"].kernel_name(N, 0, args.variant), rows, cols, N, m, v)),
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes": nbytes, "kernel_us": round(ms_kernel * 1e3, 3)},
     }
 
-    if args.extra:
+    def side_figures(r2, c2, n2, m2, v2, w2, k2):
+        by = algorithmic_bytes(r2, c2, n2, m2, v2, w2["geo"].ksp)
+        fl = 2.0 * r2 * n2 * 2 * w2["geo"].ksp
+        t_hbm, t_mma = by / (HBM_PEAK_GBS * 1e9), fl / (SMFMAC_PEAK_TFLOPS * 1e12)
+        return {"shape": "%dx%dx%d %d:2:%d" % (r2, c2, n2, v2, m2), "kernel": w2["plan"].kernel_name(n2, 0, 0),
+                "us": round(k2 * 1e3, 2), "dense_equiv_tflops": round(2.0 * r2 * c2 * n2 / (k2 * 1e-3) / 1e12, 1),
+                "hbm_gbs": round(by / (k2 * 1e-3) / 1e9, 1), "hbm_frac": round(by / (k2 * 1e-3) / 1e9 / HBM_PEAK_GBS, 3),
+                "pct_smfmac_peak": round(100 * fl / (k2 * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2),
+                "bound": "mfma" if t_mma > t_hbm else "hbm"}
+
+    if not args.no_extra:
+        # the two compute-bound workloads, so that the default line carries them: the 2:4 baseline on the FFN-up shape and
+        # the GPT-3 feed-forward matrix at 2048 tokens (each: 100 ms settle, 10 warm-up, 30 timed launches)
         extra = []
+        for (r2, c2, n2, m2, v2) in [(4096, 1024, 16384, 4, 128), (49152, 12288, 2048, 16, 128)]:
+            w2 = prepare(r2, c2, n2, m2, v2)
+            _, k2 = timed(w2, 30, 10, settle_ms=100.0)
+            extra.append(side_figures(r2, c2, n2, m2, v2, w2, k2))
+            del w2
+        out["extra"] = extra
+
+    if args.extra:
+        extra = out.get("extra", [])
         for (r2, c2, n2, m2, v2) in [(1024, 4096, 16384, 8, 64), (1024, 1024, 16384, 8, 64), (4096, 1024, 16384, 8, 128),
-                                     (1024, 4096, 4096, 8, 128), (4096, 1024, 16384, 4, 128),
+                                     (1024, 4096, 4096, 8, 128), (4096, 1024, 16384, 4, 64),
                                      (4096, 1024, 16384, 16, 64), (4096, 1024, 16384, 32, 64)]:
             w2 = prepare(r2, c2, n2, m2, v2)
-            _, k2 = timed(w2, 100, 200)
-            by = algorithmic_bytes(r2, c2, n2, m2, v2, w2["geo"].ksp)
-            extra.append({"shape": "%dx%dx%d %d:2:%d" % (r2, c2, n2, v2, m2), "us": round(k2 * 1e3, 2),
-                          "dense_equiv_tflops": round(2.0 * r2 * c2 * n2 / (k2 * 1e-3) / 1e12, 1),
-                          "hbm_gbs": round(by / (k2 * 1e-3) / 1e9, 1),
-                          "pct_smfmac_peak": round(100 * 2.0 * r2 * n2 * 2 * w2["geo"].ksp / (k2 * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2)})
+            _, k2 = timed(w2, 100, 20, settle_ms=100.0)
+            extra.append(side_figures(r2, c2, n2, m2, v2, w2, k2))
             del w2
         out["extra"] = extra
 
@@ -184,7 +219,7 @@ def main():
         w_id["plan"] = spatha.SpmmPlan(torch.from_numpy(w["vals"]).to(dev), torch.from_numpy(w["meta"].view(np.int32)).to(dev),
                                        torch.from_numpy(ident.view(np.int32)).to(dev), rows, cols, 2, m, v)
         _, k_id = timed(w_id, args.steps, args.warmup, args.variant)
-        _, k_nm = timed(w, args.steps, 50, args.variant)
+        _, k_nm = timed(w, args.steps, args.warmup, args.variant)
         out["ablation"] = {"column_loc_us": round(k_nm * 1e3, 2), "ideal_identity_column_loc_us": round(k_id * 1e3, 2),
                            "out_32b_stores_us": out32}      # null: libspatha_out32b.so has not been built
 
@@ -197,12 +232,8 @@ def main():
             gen.manual_seed(0)
             w2["B"] = torch.randn((c2, n2), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
             w2["C"] = torch.empty((r2, n2), dtype=torch.float16, device=dev)
-            _, k2 = timed(w2, 50, 100)
-            by = algorithmic_bytes(r2, c2, n2, m2, v2, w2["geo"].ksp)
-            gpt3.append({"shape": "%dx%dx%d %d:2:%d" % (r2, c2, n2, v2, m2), "kernel": w2["plan"].kernel_name(n2, 0, 0),
-                         "us": round(k2 * 1e3, 2), "dense_equiv_tflops": round(2.0 * r2 * c2 * n2 / (k2 * 1e-3) / 1e12, 1),
-                         "hbm_gbs": round(by / (k2 * 1e-3) / 1e9, 1), "hbm_frac": round(by / (k2 * 1e-3) / 1e9 / HBM_PEAK_GBS, 3),
-                         "pct_smfmac_peak": round(100 * 2.0 * r2 * n2 * 2 * w2["geo"].ksp / (k2 * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2)})
+            _, k2 = timed(w2, 50, 20, settle_ms=100.0)
+            gpt3.append(side_figures(r2, c2, n2, m2, v2, w2, k2))
         del w2
         out["gpt3"] = gpt3
 

@@ -76,6 +76,13 @@ def random_mask(rows, cols, n, m, v, mbrow=32):
     return meta, columns
 
 
+def shuffle(a):
+    """One draw of the generator's shuffle on the process-wide rand() stream (a copy of `a`, shuffled)."""
+    a = np.array(a, dtype=np.uint32)
+    lib().vo_shuffle(_p(a), int(a.size))
+    return a
+
+
 def fill_rand_ints(count):
     out = np.empty(count, np.float32)
     lib().vo_fill_rand_ints(_p(out), ctypes.c_long(count))

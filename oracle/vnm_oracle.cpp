@@ -19,9 +19,13 @@
 //   vo_decode         golden vectors, closed-form index maps
 //   vo_select_columns golden vectors incl. ties, brute force on tiny inputs
 //   vo_spmm_*         dense product of vo_decode(A) with B in float64 (numpy)
-//   vo_random_mask    invariants only (sorted distinct pairs / quadruples);
-//                     the exact rand() stream has no golden anywhere in the
-//                     reference: parity unpinned for the stream itself
+//   vo_random_mask    known answers for five shapes drawn from one stream,
+//                     derived without this file (tests/golden/
+//                     make_random_mask_kat.py: glibc's rand() and libstdc++'s
+//                     random_shuffle restated in Python, the draws walked in
+//                     the reference's order); that restatement of rand() is
+//                     held against the C library and shuffle_rand against the
+//                     real std::random_shuffle (a C++14 snippet the test builds)
 //   vo_half<->float   numpy.float16 conversion on all 65536 bit patterns
 //
 // Build: see oracle/build.py (g++ -O2 -fopenmp -shared).
@@ -330,6 +334,12 @@ int vo_sizes(int rows, int cols, int n, int m, int v, long* out4) {
 // vo_srand(1) first to start from glibc's default state.
 void vo_srand(unsigned seed) { std::srand(seed); }
 int vo_rand(void) { return std::rand(); }
+// one shuffle of a caller-held array, exposed so that the tests can hold it against libstdc++'s std::random_shuffle
+void vo_shuffle(unsigned* a, int len) {
+    std::vector<unsigned> v(a, a + len);
+    shuffle_rand(v);
+    std::copy(v.begin(), v.end(), a);
+}
 
 int vo_random_mask(int rows, int cols, int n, int m, int v, int mbrow, uint32_t* meta, uint32_t* columns) {
     Geometry g(rows, cols, n, m, v, 4, mbrow);

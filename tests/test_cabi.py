@@ -41,3 +41,35 @@ def test_spmm_entry_points_reject_bad_arguments_without_a_gpu():
     assert L.spatha_spmm_run(None, None, 8, None, None, 0, 0, None) == 1
     assert L.spatha_spmm_plan_destroy(None) == 0
     assert L.spatha_dense_gemm_f16(None, None, 8, 8, 8, None, None) == 1
+
+
+def test_unified_kernels_use_no_scratch_memory(tmp_path):
+    """The unified dense-staged kernels load operands into registers asynchronously (inline assembly, no wait at the
+    load); a register the compiler saves to scratch memory between such a load and its wait would hold a value that has
+    not arrived.  Every instantiation shipped in the library must therefore have a private segment of zero bytes (the
+    launcher checks the same at run time).  Read from the notes of the code objects embedded in libspatha.so."""
+    import shutil
+    import subprocess
+
+    import pytest
+
+    objdump, readelf = "/opt/rocm/llvm/bin/llvm-objdump", "/opt/rocm/llvm/bin/llvm-readelf"
+    if not (os.path.exists(objdump) and os.path.exists(readelf)):
+        pytest.skip("LLVM binary tools not present")
+    lib = tmp_path / "libspatha.so"
+    shutil.copy(_lib.LIB_PATH, lib)
+    subprocess.check_call([objdump, "--offloading", str(lib)], cwd=tmp_path, stdout=subprocess.DEVNULL)
+    found = {}
+    for f in sorted(os.listdir(tmp_path)):
+        if "amdgcn" not in f:
+            continue
+        notes = subprocess.check_output([readelf, "--notes", str(tmp_path / f)]).decode()
+        name = None
+        for line in notes.splitlines():
+            line = line.strip()
+            if line.startswith(".name:"):
+                name = line.split(":", 1)[1].strip()
+            elif line.startswith(".private_segment_fixed_size:") and name and "spmm_du_kernel" in name:
+                found[name] = int(line.split(":", 1)[1])
+    assert len(found) >= 4, found                 # two output layouts x (m <= 8, m <= 16)
+    assert all(size == 0 for size in found.values()), found

@@ -21,7 +21,7 @@ CONFIG1 = ("--sparsity-type n-to-m --spmm spatha --gemm cuBlas --precision half 
 
 REFERENCE_COLUMNS = ("algo,arch,m,k,n,meta_block_sz,block_sz,nn_row,mm_row,density,bm,bn,bk,wm,wn,wk,mm,mn,mk,nstage,"
                      "spmm_time,gemm_time,speedup,error").split(",")       # benchmark/run_ablation2.sh:12
-APPENDED_COLUMNS = "spmm_us,dense_equiv_tflops,pct_smfmac_peak,hbm_gbs,kernel,cpu_encode_decode_s,cpu_threads".split(",")
+APPENDED_COLUMNS = "spmm_us,dense_equiv_tflops,pct_smfmac_peak,hbm_gbs,kernel,cpu_encode_decode_s,cpu_threads,gemm_impl".split(",")
 
 
 def _run(args, timeout=300):
@@ -87,6 +87,7 @@ def test_config1_invocation_passes_its_own_check(gpu):
     want_tflops = 2.0 * 1024 * 4096 * 4096 / (spmm_ms * 1e-3) / 1e12
     assert abs(float(row["dense_equiv_tflops"]) - want_tflops) <= 0.01 * want_tflops
     assert row["kernel"].startswith("smfmac16x16x64_")
+    assert row["gemm_impl"] == "hipblaslt"            # the speed-up column is against the vendor library's dense GEMM
 
 
 @pytest.mark.gpu

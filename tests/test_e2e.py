@@ -77,6 +77,89 @@ def test_bert_encoder_swap_runs_and_tracks_masked_dense(gpu):
     assert (a - b).abs().max().item() <= 5e-2
 
 
+def _mask_encoder_linears(model, gpu):
+    """Gives the encoder Linears of a dense model the harness's fixed 2:8 pattern (entries 0 and 2 of every group)."""
+    for name, mod in model.named_modules():
+        if isinstance(mod, torch.nn.Linear) and "encoder.layer" in name:
+            w = mod.weight
+            kept = torch.zeros(8, device=gpu, dtype=w.dtype)
+            kept[0] = kept[2] = 1
+            mod.weight.copy_((w.reshape(w.shape[0], -1, 8) * kept).reshape(w.shape))
+    return model
+
+
+@pytest.mark.gpu
+def test_bert_large_full_size_tracks_masked_dense(gpu):
+    """The end-to-end configuration at full size: 24 layers, hidden 1024, 16 heads, feed-forward 4096, batch 32 x 512
+    token ids over a 30522-entry vocabulary, every encoder Linear in 64:2:8 through the SpMM operator, against the dense
+    fp16 model whose weights carry the same mask.  Both are fp16 evaluations of the same function; the tolerance is the
+    one of the two-layer test, on every element of the last hidden state."""
+    from venom_amd.bert import SrnmSpmm, build_bert_large, linear_to_spmm
+
+    torch.set_grad_enabled(False)
+    print("bert-large 24 layers, 32 x 512", flush=True)
+    sparse = linear_to_spmm(build_bert_large(layers=24).to(gpu).half(), 2, 8, 64)
+    assert sum(isinstance(mod, SrnmSpmm) for mod in sparse.modules()) == 24 * 6
+    g = torch.Generator(device=gpu)
+    g.manual_seed(0)
+    ids = torch.randint(0, 30522, (32, 512), device=gpu, generator=g)
+    a = sparse(ids).last_hidden_state.float()
+    del sparse
+    dense = _mask_encoder_linears(build_bert_large(layers=24).to(gpu).half(), gpu)
+    b = dense(ids).last_hidden_state.float()
+    assert a.shape == (32, 512, 1024) and torch.isfinite(a).all()
+    diff = (a - b).abs()
+    print("max abs difference %.4g, mean %.4g" % (diff.max().item(), diff.mean().item()), flush=True)
+    assert diff.max().item() <= 5e-2
+
+
+@pytest.mark.gpu
+def test_gpt3_block_swap_tracks_masked_dense(gpu):
+    """The GPT-3 block harness at reduced width (one GPT2Block, width 512, 8 heads, 1 x 256 tokens): its four Conv1D
+    projections become SpMM layers over the transposed weight, and the block tracks the dense block whose weights carry
+    the same mask.  128:2:16, the format of the GPT-3 feed-forward configuration."""
+    from transformers.pytorch_utils import Conv1D
+    from venom_amd.bert import SrnmSpmm
+    from venom_amd.gpt2 import conv1d_to_spmm
+    from venom_amd.gpt3 import build_gpt3_block
+
+    torch.set_grad_enabled(False)
+    width, heads, tokens, m = 512, 8, 256, 16
+    dense = build_gpt3_block(width, heads, tokens).half().to(gpu)
+    sparse = conv1d_to_spmm(build_gpt3_block(width, heads, tokens).half().to(gpu), 2, m, 128)
+    assert sum(isinstance(mod, SrnmSpmm) for mod in sparse.modules()) == 4
+    assert not any(isinstance(mod, Conv1D) for mod in sparse.modules())
+    shapes = sorted((mod.nrows_sp, mod.ncols_sp) for mod in sparse.modules() if isinstance(mod, SrnmSpmm))
+    assert shapes == sorted([(3 * width, width), (width, width), (4 * width, width), (width, 4 * width)])
+    for mod in dense.modules():
+        if isinstance(mod, Conv1D):
+            w = mod.weight                                   # [in, out]
+            kept = torch.zeros(m, device=gpu, dtype=w.dtype)
+            kept[0] = kept[2] = 1
+            wt = w.t().reshape(w.shape[1], -1, m) * kept
+            mod.weight.copy_(wt.reshape(w.shape[1], w.shape[0]).t())
+    x = torch.rand((1, tokens, width), device=gpu).half()
+    a = sparse(x)
+    b = dense(x)
+    a = (a[0] if isinstance(a, tuple) else a).float()
+    b = (b[0] if isinstance(b, tuple) else b).float()
+    assert a.shape == (1, tokens, width) and torch.isfinite(a).all()
+    assert (a - b).abs().max().item() <= 5e-2
+
+
+def test_gpt3_harness_prints_the_reference_rows(capsys):
+    """report_time of the GPT-3 harness: first field 2, then n, m (0, 0 for the dense row), V, mean, median, std, count
+    (end2end/gpt3_pytorch.py:144-159)."""
+    from venom_amd import gpt3
+
+    gpt3.report_time("n:m", [0.002, 0.004], 2, 16, 128)
+    gpt3.report_time("dense", [0.001], 2, 16, 128)
+    rows = capsys.readouterr().out.strip().splitlines()
+    f = rows[0].split(",")
+    assert f[:4] == ["2", "2", "16", "128"] and abs(float(f[4]) - 3.0) < 1e-9 and f[-1] == "2"
+    assert rows[1].split(",")[:4] == ["2", "0", "0", "128"]
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("rows,cols", [(64, 64), (200, 328), (16384, 1024), (8, 4104), (37, 50)])
 def test_transpose_matches_torch(gpu, rows, cols):

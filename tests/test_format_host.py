@@ -125,6 +125,21 @@ def test_random_pattern_equals_oracle_stream(rows, cols, m, v):
     assert np.array_equal(vals.astype(np.float32), ovals)
 
 
+def test_random_pattern_known_answers():
+    """The library's generator against answers derived without it and without the oracle: five matrices drawn one after
+    another from the C library's stream (tests/golden/make_random_mask_kat.py walks glibc's rand() and libstdc++'s
+    random_shuffle in the order of src/format/format_sr_nm.cpp:151-237)."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "random_mask_kat.json")) as f:
+        kat = json.load(f)
+    oracle.srand(1)
+    for c in kat:
+        meta, columns = F.random_pattern(c["rows"], c["cols"], 2, c["m"], c["v"])
+        assert np.array_equal(meta, np.array(c["metadata"], np.uint32)), (c["rows"], c["cols"])
+        assert np.array_equal(columns, np.array(c["columns"], np.uint32)), (c["rows"], c["cols"])
+
+
 def test_meta_blob_layout():
     meta = np.arange(1, 12, dtype=np.uint32)          # 11 words -> column-loc starts at word 16
     columns = np.arange(100, 105, dtype=np.uint32)

@@ -1,6 +1,7 @@
 """Pins the CPU oracle: golden vectors written by the reference's own Python host code,
 closed-form layout maps, brute force on tiny inputs, numpy for the arithmetic."""
 import itertools
+import os
 
 import numpy as np
 import pytest
@@ -157,3 +158,112 @@ def test_random_mask_invariants():
     full_tiles = (full // 4) * 4
     assert (lo[:, :full_tiles] < hi[:, :full_tiles]).all()
     assert (nib[:, full_tiles:] == 0).all()          # partial last tile stays zero when m divides cols
+
+
+# --- the random pattern generator's stream (src/format/format_sr_nm.cpp:151-237) ---------------------------------
+
+def _kat_module():
+    import importlib.util
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "make_random_mask_kat.py")
+    spec = importlib.util.spec_from_file_location("make_random_mask_kat", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_python_restatement_of_glibc_rand_equals_the_c_library():
+    """The known answers below rest on a pure-Python restatement of glibc's rand(); it must reproduce the C library's
+    stream after srand(1), which is also the stream of a process that never seeds (the reference never does)."""
+    import ctypes
+    libc = ctypes.CDLL(None)
+    libc.srand(1)
+    want = [libc.rand() for _ in range(5000)]
+    assert _kat_module().glibc_rand_stream(1, 5000) == want
+    assert want[:3] == [1804289383, 846930886, 1681692777]
+
+
+def test_shuffle_equals_libstdcxx_random_shuffle(tmp_path):
+    """The oracle's shuffle and the Python one against the real std::random_shuffle (removed in C++17, so a C++14
+    snippet built here), on arrays that persist from call to call as the generator's do."""
+    import subprocess
+    src = tmp_path / "rs.cpp"
+    src.write_text("""
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+int main() {
+    std::srand(1);
+    std::vector<unsigned> a{0, 1, 2, 3}, b{0, 1, 2, 3, 4, 5, 6, 7};
+    for (int t = 0; t < 200; t++) {
+        std::random_shuffle(a.begin(), a.end());
+        std::sort(a.begin(), a.begin() + 2);
+        for (unsigned x : a) std::printf("%u ", x);
+        std::random_shuffle(b.begin(), b.end());
+        std::sort(b.begin(), b.begin() + 4);
+        for (unsigned x : b) std::printf("%u ", x);
+        std::printf("\\n");
+    }
+    return 0;
+}
+""")
+    exe = tmp_path / "rs"
+    subprocess.check_call(["g++", "-std=c++14", "-O1", "-Wno-deprecated-declarations", "-o", str(exe), str(src)])
+    want = [[int(x) for x in line.split()] for line in subprocess.check_output([str(exe)]).decode().splitlines()]
+    assert len(want) == 200
+    oracle.srand(1)
+    a, b = np.arange(4, dtype=np.uint32), np.arange(8, dtype=np.uint32)
+    stream = _kat_module().Stream(1)
+    pa, pb = [0, 1, 2, 3], list(range(8))
+    for row in want:
+        a = oracle.shuffle(a); a[:2] = np.sort(a[:2])
+        b = oracle.shuffle(b); b[:4] = np.sort(b[:4])
+        stream.shuffle(pa); pa[:2] = sorted(pa[:2])
+        stream.shuffle(pb); pb[:4] = sorted(pb[:4])
+        assert list(a) + list(b) == row and pa + pb == row
+
+
+def test_random_mask_known_answers():
+    """32 x 32, 2:8, V = 32, first matrix of a process (stream position 0).  Hand walk of the first word
+    (format_sr_nm.cpp:157-177; glibc rand() after srand(1) = 1804289383, 846930886, 1681692777, 1714636915, 1957747793,
+    424238335, 719885386, 1649760492, 596516649, ...; a shuffle of {a0..a3} swaps a1 with a[r % 2], a2 with a[r % 3],
+    a3 with a[r % 4]):
+      group 0: {0,1,2,3}: 1804289383 % 2 = 1 (no swap), 846930886 % 3 = 1 -> {0,2,1,3}, 1681692777 % 4 = 1 -> {0,3,1,2};
+               first two sorted = (0, 3) -> bits 0b1100 = 0xC
+      group 1: {0,3,1,2}: 1714636915 % 2 = 1, 1957747793 % 3 = 2, 424238335 % 4 = 3: no swap; pair (0, 3) -> 0xC
+      group 2: {0,3,1,2}: 719885386 % 2 = 0 -> {3,0,1,2}, 1649760492 % 3 = 0 -> {1,0,3,2}, 596516649 % 4 = 1 -> {1,2,3,0};
+               pair (1, 2) -> 1 | 2 << 2 = 0x9
+    so the word ends in ...9CC, and 16 words x 8 groups x 3 draws = 384 draws precede the column-loc draws
+    (:213-229), whose first shuffle of {0..7} uses draws 384..390 and leaves (1, 3, 4, 5) in front."""
+    oracle.srand(1)
+    meta, columns = oracle.random_mask(32, 32, 2, 8, 32)
+    assert [hex(int(w)) for w in meta[:4]] == ["0xd89e99cc", "0xcdc9dd4d", "0xed8ed4c9", "0x9c448ee9"]
+    assert int(meta[15]) == 0xEDC494E9 and not meta[16:].any()       # the second tile of the padded row stays zero
+    assert columns.reshape(-1, 4)[:4].tolist() == [[1, 3, 4, 5], [1, 3, 4, 6], [1, 3, 4, 6], [1, 5, 6, 7]]
+    assert not columns.reshape(-1, 4)[4:].any()
+
+
+def test_random_mask_stream_over_consecutive_matrices():
+    """Five matrices drawn one after another from one stream (complete tiles, complete groups beyond the last tile,
+    K % m != 0 tails, m = 16, plain 2:4, several 32-row and V-row blocks) against answers derived without the oracle
+    (tests/golden/make_random_mask_kat.py)."""
+    import json
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "random_mask_kat.json")) as f:
+        kat = json.load(f)
+    assert len(kat) == 5
+    oracle.srand(1)
+    for c in kat:
+        meta, columns = oracle.random_mask(c["rows"], c["cols"], 2, c["m"], c["v"])
+        assert np.array_equal(meta, np.array(c["metadata"], np.uint32)), c["rows"]
+        assert np.array_equal(columns, np.array(c["columns"], np.uint32)), c["rows"]
+    # the stream has advanced by exactly the number of draws the walk counts
+    import ctypes
+    libc = ctypes.CDLL(None)
+    libc.srand(1)
+    for _ in range(kat[-1]["draws_after"]):
+        libc.rand()
+    want_next = libc.rand()
+    oracle.srand(1)
+    for c in kat:
+        oracle.random_mask(c["rows"], c["cols"], 2, c["m"], c["v"])
+    assert oracle.lib().vo_rand() == want_next

@@ -302,8 +302,13 @@ def test_config1_gaussian_within_tolerance(gpu):
     assert (np.abs(got[:, :256] - want) / np.maximum(np.abs(exact[:, :256]), 1.0)).max() <= REL_TOL
 
 
-@pytest.mark.parametrize("rows,cols,N,m,v", [(4096, 1024, 16384, 8, 64), (1024, 4096, 16384, 8, 64),
-                                             (4096, 1024, 16384, 4, 128), (1024, 1024, 16384, 32, 128)])
+# every cell of the sparsity sweep on the BERT-large linear shapes (A in {1024 x 1024, 4096 x 1024, 1024 x 4096},
+# 16384 columns of B, V in {64, 128}, 2:M with M in {8, 16, 32}) plus the plain 2:4 baseline on the feed-forward shape
+SWEEP_CELLS = [(r, c, 16384, m, v) for (r, c) in ((1024, 1024), (4096, 1024), (1024, 4096)) for v in (64, 128)
+               for m in (8, 16, 32)] + [(4096, 1024, 16384, 4, 128), (4096, 1024, 16384, 4, 64)]
+
+
+@pytest.mark.parametrize("rows,cols,N,m,v", SWEEP_CELLS)
 def test_full_size_checksums(gpu, rows, cols, N, m, v):
     """BERT-large shapes at full size: row sums and column sums of C against products the CPU
     can afford (C 1 = A (B 1), 1^T C = (1^T A) B), exact for small integers."""
@@ -329,10 +334,12 @@ def test_full_size_checksums(gpu, rows, cols, N, m, v):
     assert torch.equal(Ct.t(), C)
 
 
-@pytest.mark.parametrize("N", [16, 256])
+@pytest.mark.parametrize("N", [16, 256, 2048])
 def test_gpt3_ffn_shape_blocks_within_tolerance(gpu, N):
     """GPT-3 feed-forward shape: A 49152 x 12288 in 128:2:16, values ~N(0, 0.02), B ~N(0, 1); N = 16 runs on the skinny
-    kernel.  Three V-row blocks of C are compared with the float64 product of their decoded rows."""
+    kernel, N = 2048 is the compute-bound end.  Three V-row blocks of C are compared with the float64 product of their
+    decoded rows."""
+    print("gpt3 ffn", N, flush=True)
     rows, cols, m, v = 49152, 12288, 16, 128
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=0, value_std=0.02)
     g = F.geometry(rows, cols, 2, m, v)
@@ -350,6 +357,45 @@ def test_gpt3_ffn_shape_blocks_within_tolerance(gpu, N):
         want = dense @ Bh
         got = C[b * v:(b + 1) * v].cpu().numpy().astype(np.float64)
         assert (np.abs(got - want) / np.maximum(np.abs(want), 1.0)).max() <= REL_TOL
+
+
+K_TAIL_CASES = [
+    # rows, cols, N, m, v : cols % (16 m) != 0, so the last k-step of a dense-staged kernel spans rows beyond K
+    (1024, 200, 264, 8, 64),
+    (512, 650, 136, 10, 64),
+    (256, 100, 72, 8, 64),
+    (512, 200, 136, 8, 32),
+    (768, 450, 264, 7, 192),
+]
+
+
+@pytest.mark.parametrize("rows,cols,N,m,v", K_TAIL_CASES)
+def test_rows_beyond_k_are_never_read(gpu, rows, cols, N, m, v):
+    """B is the leading part of a larger fp16 buffer whose remainder is filled with NaN (0x7E00).  A kernel that stages
+    dense B rows must not fetch the rows of its last k-step that lie beyond K: they multiply zero-valued operands, and
+    0 * NaN = NaN would show in every output of the tile.  Every kernel that takes the shape must match the oracle bit
+    for bit."""
+    print("k tail", rows, cols, N, m, v, flush=True)
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=rows + N, integer_values=True)
+    rng = np.random.default_rng(N)
+    B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B)
+    guard_rows = 16 * m + 64                      # more than one k-step of dense rows
+    big = torch.full(((cols + guard_rows) * N,), float("nan"), dtype=torch.float16, device=gpu)
+    big[:cols * N] = _dev(B, gpu).reshape(-1)
+    dB = big[:cols * N].view(cols, N)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    ran = 0
+    for variant in range(spatha.num_variants()):
+        name = plan.kernel_name(N, 0, variant)
+        if name is None:
+            continue
+        ran += 1
+        print("   variant", variant, name, flush=True)
+        got = plan.run(dB, variant=variant)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16)), (variant, name)
+    assert ran >= 3
 
 
 def test_linearity_in_B(gpu):

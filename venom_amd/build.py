@@ -35,23 +35,38 @@ def _run(cmd, verbose):
     subprocess.check_call(cmd)
 
 
-def build(verbose=False, with_driver=True):
+def _compile_all(jobs, verbose):
+    """Runs the compile commands side by side (the kernel file takes a minute, the others seconds)."""
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
+        for f in [pool.submit(_run, cmd, verbose) for cmd in jobs]:
+            f.result()
+
+
+def build(verbose=False, with_driver=True, with_out_32b=False):
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
-    objs = []
+    objs, jobs = [], []
     for src in CXX_SOURCES:
         obj = os.path.join(OBJDIR, src + ".o")
-        _run(["g++"] + CXX_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj], verbose)
+        jobs.append(["g++"] + CXX_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
         objs.append(obj)
     for src in HIP_SOURCES:
         obj = os.path.join(OBJDIR, src + ".o")
         lang = ["-x", "hip"] if src.endswith(".hip") else []
-        _run([HIPCC] + HIP_FLAGS + lang + ["-c", os.path.join(CSRC, src), "-o", obj], verbose)
+        jobs.append([HIPCC] + HIP_FLAGS + lang + ["-c", os.path.join(CSRC, src), "-o", obj])
         objs.append(obj)
+    if with_out_32b:
+        jobs.append(_out_32b_compile())
+    _compile_all(jobs, verbose)
+    if with_out_32b:
+        _out_32b_link(verbose)
     _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB] + objs + ["-lgomp"], verbose)
     if with_driver and os.path.exists(os.path.join(CSRC, "benchmark_spmm.cpp")):
-        _run([HIPCC] + HIP_FLAGS + [os.path.join(CSRC, "benchmark_spmm.cpp"), "-o", BENCH, "-L" + LIBDIR, "-lspatha",
-                                    "-Wl,-rpath,$ORIGIN", "-lgomp"], verbose)
+        # the driver alone links the vendor GEMM (hipBLASLt), the baseline of its gemm_time / speedup columns
+        _run([HIPCC] + HIP_FLAGS + [os.path.join(CSRC, "benchmark_spmm.cpp"), os.path.join(CSRC, "vendor_gemm.cpp"), "-o", BENCH,
+                                    "-L" + LIBDIR, "-lspatha", "-Wl,-rpath,$ORIGIN", "-L/opt/rocm/lib", "-lhipblaslt", "-lgomp"],
+             verbose)
     return LIB
 
 
@@ -59,16 +74,23 @@ def build_out_32b(verbose=False):
     """The OUT_32B ablation build (the reference's compile-time switch of that name, CMakeLists.txt:25-33): the same
     library with every 16-byte row-major store of C issued as four 4-byte stores -> venom_amd/lib/libspatha_out32b.so.
     Needs the objects of a normal build; `SPATHA_LIBRARY=<that file>` makes the Python binding load it."""
+    _run(_out_32b_compile(), verbose)
+    return _out_32b_link(verbose)
+
+
+def _out_32b_compile():
+    obj = os.path.join(OBJDIR, "spmm_kernels.out32b.o")
+    return [HIPCC] + HIP_FLAGS + ["-DSPATHA_OUT_32B", "-x", "hip", "-c", os.path.join(CSRC, "spmm_kernels.hip"), "-o", obj]
+
+
+def _out_32b_link(verbose):
     lib = os.path.join(LIBDIR, "libspatha_out32b.so")
     obj = os.path.join(OBJDIR, "spmm_kernels.out32b.o")
-    _run([HIPCC] + HIP_FLAGS + ["-DSPATHA_OUT_32B", "-x", "hip", "-c", os.path.join(CSRC, "spmm_kernels.hip"), "-o", obj], verbose)
     objs = [os.path.join(OBJDIR, s + ".o") for s in CXX_SOURCES + HIP_SOURCES if s != "spmm_kernels.hip"] + [obj]
     _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", lib] + objs + ["-lgomp"], verbose)
     return lib
 
 
 if __name__ == "__main__":
-    build(verbose=True)
-    if "--ablation" in sys.argv[1:]:
-        build_out_32b(verbose=True)
+    build(verbose=True, with_out_32b="--ablation" in sys.argv[1:])
     sys.exit(0)

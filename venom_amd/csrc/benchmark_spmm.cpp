@@ -16,7 +16,11 @@
 //   spmm_code,arch,m,k,n,meta_block_sz,block_sz,nn_row,mm_row,density,bm,bn,bk,wm,wn,wk,mm,mn,mk,
 //   nstage,spmm_time_ms,gemm_time_ms,speedup,error
 // followed by appended columns: spmm_us,dense_equiv_tflops,pct_smfmac_peak,hbm_gbs,kernel,
-//   cpu_encode_decode_s,cpu_threads
+//   cpu_encode_decode_s,cpu_threads,gemm_impl
+// gemm_time_ms / speedup are against the vendor library's dense fp16 GEMM (hipBLASLt; the reference's column is
+// against cuBLAS, src/gemm/cublas_gemm.cpp:54-96); gemm_impl says which GEMM was timed ("hipblaslt", or "in-tree"
+// when the vendor library has no kernel for the shape).  --check always compares with the library's own exact
+// dense product (spatha_dense_gemm_f16).
 
 #include <hip/hip_runtime_api.h>
 
@@ -31,6 +35,7 @@
 #include <vector>
 
 #include "../../include/spatha.h"
+#include "vendor_gemm.h"
 
 namespace {
 
@@ -179,11 +184,18 @@ int main(int argc, const char** argv) {
         }
     }
 
-    // ---- host format conversion, timed: decode (the dense operand of the check) and re-encode
+    // ---- host format conversion, timed: decode (the dense operand of the check) and re-encode of that dense matrix
+    //      (non-zero driven, as the reference's init_from_dense does, src/format/format_sr_nm.cpp:108-149)
     const int threads = (int)std::thread::hardware_concurrency();
     std::vector<uint16_t> hDense((size_t)m * k);
     auto t0 = std::chrono::steady_clock::now();
     SPATHA_OK_OR_DIE(spatha_vnm_decode_f16(hVal.data(), hMeta.data(), hCols.data(), m, k, nn_row, mm_row, V, hDense.data(), 0));
+    {
+        std::vector<uint16_t> reVal((size_t)geo.n_values);
+        std::vector<uint32_t> reMeta((size_t)geo.n_metadata, 0u);
+        SPATHA_OK_OR_DIE(spatha_vnm_encode_f16(hDense.data(), nullptr, hCols.data(), m, k, nn_row, mm_row, V, reVal.data(),
+                                               reMeta.data(), 0));
+    }
     double cpu_convert_s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
 
     // ---- device
@@ -227,20 +239,39 @@ int main(int argc, const char** argv) {
     // ---- timing: 10 warm-up + 100 timed launches between two events (src/cuda_utils.h:61-87)
     float spmm_ms = 0.f;
     SPATHA_OK_OR_DIE(spatha_spmm_time(plan, dB, n, nullptr, dC, SPATHA_OUT_ROW_MAJOR, variant, 11, 100, nullptr, &spmm_ms));
+    // dense baseline: the vendor GEMM, 10 warm-up + 100 timed launches like the SpMM (into a buffer of its own);
+    // the exact in-tree product that --check compares with is computed afterwards
     float gemm_ms = 0.f;
+    const char* gemm_impl = "hipblaslt";
     {
         hipEvent_t e0, e1;
         HIP_OK(hipEventCreate(&e0));
         HIP_OK(hipEventCreate(&e1));
-        for (int i = 0; i < 3; i++) SPATHA_OK_OR_DIE(spatha_dense_gemm_f16(dDense, dB, m, kpad, n, dCref, nullptr));
-        const int reps = 20;
+        VendorGemm* vg = vendor_gemm_create(m, kpad, n);
+        uint16_t* dCvendor = nullptr;
+        if (vg) HIP_OK(hipMalloc((void**)&dCvendor, (size_t)m * n * 2));
+        auto run_gemm = [&]() {
+            if (vg) {
+                if (vendor_gemm_run(vg, dDense, dB, dCvendor, nullptr) != 0) die("hipBLASLt matmul failed");
+            } else {
+                SPATHA_OK_OR_DIE(spatha_dense_gemm_f16(dDense, dB, m, kpad, n, dCref, nullptr));
+            }
+        };
+        if (!vg) gemm_impl = "in-tree";
+        const int reps = vg ? 100 : 20;
+        for (int i = 0; i < (vg ? 10 : 3); i++) run_gemm();
         HIP_OK(hipEventRecord(e0, nullptr));
-        for (int i = 0; i < reps; i++) SPATHA_OK_OR_DIE(spatha_dense_gemm_f16(dDense, dB, m, kpad, n, dCref, nullptr));
+        for (int i = 0; i < reps; i++) run_gemm();
         HIP_OK(hipEventRecord(e1, nullptr));
         HIP_OK(hipEventSynchronize(e1));
         HIP_OK(hipEventElapsedTime(&gemm_ms, e0, e1));
         gemm_ms /= reps;
+        vendor_gemm_destroy(vg);
+        if (dCvendor) (void)hipFree(dCvendor);
+        HIP_OK(hipEventDestroy(e0));
+        HIP_OK(hipEventDestroy(e1));
     }
+    if (check) SPATHA_OK_OR_DIE(spatha_dense_gemm_f16(dDense, dB, m, kpad, n, dCref, nullptr));
 
     int error = 0;
     if (check) {
@@ -265,8 +296,8 @@ int main(int argc, const char** argv) {
     std::printf("%d,%s,%d,%d,%d,%d,%d,%d,%d,%g,%d,%d,%d,%d,%d,%d,%d,%d,%d,%d,%g,%g,%g,%d", spmm_code, "gfx950", m, k, n,
                 meta_block_sz, block_sz, nn_row, mm_row, (double)density, bm, bn, bk, wm, wn, wk, mm, mn, mk, nstage,
                 spmm_ms, gemm_ms, gemm_ms / spmm_ms, error);
-    std::printf(",%.3f,%.1f,%.2f,%.1f,%s,%.4f,%d\n", spmm_ms * 1e3, flops_dense / t / 1e12, 100.0 * flops_sparse / t / 5.033e15,
-                bytes / t / 1e9, kname, cpu_convert_s, threads);
+    std::printf(",%.3f,%.1f,%.2f,%.1f,%s,%.4f,%d,%s\n", spmm_ms * 1e3, flops_dense / t / 1e12, 100.0 * flops_sparse / t / 5.033e15,
+                bytes / t / 1e9, kname, cpu_convert_s, threads, gemm_impl);
 
     spatha_spmm_plan_destroy(plan);
     for (void* ptr : {(void*)dB, (void*)dC, (void*)dCref, (void*)dVal, (void*)dMeta, (void*)dCols, (void*)dDense}) (void)hipFree(ptr);

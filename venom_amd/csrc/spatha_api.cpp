@@ -14,20 +14,7 @@
 #include "spmm_kernels.h"
 #include "vnm_format.h"
 
-struct spatha_spmm_plan {
-    spatha_vnm_geometry geo;
-    int S;                 // k-steps of 64 compressed B rows
-    int half_tiles;        // V % 64 != 0: operands packed in the order of the half-tile kernels
-    int device;
-    int cus;               // compute units of that device
-    uint16_t* apack;
-    uint32_t* rowtab;
-    void* zeros;           // 1 KiB of zeros on the device
-    uint16_t* gtab;        // gather table of the dense-staged kernels (m <= 8, rows % 256 == 0), or null
-    uint16_t* gtab_tiles;  // tile-major copy for the flag-synchronised kernel
-    size_t gtab_tiles_bytes, gtab_bytes;
-    size_t apack_bytes, rowtab_bytes;
-};
+#include "spatha_internal.h"
 
 namespace {
 thread_local int g_last_hip_error = 0;
@@ -42,7 +29,7 @@ bool variant_has_fused_writeout(int variant) {
     using namespace spatha;
     return (variant >= SPMM_VARIANT_P128x128_S4 && variant <= SPMM_VARIANT_W64x256_S3) ||      // pipelined, persistent, wave-specialised
            (variant >= SPMM_VARIANT_T128x256_S3 && variant <= SPMM_VARIANT_DS256x128_S3_C8) ||
-           variant == SPMM_VARIANT_DSH256x128_S3_C8 || variant == SPMM_VARIANT_DU512x128_S4;
+           variant == SPMM_VARIANT_DSH256x128_S3_C8;
 }
 
 bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = false) {
@@ -69,7 +56,8 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = f
         return false;
     }
     if (variant == SPMM_VARIANT_DU512x128_S4) {
-        if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 512 != 0 || !plan->gtab || plan->half_tiles) return false;
+        if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 512 != 0 || !plan->gtab || plan->half_tiles || fused)
+            return false;
         if (plan->gtab_bytes >= 0xE0000000ull) return false;
     }
     if (variant == SPMM_VARIANT_DU512x128_M16) {
@@ -219,6 +207,44 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
 }
 }  // namespace
 
+namespace spatha {
+
+int note_hip_error(hipError_t e) { return hip_fail(e); }
+
+void plan_layout(int rows, int m, int v, int ksp, PlanLayout* out) {
+    out->S = (ksp + 31) / 32;
+    out->half_tiles = (v % 64 != 0);      // V = 32, 96, ...: a wave tile spans two V blocks
+    out->apack_bytes = (size_t)(rows / 64) * out->S * APACK_BLOCK;
+    out->rowtab_bytes = (size_t)(rows / v) * out->S * 64 * 4;
+    out->gtab_bytes = 0;
+    out->gtab_tiles_bytes = 0;
+    if ((m <= 8 && rows % 256 == 0) || (m <= 16 && rows % 512 == 0 && !out->half_tiles)) {
+        // gather table of the dense-staged kernels: one entry per 64-row block, or per 32-row block when V % 64 != 0
+        const int block_rows = out->half_tiles ? 32 : 64;
+        out->gtab_bytes = (size_t)(rows / block_rows) * out->S * 64 * 2;
+    }
+    if (v % 64 == 0 && m <= 8 && rows % 256 == 0) out->gtab_tiles_bytes = (size_t)(rows / 256) * out->S * 512;
+}
+
+hipError_t plan_pack(const spatha_spmm_plan* plan, const uint16_t* values_dev, const uint32_t* metadata_dev,
+                     const uint32_t* columns_dev, hipStream_t stream) {
+    const spatha_vnm_geometry& geo = plan->geo;
+    hipError_t e = launch_pack(values_dev, metadata_dev, columns_dev, geo.rows, geo.cols, geo.m, geo.v, geo.ksp, plan->S,
+                               plan->half_tiles, plan->apack, plan->rowtab, stream);
+    if (e != hipSuccess) return e;
+    if (plan->gtab) {
+        e = launch_pack_gtab(columns_dev, geo.rows, geo.m, geo.v, geo.ksp, plan->S, plan->half_tiles ? 32 : 64, plan->gtab, stream);
+        if (e != hipSuccess) return e;
+    }
+    if (plan->gtab_tiles) {
+        e = launch_pack_gtab_tiles(columns_dev, geo.rows, geo.m, geo.v, geo.ksp, plan->S, plan->gtab_tiles, stream);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+}  // namespace spatha
+
 extern "C" {
 
 const char* spatha_status_string(int status) {
@@ -343,47 +369,27 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     if (e != hipSuccess || ndev == 0) { g_last_hip_error = (int)e; return SPATHA_ERR_NO_DEVICE; }
     spatha_spmm_plan* plan = new (std::nothrow) spatha_spmm_plan();
     if (!plan) return SPATHA_ERR_BAD_ARGUMENT;
+    spatha::PlanLayout lay;
+    spatha::plan_layout(rows, m, v, geo.ksp, &lay);
     plan->geo = geo;
-    plan->S = (geo.ksp + 31) / 32;
-    plan->half_tiles = (v % 64 != 0);      // V = 32, 96, ...: a wave tile spans two V blocks
-    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr; plan->gtab_tiles = nullptr; plan->gtab_tiles_bytes = 0; plan->gtab_bytes = 0;
+    plan->S = lay.S;
+    plan->half_tiles = lay.half_tiles;
+    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr; plan->gtab_tiles = nullptr;
+    plan->apack_bytes = lay.apack_bytes; plan->rowtab_bytes = lay.rowtab_bytes;
+    plan->gtab_bytes = lay.gtab_bytes; plan->gtab_tiles_bytes = lay.gtab_tiles_bytes;
     e = hipGetDevice(&plan->device);
     if (e != hipSuccess) { delete plan; return hip_fail(e); }
     plan->cus = 0;
     if (hipDeviceGetAttribute(&plan->cus, hipDeviceAttributeMultiprocessorCount, plan->device) != hipSuccess) plan->cus = 0;
-    const size_t a_bytes = (size_t)(rows / 64) * plan->S * spatha::APACK_BLOCK;
-    const size_t r_bytes = (size_t)(rows / v) * plan->S * 64 * 4;
-    plan->apack_bytes = a_bytes; plan->rowtab_bytes = r_bytes;
-    if ((e = hipMalloc((void**)&plan->apack, a_bytes)) != hipSuccess ||
-        (e = hipMalloc((void**)&plan->rowtab, r_bytes)) != hipSuccess ||
+    if ((e = hipMalloc((void**)&plan->apack, lay.apack_bytes)) != hipSuccess ||
+        (e = hipMalloc((void**)&plan->rowtab, lay.rowtab_bytes)) != hipSuccess ||
         (e = hipMalloc(&plan->zeros, 1024)) != hipSuccess ||
-        (e = hipMemsetAsync(plan->zeros, 0, 1024, (hipStream_t)stream)) != hipSuccess) {
+        (e = hipMemsetAsync(plan->zeros, 0, 1024, (hipStream_t)stream)) != hipSuccess ||
+        (lay.gtab_bytes && (e = hipMalloc((void**)&plan->gtab, lay.gtab_bytes)) != hipSuccess) ||
+        (lay.gtab_tiles_bytes && (e = hipMalloc((void**)&plan->gtab_tiles, lay.gtab_tiles_bytes)) != hipSuccess) ||
+        (e = spatha::plan_pack(plan, values_dev, metadata_dev, columns_dev, (hipStream_t)stream)) != hipSuccess) {
         spatha_spmm_plan_destroy(plan);
         return hip_fail(e);
-    }
-    e = spatha::launch_pack(values_dev, metadata_dev, columns_dev, rows, cols, m, v, geo.ksp, plan->S, plan->half_tiles,
-                            plan->apack, plan->rowtab, (hipStream_t)stream);
-    if (e != hipSuccess) { spatha_spmm_plan_destroy(plan); return hip_fail(e); }
-    if ((m <= 8 && rows % 256 == 0) || (m <= 16 && rows % 512 == 0 && !plan->half_tiles)) {
-        // gather table of the dense-staged kernels: one entry per 64-row block, or per 32-row block when V % 64 != 0
-        const int block_rows = plan->half_tiles ? 32 : 64;
-        const size_t g_bytes = (size_t)(rows / block_rows) * plan->S * 64 * 2;
-        plan->gtab_bytes = g_bytes;
-        if ((e = hipMalloc((void**)&plan->gtab, g_bytes)) != hipSuccess ||
-            (e = spatha::launch_pack_gtab(columns_dev, rows, m, v, geo.ksp, plan->S, block_rows, plan->gtab,
-                                          (hipStream_t)stream)) != hipSuccess) {
-            spatha_spmm_plan_destroy(plan);
-            return hip_fail(e);
-        }
-    }
-    if (v % 64 == 0 && m <= 8 && rows % 256 == 0) {
-        plan->gtab_tiles_bytes = (size_t)(rows / 256) * plan->S * 512;
-        if ((e = hipMalloc((void**)&plan->gtab_tiles, plan->gtab_tiles_bytes)) != hipSuccess ||
-            (e = spatha::launch_pack_gtab_tiles(columns_dev, rows, m, v, geo.ksp, plan->S, plan->gtab_tiles,
-                                                (hipStream_t)stream)) != hipSuccess) {
-            spatha_spmm_plan_destroy(plan);
-            return hip_fail(e);
-        }
     }
     *out = plan;
     return SPATHA_OK;
@@ -401,8 +407,10 @@ int spatha_spmm_plan_destroy(spatha_spmm_plan* plan) {
     return first == hipSuccess ? SPATHA_OK : hip_fail(first);
 }
 
-static int run_spmm(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, uint16_t* out_dev,
-                    int out_layout, int activation, bool fused_entry, int variant, void* stream) {
+}  // extern "C"
+
+int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, uint16_t* out_dev,
+                     int out_layout, int activation, bool fused_entry, int variant, void* stream) {
     if (!plan || !B_dev || !out_dev || N <= 0) return SPATHA_ERR_BAD_ARGUMENT;
     if (out_layout != SPATHA_OUT_ROW_MAJOR && out_layout != SPATHA_OUT_TRANSPOSED) return SPATHA_ERR_BAD_ARGUMENT;
     if (!fused_entry && out_layout == SPATHA_OUT_ROW_MAJOR && bias_dev) return SPATHA_ERR_BAD_ARGUMENT;
@@ -440,14 +448,16 @@ static int run_spmm(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
     return e == hipSuccess ? SPATHA_OK : hip_fail(e);
 }
 
+extern "C" {
+
 int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
                     uint16_t* out_dev, int out_layout, int variant, void* stream) {
-    return run_spmm(plan, B_dev, N, bias_dev, out_dev, out_layout, SPATHA_ACT_NONE, false, variant, stream);
+    return spatha::plan_run(plan, B_dev, N, bias_dev, out_dev, out_layout, SPATHA_ACT_NONE, false, variant, stream);
 }
 
 int spatha_spmm_run_fused(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
                           uint16_t* out_dev, int out_layout, int activation, int variant, void* stream) {
-    return run_spmm(plan, B_dev, N, bias_dev, out_dev, out_layout, activation, true, variant, stream);
+    return spatha::plan_run(plan, B_dev, N, bias_dev, out_dev, out_layout, activation, true, variant, stream);
 }
 
 int spatha_spmm_num_variants(void) { return spatha::SPMM_VARIANT_COUNT; }

@@ -960,6 +960,12 @@ __device__ __forceinline__ i32x4 make_buffer(const void* base, uint32_t bytes) {
     r.w = 0x00020000;
     return r;
 }
+// Descriptor of the part of a buffer that starts `off` bytes in (off is wave-uniform).  The range check of a raw buffer
+// compares the vector offset (plus the instruction's immediate) with the record count and leaves the scalar offset
+// out, so a window that moves through the buffer is expressed here, in base and count, never as a scalar offset.
+__device__ __forceinline__ i32x4 buffer_window(const void* base, uint32_t bytes, uint32_t off) {
+    return make_buffer((const char*)base + off, off < bytes ? bytes - off : 0u);
+}
 __device__ __forceinline__ void bdma_b128(uint32_t voff, i32x4 rsrc, uint32_t soff, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc),
                  "s"(soff)
@@ -2061,8 +2067,9 @@ __device__ __forceinline__ void store_block_transposed_slab4(const float4_t (&ac
 // consumer picks its V block's 4-of-m rows through the ADDRESSES of its transposing reads:
 // gtab holds, per (64-row block, k-step, lane class), the LDS byte offset of the row a lane has to
 // read for each of its four fragments (row * 256 + swizzle), built once per matrix.
-// Rows beyond K come back as zeros from the buffer bounds check, so padding groups (whose
-// column offsets are 0) and tail groups need no special case.
+// Rows beyond K come back as zeros from the buffer range check (the producers' descriptor is the
+// window of B that starts at the step's first row, so the check sees the row's true distance from
+// the end of B), so padding groups (whose column offsets are 0) and tail groups need no special case.
 // With four consumer waves, wave w owns rows 128*(w/2) .. +127 (two 64-row blocks) x columns
 // 64*(w%2) .. +63; with eight, rows 64*(w/2) .. +63 (two waves per SIMD hide each other's LDS
 // latency and barrier waits).  Producers need no row table: B rows are consecutive.
@@ -2128,8 +2135,10 @@ __device__ __forceinline__ void ds_producer(const SpmmParams& p, const TileWalk&
     set_voff();
     auto issue_batch = [&]() {
         const uint32_t stage = smem_base + is_stage;
+        // the step's window of B: rows of the step that lie beyond K fail the range check and arrive as zeros
+        const i32x4 rsrc_step = buffer_window(p.B, p.b_bytes, b_soff);
 #pragma unroll
-        for (int j = 0; j < NB_LOADS; j++) bdma_b128(voff[j], rsrc_b, b_soff, stage + (PR * NB_LOADS + j) * 1024);
+        for (int j = 0; j < NB_LOADS; j++) bdma_b128(voff[j], rsrc_step, 0, stage + (PR * NB_LOADS + j) * 1024);
 #pragma unroll
         for (int k = 0; k < NA_LOADS; k++) {
             const int a = PR * NA_LOADS + k;
@@ -2813,11 +2822,12 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
         }
     };
     set_voff();
-    uint32_t dma_stage = 0, dma_soff = 0;         // target and source offset of the stage being issued
+    uint32_t dma_stage = 0;                       // target of the stage being issued
+    i32x4 dma_rsrc = rsrc_b;                      // its window of B (rows of the step beyond K fail the range check: zeros)
     uint32_t dma_voff[NB];
     auto stage_begin = [&]() {                    // fixes the addresses of the next stage and advances the cursor
         dma_stage = smem_base + is_stage + wave * (NB * 1024);
-        dma_soff = b_soff;
+        dma_rsrc = buffer_window(p.B, p.b_bytes, b_soff);
 #pragma unroll
         for (int j = 0; j < NB; j++) dma_voff[j] = voff[j];
         is_stage = (is_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : is_stage + STAGE_BYTES;
@@ -2829,7 +2839,7 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
             set_voff();
         }
     };
-    auto stage_op = [&](int j) { bdma_b128(dma_voff[j], rsrc_b, dma_soff, dma_stage + j * 1024); };
+    auto stage_op = [&](int j) { bdma_b128(dma_voff[j], dma_rsrc, 0, dma_stage + j * 1024); };
     auto issue_stage = [&]() {
         stage_begin();
 #pragma unroll
@@ -3026,7 +3036,14 @@ static hipError_t launch_du(const SpmmParams& p, hipStream_t stream) {
     void (*kern)(SpmmParams) = spmm_du_kernel<OUT_LAYOUT, FUSE, M_>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        // The kernel's register loads complete asynchronously into named variables; a compiler-made copy of such a
+        // variable to scratch memory between the load and its wait would save a value that has not arrived.  An
+        // instantiation with any scratch memory is therefore refused.
+        hipFuncAttributes fa;
+        hipError_t e = hipFuncGetAttributes(&fa, (const void*)kern);
+        if (e != hipSuccess) return e;
+        if (fa.localSizeBytes != 0) return hipErrorNotSupported;
+        e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
         int dev = 0;
         if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
@@ -3147,8 +3164,9 @@ __device__ __forceinline__ void dsf_producer(const SpmmParams& p, const TileWalk
         }
         if (!SPATHA_KNOB(8)) {
             const uint32_t stage = smem_base + st * STAGE_BYTES;
+            const i32x4 rsrc_step = buffer_window(p.B, p.b_bytes, b_soff);      // rows of the step beyond K: zeros
 #pragma unroll
-            for (int j = 0; j < NB_LOADS; j++) bdma_b128(voff[j], rsrc_b, b_soff, stage + (PR * NB_LOADS + j) * 1024);
+            for (int j = 0; j < NB_LOADS; j++) bdma_b128(voff[j], rsrc_step, 0, stage + (PR * NB_LOADS + j) * 1024);
 #pragma unroll
             for (int k = 0; k < NA_LOADS; k++) {
                 const int a = PR * NA_LOADS + k;
@@ -3882,13 +3900,17 @@ hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStre
     if (variant == SPMM_VARIANT_DSH256x128_S3_C8)
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_ds<8, 3, 4, 8, SPATHA_OUT_TRANSPOSED, false, true>(p, stream)
                                                    : launch_ds<8, 3, 4, 8, SPATHA_OUT_ROW_MAJOR, false, true>(p, stream);
-    if (variant == SPMM_VARIANT_DU512x128_S4)
-        return out_layout == SPATHA_OUT_TRANSPOSED
-                   ? (p.fuse ? launch_du<SPATHA_OUT_TRANSPOSED, true>(p, stream) : launch_du<SPATHA_OUT_TRANSPOSED, false>(p, stream))
-                   : (p.fuse ? launch_du<SPATHA_OUT_ROW_MAJOR, true>(p, stream) : launch_du<SPATHA_OUT_ROW_MAJOR, false>(p, stream));
-    if (variant == SPMM_VARIANT_DU512x128_M16)
+    // (no fused write-out: that instantiation needs scratch memory, which the kernel's asynchronous register loads rule out)
+    if (variant == SPMM_VARIANT_DU512x128_S4) {
+        if (p.fuse) return hipErrorNotSupported;
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_du<SPATHA_OUT_TRANSPOSED, false>(p, stream)
+                                                   : launch_du<SPATHA_OUT_ROW_MAJOR, false>(p, stream);
+    }
+    if (variant == SPMM_VARIANT_DU512x128_M16) {
+        if (p.fuse) return hipErrorNotSupported;
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_du<SPATHA_OUT_TRANSPOSED, false, 16>(p, stream)
                                                    : launch_du<SPATHA_OUT_ROW_MAJOR, false, 16>(p, stream);
+    }
     if (variant == SPMM_VARIANT_DSF256x128_S3)
         return out_layout == SPATHA_OUT_TRANSPOSED ? launch_dsf<8, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream)
                                                    : launch_dsf<8, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);

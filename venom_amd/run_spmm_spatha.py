@@ -16,7 +16,7 @@ import sys
 from . import _lib
 
 HEADER = ("algo,arch,m,k,n,meta_block_sz,block_sz,nn_row,mm_col,density,bm,bn,bk,wm,wn,wk,mm,mn,mk,nstage,"
-          "spmm_time,gemm_time,speedup,error,spmm_us,tflops_dense_equiv,pct_sparse_peak,gbs,kernel,convert_s,threads")
+          "spmm_time,gemm_time,speedup,error,spmm_us,tflops_dense_equiv,pct_sparse_peak,gbs,kernel,convert_s,threads,gemm_impl")
 # (rows, cols) of the linear layers: BERT-base 768 / 3072, BERT-large 1024 / 4096 (run_spmm_spatha.sh:12-30)
 LAYERS = [(768, 768), (3072, 768), (768, 3072), (1024, 1024), (4096, 1024), (1024, 4096)]
 M_VALUES = [4, 7, 8, 10, 20, 40, 100]

@@ -183,6 +183,19 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
 int spatha_spmm_run_fused(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
                           uint16_t* out_dev, int out_layout, int activation, int variant, void* stream);
 
+/* One SpMM straight from the canonical arrays, for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same result as
+ * spatha_spmm_plan_create + spatha_spmm_run (automatic kernel choice) + spatha_spmm_plan_destroy on the same arguments,
+ * but the derived copies of A that a plan would hipMalloc live in a fixed 8 MiB array in device memory that belongs to
+ * the library (each GPU the library runs on holds its own copy until the process ends), and the call allocates and
+ * frees nothing: it launches the pack kernels and the SpMM kernel on `stream`.  A matrix whose derived copies exceed
+ * the array is refused with SPATHA_ERR_TOO_LARGE (the array holds e.g. 4096 x 1024 or 1024 x 4096 at 2:8 and
+ * 4096 x 1024 at 2:4).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race; calls ordered on one stream do not. */
+int spatha_spmm_run_noalloc(int rows, int cols, int n, int m, int v, const uint16_t* values_dev,
+                            const uint32_t* metadata_dev, const uint32_t* columns_dev, const uint16_t* B_dev, int N,
+                            const uint16_t* bias_dev, uint16_t* out_dev, int out_layout, void* stream);
+
 /* Kernel variants are numbered 1 .. spatha_spmm_num_variants() - 1; 0 selects automatically. */
 int spatha_spmm_num_variants(void);
 

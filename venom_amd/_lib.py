@@ -46,6 +46,8 @@ SIGNATURES = {
     "spatha_spmm_plan_destroy": (c_int, [c_void_p]),
     "spatha_spmm_run": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "spatha_spmm_run_fused": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "spatha_spmm_run_noalloc": (c_int, [c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                        c_void_p, c_int, c_void_p]),
     "spatha_spmm_num_variants": (c_int, []),
     "spatha_spmm_kernel_name": (c_char_p, [c_void_p, c_int, c_int, c_int]),
     "spatha_spmm_time": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, POINTER(c_float)]),

@@ -25,7 +25,8 @@ HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Xclang", 
              "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fopenmp", "-Wall"]
 
-HIP_SOURCES = ["spmm_kernels.hip", "dense_gemm.hip", "transpose.hip", "layernorm.hip", "select_gpu.hip", "spatha_api.cpp"]
+HIP_SOURCES = ["spmm_kernels.hip", "dense_gemm.hip", "transpose.hip", "layernorm.hip", "select_gpu.hip", "spmm_static.hip",
+               "spatha_api.cpp"]
 CXX_SOURCES = ["vnm_format.cpp"]
 
 

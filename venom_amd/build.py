@@ -25,8 +25,10 @@ HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Xclang", 
              "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fopenmp", "-Wall"]
 
-HIP_SOURCES = ["spmm_kernels.hip", "dense_gemm.hip", "transpose.hip", "layernorm.hip", "select_gpu.hip", "spmm_static.hip",
-               "spatha_api.cpp"]
+# the SpMM kernels, one source per family (spmm_device.h holds what they share)
+KERNEL_SOURCES = ["spmm_gathered.hip", "spmm_warpspec.hip", "spmm_densestage.hip", "spmm_unified.hip", "spmm_skinny.hip"]
+HIP_SOURCES = KERNEL_SOURCES + ["spmm_pack.hip", "spmm_dispatch.hip", "dense_gemm.hip", "transpose.hip", "layernorm.hip",
+                                "select_gpu.hip", "spmm_static.hip", "spatha_api.cpp"]
 CXX_SOURCES = ["vnm_format.cpp"]
 
 
@@ -58,7 +60,7 @@ def build(verbose=False, with_driver=True, with_out_32b=False):
         jobs.append([HIPCC] + HIP_FLAGS + lang + ["-c", os.path.join(CSRC, src), "-o", obj])
         objs.append(obj)
     if with_out_32b:
-        jobs.append(_out_32b_compile())
+        jobs += _out_32b_compile()
     _compile_all(jobs, verbose)
     if with_out_32b:
         _out_32b_link(verbose)
@@ -75,19 +77,18 @@ def build_out_32b(verbose=False):
     """The OUT_32B ablation build (the reference's compile-time switch of that name, CMakeLists.txt:25-33): the same
     library with every 16-byte row-major store of C issued as four 4-byte stores -> venom_amd/lib/libspatha_out32b.so.
     Needs the objects of a normal build; `SPATHA_LIBRARY=<that file>` makes the Python binding load it."""
-    _run(_out_32b_compile(), verbose)
+    _compile_all(_out_32b_compile(), verbose)
     return _out_32b_link(verbose)
 
 
 def _out_32b_compile():
-    obj = os.path.join(OBJDIR, "spmm_kernels.out32b.o")
-    return [HIPCC] + HIP_FLAGS + ["-DSPATHA_OUT_32B", "-x", "hip", "-c", os.path.join(CSRC, "spmm_kernels.hip"), "-o", obj]
+    return [[HIPCC] + HIP_FLAGS + ["-DSPATHA_OUT_32B", "-x", "hip", "-c", os.path.join(CSRC, src), "-o",
+                                   os.path.join(OBJDIR, src + ".out32b.o")] for src in KERNEL_SOURCES]
 
 
 def _out_32b_link(verbose):
     lib = os.path.join(LIBDIR, "libspatha_out32b.so")
-    obj = os.path.join(OBJDIR, "spmm_kernels.out32b.o")
-    objs = [os.path.join(OBJDIR, s + ".o") for s in CXX_SOURCES + HIP_SOURCES if s != "spmm_kernels.hip"] + [obj]
+    objs = [os.path.join(OBJDIR, s + (".out32b.o" if s in KERNEL_SOURCES else ".o")) for s in CXX_SOURCES + HIP_SOURCES]
     _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", lib] + objs + ["-lgomp"], verbose)
     return lib
 

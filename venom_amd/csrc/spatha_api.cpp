@@ -27,9 +27,25 @@ inline int hip_fail(hipError_t e) {
 // kernels whose write-out can apply bias and activation ahead of either output layout
 bool variant_has_fused_writeout(int variant) {
     using namespace spatha;
-    return (variant >= SPMM_VARIANT_P128x128_S4 && variant <= SPMM_VARIANT_W64x256_S3) ||      // pipelined, persistent, wave-specialised
-           (variant >= SPMM_VARIANT_T128x256_S3 && variant <= SPMM_VARIANT_DS256x128_S3_C8) ||
-           variant == SPMM_VARIANT_DSH256x128_S3_C8;
+    switch (variant) {
+        case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_R64x256_S3:
+        case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x256_S3: case SPMM_VARIANT_W64x256_S3:
+        case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DSH256x128_S3_C8:
+            return true;
+        default:
+            return false;
+    }
+}
+
+// kernels that address B, the packed operands and the tables through buffer descriptors (32-bit offsets)
+bool variant_uses_buffer_descriptors(int variant) {
+    using namespace spatha;
+    switch (variant) {
+        case SPMM_VARIANT_128x128: case SPMM_VARIANT_64x256: case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P64x256_S2:
+            return false;
+        default:
+            return true;
+    }
 }
 
 bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = false) {
@@ -41,38 +57,29 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = f
     const bool half_variant = variant == SPMM_VARIANT_H64x256_S2 || variant == SPMM_VARIANT_H64x128_S3 ||
                               variant == SPMM_VARIANT_H64x128_S2 || variant == SPMM_VARIANT_DSH256x128_S3_C8;
     if (half_variant != (plan->half_tiles != 0)) return false;       // the packed operand order differs
+    const uint64_t b_bytes = (uint64_t)plan->geo.cols * (uint64_t)N * 2u;
     if (variant == SPMM_VARIANT_DSH256x128_S3_C8) {
         if (plan->geo.m > 8 || plan->geo.rows % 256 != 0 || !plan->gtab) return false;
-        const uint64_t bb = (uint64_t)plan->geo.cols * (uint64_t)N * 2u;       // 32-bit buffer offsets
-        return bb < 0xE0000000ull && plan->apack_bytes < 0xE0000000ull;
+        return b_bytes < 0xE0000000ull && plan->apack_bytes < 0xE0000000ull;
     }
     if (half_variant) return plan->geo.cols <= 65535 && spmm_variant_lds(variant, plan->S) <= 160 * 1024;
-    if (variant == SPMM_VARIANT_DS256x128_S3 || variant == SPMM_VARIANT_DS256x128_S2 ||
-        variant == SPMM_VARIANT_DS256x128_S3_C8 || variant == SPMM_VARIANT_DS256x128_S3_PP ||
-        variant == SPMM_VARIANT_DSF256x128_S3) {
+    const bool unified = variant == SPMM_VARIANT_DU512x128_S4 || variant == SPMM_VARIANT_DU512x128_M16;
+    if (variant == SPMM_VARIANT_DS256x128_S3_C8 || variant == SPMM_VARIANT_DS256x128_S3_PP) {
         // four 64-row blocks per tile; all 16*m dense rows of a k-step must fit one stage
         if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 256 != 0 || !plan->gtab) return false;
-    } else if (variant != SPMM_VARIANT_DU512x128_S4 && variant != SPMM_VARIANT_DU512x128_M16 && plan->geo.v % bm != 0) {
+    } else if (unified) {
+        // no fused write-out (that instantiation would need scratch memory)
+        if (plan->geo.v % 64 != 0 || plan->geo.rows % 512 != 0 || !plan->gtab || plan->half_tiles || fused) return false;
+        if (variant == SPMM_VARIANT_DU512x128_S4 ? plan->geo.m > 8 : (plan->geo.m <= 8 || plan->geo.m > 16)) return false;
+        if (plan->gtab_bytes >= 0xE0000000ull) return false;
+    } else if (plan->geo.v % bm != 0) {
         return false;
-    }
-    if (variant == SPMM_VARIANT_DU512x128_S4) {
-        if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 512 != 0 || !plan->gtab || plan->half_tiles || fused)
-            return false;
-        if (plan->gtab_bytes >= 0xE0000000ull) return false;
-    }
-    if (variant == SPMM_VARIANT_DU512x128_M16) {
-        if (plan->geo.v % 64 != 0 || plan->geo.m <= 8 || plan->geo.m > 16 || plan->geo.rows % 512 != 0 || !plan->gtab ||
-            plan->half_tiles || fused)
-            return false;
-        if (plan->gtab_bytes >= 0xE0000000ull) return false;
     }
     if (variant == SPMM_VARIANT_SKINNY && N > 64) return false;
     if (spmm_variant_lds(variant, plan->S) > 160 * 1024) return false;      // row table kept in LDS
-    if (variant >= SPMM_VARIANT_R128x128_S4) {
-        // buffer-descriptor kernels address B, the packed operands and the row table with 32-bit offsets
-        const uint64_t bb = (uint64_t)plan->geo.cols * (uint64_t)N * 2u;
-        if (bb >= 0xE0000000ull || plan->apack_bytes >= 0xE0000000ull || plan->rowtab_bytes >= 0xE0000000ull) return false;
-    }
+    if (variant_uses_buffer_descriptors(variant) &&
+        (b_bytes >= 0xE0000000ull || plan->apack_bytes >= 0xE0000000ull || plan->rowtab_bytes >= 0xE0000000ull))
+        return false;
     return true;
 }
 
@@ -217,13 +224,11 @@ void plan_layout(int rows, int m, int v, int ksp, PlanLayout* out) {
     out->apack_bytes = (size_t)(rows / 64) * out->S * APACK_BLOCK;
     out->rowtab_bytes = (size_t)(rows / v) * out->S * 64 * 4;
     out->gtab_bytes = 0;
-    out->gtab_tiles_bytes = 0;
     if ((m <= 8 && rows % 256 == 0) || (m <= 16 && rows % 512 == 0 && !out->half_tiles)) {
         // gather table of the dense-staged kernels: one entry per 64-row block, or per 32-row block when V % 64 != 0
         const int block_rows = out->half_tiles ? 32 : 64;
         out->gtab_bytes = (size_t)(rows / block_rows) * out->S * 64 * 2;
     }
-    if (v % 64 == 0 && m <= 8 && rows % 256 == 0) out->gtab_tiles_bytes = (size_t)(rows / 256) * out->S * 512;
 }
 
 hipError_t plan_pack(const spatha_spmm_plan* plan, const uint16_t* values_dev, const uint32_t* metadata_dev,
@@ -234,10 +239,6 @@ hipError_t plan_pack(const spatha_spmm_plan* plan, const uint16_t* values_dev, c
     if (e != hipSuccess) return e;
     if (plan->gtab) {
         e = launch_pack_gtab(columns_dev, geo.rows, geo.m, geo.v, geo.ksp, plan->S, plan->half_tiles ? 32 : 64, plan->gtab, stream);
-        if (e != hipSuccess) return e;
-    }
-    if (plan->gtab_tiles) {
-        e = launch_pack_gtab_tiles(columns_dev, geo.rows, geo.m, geo.v, geo.ksp, plan->S, plan->gtab_tiles, stream);
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -374,9 +375,9 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     plan->geo = geo;
     plan->S = lay.S;
     plan->half_tiles = lay.half_tiles;
-    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr; plan->gtab_tiles = nullptr;
+    plan->apack = nullptr; plan->rowtab = nullptr; plan->zeros = nullptr; plan->gtab = nullptr;
     plan->apack_bytes = lay.apack_bytes; plan->rowtab_bytes = lay.rowtab_bytes;
-    plan->gtab_bytes = lay.gtab_bytes; plan->gtab_tiles_bytes = lay.gtab_tiles_bytes;
+    plan->gtab_bytes = lay.gtab_bytes;
     e = hipGetDevice(&plan->device);
     if (e != hipSuccess) { delete plan; return hip_fail(e); }
     plan->cus = 0;
@@ -386,7 +387,6 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
         (e = hipMalloc(&plan->zeros, 1024)) != hipSuccess ||
         (e = hipMemsetAsync(plan->zeros, 0, 1024, (hipStream_t)stream)) != hipSuccess ||
         (lay.gtab_bytes && (e = hipMalloc((void**)&plan->gtab, lay.gtab_bytes)) != hipSuccess) ||
-        (lay.gtab_tiles_bytes && (e = hipMalloc((void**)&plan->gtab_tiles, lay.gtab_tiles_bytes)) != hipSuccess) ||
         (e = spatha::plan_pack(plan, values_dev, metadata_dev, columns_dev, (hipStream_t)stream)) != hipSuccess) {
         spatha_spmm_plan_destroy(plan);
         return hip_fail(e);
@@ -402,7 +402,6 @@ int spatha_spmm_plan_destroy(spatha_spmm_plan* plan) {
     if (plan->rowtab && (e = hipFree(plan->rowtab)) != hipSuccess && first == hipSuccess) first = e;
     if (plan->zeros && (e = hipFree(plan->zeros)) != hipSuccess && first == hipSuccess) first = e;
     if (plan->gtab && (e = hipFree(plan->gtab)) != hipSuccess && first == hipSuccess) first = e;
-    if (plan->gtab_tiles && (e = hipFree(plan->gtab_tiles)) != hipSuccess && first == hipSuccess) first = e;
     delete plan;
     return first == hipSuccess ? SPATHA_OK : hip_fail(first);
 }
@@ -427,7 +426,6 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
     spatha::SpmmParams p;
     p.apack = plan->apack; p.rowtab = plan->rowtab;
     p.B = B_dev; p.bias = bias_dev; p.C = out_dev; p.zeros = plan->zeros; p.gtab = plan->gtab;
-    p.gtab_tiles = plan->gtab_tiles; p.gtab_tiles_bytes = (uint32_t)plan->gtab_tiles_bytes;
     p.gtab_bytes = (uint32_t)plan->gtab_bytes;
     p.rows = plan->geo.rows; p.cols = plan->geo.cols; p.N = N; p.S = plan->S; p.v = plan->geo.v; p.m = plan->geo.m;
     const int bm = spatha::spmm_variant_bm(var), bn = spatha::spmm_variant_bn(var);

@@ -17,8 +17,7 @@ struct spatha_spmm_plan {
     uint32_t* rowtab;
     void* zeros;           // 1 KiB of zeros on the device
     uint16_t* gtab;        // gather table of the dense-staged kernels (m <= 8, rows % 256 == 0), or null
-    uint16_t* gtab_tiles;  // tile-major copy for the flag-synchronised kernel
-    size_t gtab_tiles_bytes, gtab_bytes;
+    size_t gtab_bytes;
     size_t apack_bytes, rowtab_bytes;
 };
 
@@ -27,7 +26,7 @@ namespace spatha {
 // sizes of a plan's derived copies (a size of 0: the copy is not made for this shape)
 struct PlanLayout {
     int S, half_tiles;
-    size_t apack_bytes, rowtab_bytes, gtab_bytes, gtab_tiles_bytes;
+    size_t apack_bytes, rowtab_bytes, gtab_bytes;
 };
 void plan_layout(int rows, int m, int v, int ksp, PlanLayout* out);
 

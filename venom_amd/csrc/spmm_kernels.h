@@ -14,8 +14,6 @@ struct SpmmParams {
     const uint16_t* apack;    // packed A operands + sparse-index words, APACK_BLOCK bytes per (64 rows, k-step)
     const uint32_t* rowtab;   // gathered B row per LDS row
     const uint16_t* gtab;     // dense-staged kernels: LDS offset per (64-row block, step, lane class, fragment), or null
-    const uint16_t* gtab_tiles;  // the same table, tile-major (512 B per 256-row tile and step), or null
-    uint32_t gtab_tiles_bytes;
     uint32_t gtab_bytes;      // size of gtab (buffer descriptor of the unified dense-staged kernel)
     const uint16_t* B;        // cols x N, row-major
     const uint16_t* bias;     // rows, or null
@@ -34,45 +32,30 @@ struct SpmmParams {
 
 enum {
     SPMM_VARIANT_AUTO = 0,
-    SPMM_VARIANT_128x128 = 1,      // register-staged, 2 LDS stages
+    // gathered B stages (any m)
+    SPMM_VARIANT_128x128 = 1,           // register-staged, 2 LDS stages: first kernel, fallback
     SPMM_VARIANT_64x256 = 2,
-    SPMM_VARIANT_P128x128_S4 = 3,  // direct-to-LDS pipeline
-    SPMM_VARIANT_P128x128_S3 = 4,
-    SPMM_VARIANT_P64x256_S2 = 5,
-    SPMM_VARIANT_P64x256_S3 = 6,
-    SPMM_VARIANT_P128x128_S6 = 7,
-    SPMM_VARIANT_P64x256_S4 = 8,
-    SPMM_VARIANT_R128x128_S4 = 9,  // persistent, pipeline runs across tiles
-    SPMM_VARIANT_R128x128_S5 = 10,
-    SPMM_VARIANT_R128x128_S2 = 11,
-    SPMM_VARIANT_R64x256_S3 = 12,
-    SPMM_VARIANT_R64x256_S4 = 13,
-    SPMM_VARIANT_W128x128_S5 = 14,  // persistent + producer/consumer wave specialisation
-    SPMM_VARIANT_W128x128_S3 = 15,
-    SPMM_VARIANT_W128x128_S2 = 16,
-    SPMM_VARIANT_W128x256_S3 = 17,
-    SPMM_VARIANT_W64x256_S2 = 18,
-    SPMM_VARIANT_W64x256_S3 = 19,
-    SPMM_VARIANT_D128x256_S3 = 20,  // wave-specialised + write-out deferred into the next tile
-    SPMM_VARIANT_D128x128_S3 = 21,
-    SPMM_VARIANT_D128x128_S5 = 22,
-    SPMM_VARIANT_D64x256_S3 = 23,
-    SPMM_VARIANT_T128x256_S3 = 24,  // wave-specialised, each consumer wave owns 128 x 64
-    SPMM_VARIANT_T128x128_S4 = 25,
-    SPMM_VARIANT_T128x128_S5 = 26,
-    SPMM_VARIANT_DS256x128_S3 = 27,  // m <= 8: all 16*m dense B rows of a k-step staged once for four 64-row blocks
-    SPMM_VARIANT_DS256x128_S2 = 28,
-    SPMM_VARIANT_DS256x128_S3_C8 = 29,  // eight 64 x 64 consumer waves (two per SIMD)
-    SPMM_VARIANT_DS256x128_S3_PP = 30,  // eight consumers in two phase groups (ping-pong)
-    SPMM_VARIANT_DSF256x128_S3 = 31,    // dense-staged, LDS flag counters instead of workgroup barriers
-    SPMM_VARIANT_SKINNY = 32,           // N <= 64: one 64-row tile per workgroup, k split over four waves, B straight from L2
-    SPMM_VARIANT_H64x256_S2 = 33,       // V % 64 != 0: a 64-row tile spans two V blocks, two gathered B sets per stage
-    SPMM_VARIANT_H64x128_S3 = 34,
-    SPMM_VARIANT_H64x128_S2 = 35,
-    SPMM_VARIANT_DSH256x128_S3_C8 = 36, // V % 64 != 0, m <= 8: dense-staged B, two gather-table entries per consumer wave
-    SPMM_VARIANT_DU512x128_S4 = 37,     // m <= 8, rows % 512 == 0: eight unified 64 x 128 waves, A operands in registers, only B staged
-    SPMM_VARIANT_DU512x128_M16 = 38,    // the same for 8 < m <= 16: 64 KB stages, two of them
-    SPMM_VARIANT_COUNT = 39
+    SPMM_VARIANT_P128x128_S3 = 3,       // global -> LDS DMA pipeline, 3 stages
+    SPMM_VARIANT_P64x256_S2 = 4,
+    SPMM_VARIANT_R64x256_S3 = 5,        // persistent: the pipeline runs across tile boundaries
+    SPMM_VARIANT_W128x128_S3 = 6,       // persistent + producer / consumer waves
+    SPMM_VARIANT_W128x256_S3 = 7,
+    SPMM_VARIANT_W64x256_S3 = 8,
+    SPMM_VARIANT_D64x256_S3 = 9,        // ... with the write-out deferred into the next tile's steps
+    SPMM_VARIANT_T128x256_S3 = 10,      // ... each consumer wave owns 128 x 64
+    // dense-staged B (m <= 8): all 16 m dense rows of a k-step staged once for the tile's 64-row blocks
+    SPMM_VARIANT_DS256x128_S3_C8 = 11,  // eight 64 x 64 consumer waves + four producers
+    SPMM_VARIANT_DS256x128_S3_PP = 12,  // the eight consumers in two phase groups
+    SPMM_VARIANT_SKINNY = 13,           // N <= 64: one 64-row tile per workgroup, k split over four waves, B straight from L2
+    // V % 64 != 0: a 64-row tile spans two V blocks
+    SPMM_VARIANT_H64x256_S2 = 14,       // two gathered B sets per stage
+    SPMM_VARIANT_H64x128_S3 = 15,
+    SPMM_VARIANT_H64x128_S2 = 16,
+    SPMM_VARIANT_DSH256x128_S3_C8 = 17, // m <= 8: dense-staged B, two gather-table entries per consumer wave
+    // unified waves, A operands in registers, only B staged (rows % 512 == 0)
+    SPMM_VARIANT_DU512x128_S4 = 18,     // m <= 8
+    SPMM_VARIANT_DU512x128_M16 = 19,    // 8 < m <= 16: 64 KB stages, two of them
+    SPMM_VARIANT_COUNT = 20
 };
 
 const char* spmm_variant_name(int variant);
@@ -81,6 +64,14 @@ int spmm_variant_bn(int variant);
 int spmm_variant_lds(int variant, int S);
 
 hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
+
+// one launch switch per kernel family (spmm_gathered.hip, spmm_warpspec.hip, spmm_densestage.hip, spmm_unified.hip,
+// spmm_skinny.hip); hipErrorInvalidValue for an id of another family
+hipError_t launch_gathered(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
+hipError_t launch_warpspec(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
+hipError_t launch_densestage(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
+hipError_t launch_unified(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
+hipError_t launch_skinny_family(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
                        int m, int v, int ksp, int S, int half_tiles, uint16_t* apack, uint32_t* rowtab, hipStream_t stream);
@@ -96,9 +87,6 @@ hipError_t launch_select_winners(const float* dense_abs_dev, int rows, int cols,
 
 hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, int block_rows, uint16_t* gtab,
                             hipStream_t stream);
-
-hipError_t launch_pack_gtab_tiles(const uint32_t* columns, int rows, int m, int v, int ksp, int S, uint16_t* gtab,
-                                  hipStream_t stream);
 
 hipError_t launch_transpose_f16(const uint16_t* in, int rows, int cols, uint16_t* out, hipStream_t stream);
 hipError_t launch_add_layernorm_f16(const uint16_t* x, const uint16_t* residual, const uint16_t* gamma, const uint16_t* beta,

@@ -59,12 +59,11 @@ extern "C" int spatha_spmm_run_noalloc(int rows, int cols, int n, int m, int v, 
     if (rows % 64 != 0) return SPATHA_ERR_UNSUPPORTED;
     spatha::PlanLayout lay;
     spatha::plan_layout(rows, m, v, geo.ksp, &lay);
-    // [zeros 1 KiB][packed operands][row table][gather table][tile-major gather table], each at a multiple of 256 bytes
+    // [zeros 1 KiB][packed operands][row table][gather table], each at a multiple of 256 bytes
     const size_t off_apack = 1024;
     const size_t off_rowtab = off_apack + align256(lay.apack_bytes);
     const size_t off_gtab = off_rowtab + align256(lay.rowtab_bytes);
-    const size_t off_gtiles = off_gtab + align256(lay.gtab_bytes);
-    const size_t need = off_gtiles + align256(lay.gtab_tiles_bytes);
+    const size_t need = off_gtab + align256(lay.gtab_bytes);
     if (need > SCRATCH_BYTES) return SPATHA_ERR_TOO_LARGE;      // the matrix's derived copies do not fit the fixed array
 
     int ndev = 0, dev = -1;
@@ -86,9 +85,8 @@ extern "C" int spatha_spmm_run_noalloc(int rows, int cols, int n, int m, int v, 
     plan.apack = (uint16_t*)(base + off_apack);
     plan.rowtab = (uint32_t*)(base + off_rowtab);
     plan.gtab = lay.gtab_bytes ? (uint16_t*)(base + off_gtab) : nullptr;
-    plan.gtab_tiles = lay.gtab_tiles_bytes ? (uint16_t*)(base + off_gtiles) : nullptr;
     plan.apack_bytes = lay.apack_bytes; plan.rowtab_bytes = lay.rowtab_bytes;
-    plan.gtab_bytes = lay.gtab_bytes; plan.gtab_tiles_bytes = lay.gtab_tiles_bytes;
+    plan.gtab_bytes = lay.gtab_bytes;
 
     // The array keeps what the last call left: the block of zeros is cleared again, everything else is rewritten in
     // full by the pack kernels (every byte the SpMM kernels read for this shape).

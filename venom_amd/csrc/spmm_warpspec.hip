@@ -1,0 +1,544 @@
+// Producer / consumer kernels on gathered B stages: consumer waves only read LDS and issue matrix instructions,
+// producer waves only compute addresses and issue the global -> LDS DMA.
+
+#include "spmm_device.h"
+
+namespace spatha {
+
+// ---------------------------------------------------------------------------
+// Warp-specialised persistent SpMM kernel.
+//
+// The workgroup has NC = WM*WN consumer waves and NP producer waves.  Consumers do nothing
+// but read operands from LDS and issue sparse matrix instructions (and write finished tiles);
+// producers do nothing but address arithmetic and DMA issue for the stages NS-1 k-steps
+// ahead.  A wave can issue roughly one instruction every few cycles, so keeping the
+// bookkeeping out of the consumers' instruction stream is what lets their matrix pipe stay
+// busy.  One workgroup barrier per k-step joins the two roles:
+//   producer: wait own DMA of stage q | barrier | issue stage q + NS-1
+//   consumer:                           barrier | multiply stage q
+// Producer pr stands in for the wave (wm = pr / 2, wn = pr % 2) of the 2 x 2 arrangement when
+// it comes to which DMA instructions of a stage it issues.
+// ---------------------------------------------------------------------------
+
+template <class Cfg, int NP, int PR>
+__device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk& walk, char* smem, uint32_t smem_base,
+                                            int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1, PA = Cfg::PA;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int WM = BM / 64;
+    constexpr int CHUNKS = BN / 8;
+    constexpr int RPI = 1024 / ROW_BYTES;
+    constexpr int NB_LOADS = 64 / RPI / NP;          // B DMA instructions per producer per stage
+    constexpr int A_INSTR = WM * 6;                  // per wave-tile row: 4 operand blocks + 2 index blocks
+    constexpr int NA_LOADS = A_INSTR / NP;
+    constexpr int LOADS = NB_LOADS + NA_LOADS + 1;
+    static_assert(64 % (RPI * NP) == 0 && A_INSTR % NP == 0, "DMA work must split evenly over the producers");
+    static_assert((PA - 1) * LOADS < 64, "vmcnt range");
+
+    const int S = p.S, N = p.N;
+    const int Q = walk.my_tiles * S;
+    const int tiles_per_vblock = p.v / BM;
+    const i32x4 rsrc_b = make_buffer(p.B, p.b_bytes);
+    const i32x4 rsrc_a = make_buffer(p.apack, p.apack_bytes);
+    const i32x4 rsrc_rt = make_buffer(p.rowtab, p.rowtab_bytes);
+    const uint32_t row_bytes_b = (uint32_t)N * 2u;
+    constexpr uint32_t rt_base = Cfg::RT_BASE + PR * ((PA + 1) * 256);
+    const int slot_row = lane / CHUNKS, slot_chunk = lane % CHUNKS;
+    int src_chunk[NB_LOADS];
+#pragma unroll
+    for (int j = 0; j < NB_LOADS; j++) {
+        const int rho = (PR * NB_LOADS + j) * RPI + slot_row;
+        src_chunk[j] = slot_chunk ^ ((rho & 7) << 1);
+    }
+    const uint32_t lane16 = lane * 16, lane4 = lane * 4;
+    const uint32_t rt_lane_off = (uint32_t)((PR * NB_LOADS) * RPI + slot_row) * 4;
+
+    int is_tm = walk.tm0, is_tn = walk.tn0, is_step = 0;
+    uint32_t is_stage = 0;
+    uint32_t rt_read = 0;
+    int rt_tm = walk.tm0, rt_tn = walk.tn0, rt_step = 0, rt_left = Q - 1;
+    uint32_t rt_soff = (uint32_t)((rt_tm / tiles_per_vblock) * S) * 256u;
+    uint32_t a_soff = (uint32_t)((is_tm * WM) * S) * (uint32_t)APACK_BLOCK;    // wave-tile row 0 of the tile
+    uint32_t coloff[NB_LOADS];
+    auto set_coloff = [&]() {
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) {
+            const int col = is_tn * BN + src_chunk[j] * 8;
+            coloff[j] = (col < N && !SPATHA_KNOB(1)) ? (uint32_t)col * 2u : 0xF0000000u;
+        }
+    };
+    set_coloff();
+    auto rt_advance = [&]() {
+        if (rt_left > 0) {
+            --rt_left;
+            rt_soff += 256u;
+            if (++rt_step == S) {
+                rt_step = 0;
+                walk.next(rt_tm, rt_tn);
+                rt_soff = (uint32_t)((rt_tm / tiles_per_vblock) * S) * 256u;
+            }
+        }
+    };
+    auto issue_batch = [&](const uint32_t (&rows)[NB_LOADS]) {
+        const uint32_t stage = smem_base + is_stage;
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) {
+            const uint32_t voff = (rows[j] == 0xffffffffu) ? 0xF0000000u : rows[j] * row_bytes_b + coloff[j];
+            bdma_b128(voff, rsrc_b, 0, stage + (PR * NB_LOADS + j) * 1024);
+        }
+        // the A_INSTR operand / index blocks of the stage, NA_LOADS consecutive ones per producer:
+        // instruction a = wm*6 + k; k < 4: operand block k (1 KiB); k >= 4: index block k-4 (256 B)
+#pragma unroll
+        for (int k = 0; k < NA_LOADS; k++) {
+            constexpr int dummy = 0;
+            (void)dummy;
+            const int a = PR * NA_LOADS + k;
+            const int awm = a / 6, ak = a - awm * 6;
+            const uint32_t soff = a_soff + (uint32_t)(awm * S) * (uint32_t)APACK_BLOCK;
+            const uint32_t dst = stage + B_BYTES + awm * APACK_BLOCK;
+            if (ak < 4) bdma_b128(lane16, rsrc_a, soff + ak * 1024, dst + ak * 1024);
+            else bdma_b32(lane4, rsrc_a, soff + 4096 + (ak - 4) * 256, dst + 4096 + (ak - 4) * 256);
+        }
+        const uint32_t rt_write = (rt_read == 0) ? (uint32_t)PA * 256u : rt_read - 256u;
+        bdma_b32(lane4, rsrc_rt, rt_soff, smem_base + rt_base + rt_write);
+        rt_advance();
+        is_stage = (is_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : is_stage + STAGE_BYTES;
+        rt_read = (rt_read == (uint32_t)PA * 256u) ? 0u : rt_read + 256u;
+        a_soff += (uint32_t)APACK_BLOCK;
+        if (++is_step == S) {
+            is_step = 0;
+            walk.next(is_tm, is_tn);
+            a_soff = (uint32_t)((is_tm * WM) * S) * (uint32_t)APACK_BLOCK;
+            set_coloff();
+        }
+    };
+    // prologue: rows of the first PA stages through ordinary loads (nothing is in flight yet)
+    {
+        uint32_t rows0[PA][NB_LOADS];
+        int st_tm = walk.tm0, st_tn = walk.tn0, st_step = 0;
+#pragma unroll
+        for (int t = 0; t < PA; t++) {
+            const int64_t base = ((int64_t)(st_tm / tiles_per_vblock) * S + st_step) * 64;
+#pragma unroll
+            for (int j = 0; j < NB_LOADS; j++)
+                rows0[t][j] = (t < Q) ? p.rowtab[base + (PR * NB_LOADS + j) * RPI + slot_row] : 0xffffffffu;
+            if (++st_step == S) { st_step = 0; walk.next(st_tm, st_tn); }
+        }
+#pragma unroll
+        for (int t = 0; t < PA; t++) rt_advance();
+#pragma unroll
+        for (int t = 0; t < PA; t++)
+            if (t < Q) issue_batch(rows0[t]);
+    }
+    auto issue_from_ring = [&]() {
+        uint32_t rows[NB_LOADS];
+        const char* rr = smem + rt_base + rt_read + rt_lane_off;
+#pragma unroll
+        for (int j = 0; j < NB_LOADS; j++) rows[j] = *(const uint32_t*)(rr + j * (RPI * 4));
+        issue_batch(rows);
+    };
+    // steady state: PA-1 younger batches stay in flight behind the one being waited for
+    const int q_main = Q - PA > 0 ? Q - PA : 0;       // steps that still issue a batch
+    for (int q = 0; q < q_main; q++) {
+        wait_vmcnt<(PA - 1) * LOADS>();
+        __syncthreads();
+        if (!SPATHA_KNOB(8)) issue_from_ring();
+    }
+    // drain: nothing left to issue
+    for (int q = q_main; q < Q; q++) {
+        wait_stages<LOADS, PA - 1>(Q - 1 - q);
+        __syncthreads();
+    }
+}
+
+template <class Cfg, int WN, int OUT_LAYOUT>
+__device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int EPI_PITCH = Cfg::EPI_PITCH;
+    const int S = p.S, N = p.N;
+    const int wm = wave / WN, wn = wave - wm * WN;
+    float4_t acc[4][4];
+    const int li = lane & 15, kb = lane >> 4;
+    const int rrow = kb * 4 + (li >> 2);
+    const int sw = rrow & 7;
+    int tr_off[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int ch = (wn * 8 + nb * 2 + ((li & 3) >> 1)) ^ (sw << 1);
+        tr_off[nb] = rrow * ROW_BYTES + ch * 16 + (li & 1) * 8;
+    }
+    const int a_off = B_BYTES + wm * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + wm * APACK_BLOCK + 4096 + lane * 4;
+    const int j16 = lane & 15, ib = lane >> 4;
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    uint32_t c_stage = 0;
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            __syncthreads();
+            if (!SPATHA_KNOB(16)) mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {});
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+        }
+        const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+        if (p.fuse) fused_bias_act(acc, p.bias, (int64_t)cm0 + wm * 64 + ib * 16, p.act);
+        const uint16_t* bias = p.fuse ? nullptr : p.bias;
+        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+            store_block_transposed_slab<true>(acc, smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH), p.C, bias,
+                                              (int64_t)cm0 + wm * 64, cn0 + wn * 64, p.rows, N, lane, !SPATHA_KNOB(2));
+        } else if (!SPATHA_KNOB(4)) {
+            // 16-row slabs through a wave-private LDS buffer -> 128-byte row segments
+            char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int nb = 0; nb < 4; nb++)
+                        *(_Float16*)(stg + (r * 4 + ib) * EPI_PITCH + (nb * 16 + j16) * 2) = (_Float16)acc[mb][nb][r];
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int it = 0; it < 2; it++) {
+                    const int Lr = it * 8 + (lane >> 3), ch = lane & 7;
+                    const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
+                    const int col = cn0 + wn * 64 + ch * 8;
+                    u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
+                    if (col < N && !SPATHA_KNOB(2)) store_c16(p.C + ((int64_t)cm0 + wm * 64 + row) * N + col, v);
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+        walk.next(c_tm, c_tn);
+    }
+}
+
+template <class Cfg, int WN, int OUT_LAYOUT>
+__device__ __forceinline__ void ws_consumer_deferred(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int EPI_PITCH = Cfg::EPI_PITCH;
+    const int S = p.S, N = p.N;
+    const int wm = wave / WN, wn = wave - wm * WN;
+    float4_t acc[4][4];
+    uint32_t pend[4][4][2];         // previous tile: [mb][nb][r / 2] = fp16 pair (r even | r odd << 16)
+    const int li = lane & 15, kb = lane >> 4;
+    const int rrow = kb * 4 + (li >> 2);
+    const int sw = rrow & 7;
+    int tr_off[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int ch = (wn * 8 + nb * 2 + ((li & 3) >> 1)) ^ (sw << 1);
+        tr_off[nb] = rrow * ROW_BYTES + ch * 16 + (li & 1) * 8;
+    }
+    const int a_off = B_BYTES + wm * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + wm * APACK_BLOCK + 4096 + lane * 4;
+    const int j16 = lane & 15, ib = lane >> 4;
+    char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
+    const bool stores_on = !SPATHA_KNOB(2);
+
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    int pm0 = 0, pn0 = 0;           // origin of the tile held in pend
+    bool have_pend = false;
+    uint32_t c_stage = 0;
+    auto flush_part = [&](int part) {
+        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+            const int64_t row0 = (int64_t)pm0 + wm * 64 + ib * 16;
+            const int colb = pn0 + wn * 64 + j16;
+            if (part == 0) store_block_transposed<0>(pend, p.C, row0, colb, p.rows, N, stores_on);
+            else if (part == 1) store_block_transposed<1>(pend, p.C, row0, colb + 16, p.rows, N, stores_on);
+            else if (part == 2) store_block_transposed<2>(pend, p.C, row0, colb + 32, p.rows, N, stores_on);
+            else store_block_transposed<3>(pend, p.C, row0, colb + 48, p.rows, N, stores_on);
+        } else {
+            const int64_t rb = (int64_t)pm0 + wm * 64;
+            const int cb = pn0 + wn * 64;
+            if (part == 0) store_slab_row_major<0, EPI_PITCH>(pend, stg, p.C, rb, cb, N, lane, stores_on);
+            else if (part == 1) store_slab_row_major<1, EPI_PITCH>(pend, stg, p.C, rb, cb, N, lane, stores_on);
+            else if (part == 2) store_slab_row_major<2, EPI_PITCH>(pend, stg, p.C, rb, cb, N, lane, stores_on);
+            else store_slab_row_major<3, EPI_PITCH>(pend, stg, p.C, rb, cb, N, lane, stores_on);
+        }
+    };
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            __syncthreads();
+            if (!SPATHA_KNOB(16)) mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {});
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+            if (have_pend && c_step < 4 && !SPATHA_KNOB(4)) flush_part(c_step);
+        }
+        // a k-loop shorter than four steps leaves parts of the previous tile unwritten
+        if (have_pend && !SPATHA_KNOB(4))
+            for (int part = S; part < 4; part++) flush_part(part);
+        const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+        const bool with_bias = (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) && p.bias;
+        u32x4 bias_lo = {0, 0, 0, 0}, bias_hi = {0, 0, 0, 0};
+        if (with_bias) {
+            const int64_t row0 = (int64_t)cm0 + wm * 64 + ib * 16;
+            bias_lo = *(const u32x4*)(p.bias + row0);
+            bias_hi = *(const u32x4*)(p.bias + row0 + 8);
+        }
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++)
+#pragma unroll
+            for (int nb = 0; nb < 4; nb++)
+#pragma unroll
+                for (int rp = 0; rp < 2; rp++) {
+                    uint32_t w = pack_half2(acc[mb][nb][2 * rp], acc[mb][nb][2 * rp + 1]);
+                    if (with_bias) {
+                        const uint32_t bw = (mb < 2) ? bias_lo[mb * 2 + rp] : bias_hi[(mb - 2) * 2 + rp];
+                        const half2_t sum = __builtin_bit_cast(half2_t, w) + __builtin_bit_cast(half2_t, bw);
+                        w = __builtin_bit_cast(uint32_t, sum);
+                    }
+                    pend[mb][nb][rp] = w;
+                }
+        pm0 = cm0;
+        pn0 = cn0;
+        have_pend = true;
+        walk.next(c_tm, c_tn);
+    }
+    if (have_pend && !SPATHA_KNOB(4))
+        for (int part = 0; part < 4; part++) flush_part(part);
+}
+
+// ---- tall consumer: one wave owns a 128 x 64 tile (two stacked 64-row halves sharing the B
+// fragments): 32 matrix instructions per k-step for the same 16 transposing reads, so the
+// LDS and issue cost per matrix instruction drops by a third and one consumer per SIMD is enough.
+#define SPATHA_MMA8(NB, BF)                                                                                     \
+    _Pragma("unroll") for (int h_ = 0; h_ < 2; h_++) {                                                          \
+        acc[h_][0][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[h_][0], BF, acc[h_][0][NB], (int)ix[h_][0], 0, 0); \
+        acc[h_][1][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[h_][1], BF, acc[h_][1][NB], (int)ix[h_][0], 0, 1); \
+        acc[h_][2][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[h_][2], BF, acc[h_][2][NB], (int)ix[h_][1], 0, 0); \
+        acc[h_][3][NB] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[h_][3], BF, acc[h_][3][NB], (int)ix[h_][1], 0, 1); \
+    }
+
+template <int ROW_BYTES>
+__device__ __forceinline__ void mma_stage_tall(const char* st, int a_off, int i_off, const int (&tr_off)[4],
+                                               float4_t (&acc)[2][4][4]) {
+    half8_t a_cur[2][4];
+    uint32_t ix[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int mb = 0; mb < 4; mb++) a_cur[h][mb] = *(const half8_t*)(st + a_off + h * APACK_BLOCK + mb * 1024);
+        ix[h][0] = *(const uint32_t*)(st + i_off + h * APACK_BLOCK);
+        ix[h][1] = *(const uint32_t*)(st + i_off + h * APACK_BLOCK + 256);
+    }
+    half16_t bf0 = read_b_fragment<ROW_BYTES>(st, tr_off[0]);
+    half16_t bf1 = read_b_fragment<ROW_BYTES>(st, tr_off[1]);
+    __builtin_amdgcn_sched_barrier(0);
+    SPATHA_MMA8(0, bf0)
+    __builtin_amdgcn_sched_barrier(0);
+    bf0 = read_b_fragment<ROW_BYTES>(st, tr_off[2]);
+    __builtin_amdgcn_sched_barrier(0);
+    SPATHA_MMA8(1, bf1)
+    __builtin_amdgcn_sched_barrier(0);
+    bf1 = read_b_fragment<ROW_BYTES>(st, tr_off[3]);
+    __builtin_amdgcn_sched_barrier(0);
+    SPATHA_MMA8(2, bf0)
+    SPATHA_MMA8(3, bf1)
+}
+
+template <class Cfg, int WN, int OUT_LAYOUT>
+__device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
+    constexpr int EPI_PITCH = Cfg::EPI_PITCH;
+    static_assert(BM == 128, "two stacked 64-row halves");
+    const int S = p.S, N = p.N;
+    const int wn = wave;
+    float4_t acc[2][4][4];
+    const int li = lane & 15, kb = lane >> 4;
+    const int rrow = kb * 4 + (li >> 2);
+    const int sw = rrow & 7;
+    int tr_off[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int ch = (wn * 8 + nb * 2 + ((li & 3) >> 1)) ^ (sw << 1);
+        tr_off[nb] = rrow * ROW_BYTES + ch * 16 + (li & 1) * 8;
+    }
+    const int a_off = B_BYTES + lane * 16;
+    const int i_off = B_BYTES + 4096 + lane * 4;
+    const int j16 = lane & 15, ib = lane >> 4;
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    uint32_t c_stage = 0;
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int a = 0; a < 4; a++)
+#pragma unroll
+                for (int b = 0; b < 4; b++) acc[h][a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            __syncthreads();
+            if (!SPATHA_KNOB(16)) mma_stage_tall<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc);
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+        }
+        const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            if (p.fuse) fused_bias_act(acc[h], p.bias, (int64_t)cm0 + h * 64 + ib * 16, p.act);
+            if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+                if (!SPATHA_KNOB(4))
+                    store_block_transposed_slab<true>(acc[h], smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH), p.C, p.fuse ? nullptr : p.bias,
+                                                (int64_t)cm0 + h * 64, cn0 + wn * 64, p.rows, N, lane, !SPATHA_KNOB(2));
+            } else if (!SPATHA_KNOB(4)) {
+                char* stg = smem + Cfg::EPI_BASE + wave * (16 * EPI_PITCH);
+#pragma unroll
+                for (int mb = 0; mb < 4; mb++) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+#pragma unroll
+                        for (int nb = 0; nb < 4; nb++)
+                            *(_Float16*)(stg + (r * 4 + ib) * EPI_PITCH + (nb * 16 + j16) * 2) = (_Float16)acc[h][mb][nb][r];
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int it = 0; it < 2; it++) {
+                        const int Lr = it * 8 + (lane >> 3), ch = lane & 7;
+                        const int row = 16 * (Lr & 3) + 4 * mb + (Lr >> 2);
+                        const int col = cn0 + wn * 64 + ch * 8;
+                        u32x4 v = *(const u32x4*)(stg + Lr * EPI_PITCH + ch * 16);
+                        if (col < N && !SPATHA_KNOB(2)) store_c16(p.C + ((int64_t)cm0 + h * 64 + row) * N + col, v);
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+        }
+        walk.next(c_tm, c_tn);
+    }
+}
+
+// Tile 128 x (64 * WN): WN tall consumers + NP producers.
+template <int WN, int NS, int NP, int OUT_LAYOUT>
+__global__ __launch_bounds__((WN + NP) * 64) void spmm_wst_kernel(SpmmParams p) {
+    using Cfg = WsCfg<2, WN, NS, NP>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TileWalk walk;
+    walk.init(p.tiles_m, p.tiles_n);
+    if (walk.my_tiles == 0) return;
+    if (SPATHA_SKEW_ON(p)) {
+        const int units = ((blockIdx.x >> 3) & 7) * p.skew;
+        for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);
+    }
+    if (wave < WN) {
+        ws_consumer_tall<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
+    } else {
+        const int pr = wave - WN;
+        if (pr == 0) ws_producer<Cfg, NP, 0>(p, walk, smem, smem_base, lane);
+        else if (pr == 1) ws_producer<Cfg, NP, 1>(p, walk, smem, smem_base, lane);
+        else if (NP > 2 && pr == 2) ws_producer<Cfg, NP, (NP > 2 ? 2 : 0)>(p, walk, smem, smem_base, lane);
+        else if (NP > 2) ws_producer<Cfg, NP, (NP > 2 ? 3 : 0)>(p, walk, smem, smem_base, lane);
+    }
+}
+
+template <int WN, int NS, int NP, int OUT_LAYOUT>
+static hipError_t launch_wst(const SpmmParams& p, hipStream_t stream) {
+    using Cfg = WsCfg<2, WN, NS, NP>;
+    constexpr int lds = Cfg::LDS_BYTES;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static int cus = 0;
+    auto kern = spmm_wst_kernel<WN, NS, NP, OUT_LAYOUT>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        int dev = 0;
+        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int per_cu = (160 * 1024) / lds;
+    const int tiles = p.tiles_m * p.tiles_n;
+    int grid = ((cus * per_cu) / 8) * 8;
+    const int need = ((tiles + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    if (grid < 8) grid = 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3((WN + NP) * 64), lds, stream, p);
+    return hipGetLastError();
+}
+
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false>
+__global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams p) {
+    using Cfg = WsCfg<WM, WN, NS, NP>;
+    static_assert(NP == 2 || NP == 4, "producer count");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TileWalk walk;
+    walk.init(p.tiles_m, p.tiles_n);
+    if (walk.my_tiles == 0) return;
+    // Workgroups of one XCD start up to 7 * skew apart, so that tiles do not all finish (and
+    // hit HBM with their stores) at the same moment on every CU.
+    if (SPATHA_SKEW_ON(p)) {
+        const int units = ((blockIdx.x >> 3) & 7) * p.skew;
+        for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);      // 16 * 64 clocks
+    }
+    if (wave < Cfg::NC) {
+        if (DEFER) ws_consumer_deferred<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
+        else ws_consumer<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
+    } else {
+        // the producer index is a template argument: which DMA instructions a producer issues
+        // is then fixed at compile time (no branches in its loop)
+        const int pr = wave - Cfg::NC;
+        if (pr == 0) ws_producer<Cfg, NP, 0>(p, walk, smem, smem_base, lane);
+        else if (pr == 1) ws_producer<Cfg, NP, 1>(p, walk, smem, smem_base, lane);
+        else if (NP > 2 && pr == 2) ws_producer<Cfg, NP, (NP > 2 ? 2 : 0)>(p, walk, smem, smem_base, lane);
+        else if (NP > 2) ws_producer<Cfg, NP, (NP > 2 ? 3 : 0)>(p, walk, smem, smem_base, lane);
+    }
+}
+
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false>
+static hipError_t launch_ws(const SpmmParams& p, hipStream_t stream) {
+    using Cfg = WsCfg<WM, WN, NS, NP>;
+    constexpr int lds = Cfg::LDS_BYTES;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    static int cus = 0;
+    auto kern = spmm_ws_kernel<WM, WN, NS, NP, OUT_LAYOUT, DEFER>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        int dev = 0;
+        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int per_cu = (160 * 1024) / lds;
+    const int tiles = p.tiles_m * p.tiles_n;
+    int grid = cus * per_cu;
+    grid = (grid / 8) * 8;
+    const int need = ((tiles + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    if (grid < 8) grid = 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::THREADS), lds, stream, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_warpspec(int variant, int out_layout, const SpmmParams& p, hipStream_t stream) {
+    const bool t = out_layout == SPATHA_OUT_TRANSPOSED;
+    switch (variant) {
+        case SPMM_VARIANT_W128x128_S3:
+            return t ? launch_ws<2, 2, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_ws<2, 2, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
+        case SPMM_VARIANT_W128x256_S3:
+            return t ? launch_ws<2, 4, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_ws<2, 4, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
+        case SPMM_VARIANT_W64x256_S3:
+            return t ? launch_ws<1, 4, 3, 2, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_ws<1, 4, 3, 2, SPATHA_OUT_ROW_MAJOR>(p, stream);
+        case SPMM_VARIANT_D64x256_S3:
+            return t ? launch_ws<1, 4, 3, 2, SPATHA_OUT_TRANSPOSED, true>(p, stream)
+                     : launch_ws<1, 4, 3, 2, SPATHA_OUT_ROW_MAJOR, true>(p, stream);
+        case SPMM_VARIANT_T128x256_S3:
+            return t ? launch_wst<4, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_wst<4, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace spatha
+

@@ -474,7 +474,7 @@ constexpr int TR8_SLAB_BYTES = 64 * TR8_PITCH;     // per wave, 8 slab rows at a
 // BIAS_VIA_SLAB (needs ROWS8 and 128 spare bytes behind the slab): the block's 64 bias values are fetched once, ahead of
 // the first store, and the phases read them from LDS; a bias load inside a phase would make that phase wait on the
 // vector-memory counter, i.e. for every store issued so far.
-template <bool ROWS8, bool BIAS_VIA_SLAB = false>
+template <bool ROWS8, bool BIAS_VIA_SLAB = false, bool WRITE_THROUGH = true>
 __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4][4], char* stg, uint16_t* C, int64_t row0,
                                                          int col0, int N, int lane, bool stores_on,
                                                          const uint16_t* bias = nullptr) {
@@ -527,7 +527,7 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
         short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff));
         short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, stg + roff + 4 * PITCH));
         __builtin_amdgcn_wave_barrier();
-        if (ph > 0 && live) store_c16<true>(C + (row0 + held_row) * N + out_col, held);
+        if (ph > 0 && live) store_c16<WRITE_THROUGH>(C + (row0 + held_row) * N + out_col, held);
         held.x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
         held.y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
         held.z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
@@ -535,7 +535,7 @@ __device__ __forceinline__ void store_block_row_major_tr(const float4_t (&acc)[4
         const int q = 8 * sidx + q_lo;
         held_row = 16 * (q >> 2) + 4 * mb + (q & 3);
     }
-    if (live) store_c16<true>(C + (row0 + held_row) * N + out_col, held);
+    if (live) store_c16<WRITE_THROUGH>(C + (row0 + held_row) * N + out_col, held);
     __builtin_amdgcn_wave_barrier();
 }
 
@@ -675,6 +675,18 @@ struct DuCfg {
     static constexpr int NB = M_ / 2;              // DMA instructions per wave and stage (4 rows x 256 B each)
     static constexpr int ROW_BYTES = BN * 2;
     static constexpr int STAGE_BYTES = 16 * M * ROW_BYTES;
+    static constexpr int SLAB_BYTES = TT_SLAB_BYTES;
+    static_assert(SLAB_BYTES >= TR8_SLAB_BYTES + 128, "slab");
+    static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES + 8 * SLAB_BYTES;
+    static constexpr int THREADS = 512;
+};
+
+// The unified kernel in two phase groups (spmm_pingpong.hip): m <= 8, three 32 KB stages.
+struct UpCfg {
+    static constexpr int BM = 512, BN = 128, M = 8, NS = 3;
+    static constexpr int NB = 4;                   // DMA instructions per wave and stage (4 rows x 256 B each)
+    static constexpr int STAGE_BYTES = 16 * M * BN * 2;
     static constexpr int SLAB_BYTES = TT_SLAB_BYTES;
     static_assert(SLAB_BYTES >= TR8_SLAB_BYTES + 128, "slab");
     static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;

@@ -45,8 +45,8 @@ const VariantInfo kVariants[] = {
      launch_gathered},
     {SPMM_VARIANT_DSH256x128_S3_C8, "smfmac16x16x64_halftile_densestage_tile256x128_3stage_8consumers", 256, 128,
      DsCfg<8, 3, 4, 8>::LDS_BYTES, 0, launch_densestage},
-    {SPMM_VARIANT_DU512x128_S4, "smfmac16x16x64_unified_densestage_aregs_tile512x128_4stage", 512, 128, DuCfg<8>::LDS_BYTES, 0,
-     launch_unified},
+    {SPMM_VARIANT_UP512x128_S3, "smfmac16x16x64_unified_pingpong_densestage_aregs_tile512x128_3stage", 512, 128, UpCfg::LDS_BYTES, 0,
+     launch_pingpong},
     {SPMM_VARIANT_DU512x128_M16, "smfmac16x16x64_unified_densestage_aregs_tile512x128_m16_2stage", 512, 128, DuCfg<16>::LDS_BYTES, 0,
      launch_unified},
 };

@@ -53,8 +53,8 @@ enum {
     SPMM_VARIANT_H64x128_S2 = 16,
     SPMM_VARIANT_DSH256x128_S3_C8 = 17, // m <= 8: dense-staged B, two gather-table entries per consumer wave
     // unified waves, A operands in registers, only B staged (rows % 512 == 0)
-    SPMM_VARIANT_DU512x128_S4 = 18,     // m <= 8
-    SPMM_VARIANT_DU512x128_M16 = 19,    // 8 < m <= 16: 64 KB stages, two of them
+    SPMM_VARIANT_UP512x128_S3 = 18,     // m <= 8: the eight waves in two phase groups (burst of loads / matrix phase)
+    SPMM_VARIANT_DU512x128_M16 = 19,    // 8 < m <= 16: one phase group, 64 KB stages, two of them
     SPMM_VARIANT_COUNT = 20
 };
 
@@ -66,12 +66,13 @@ int spmm_variant_lds(int variant, int S);
 hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 
 // one launch switch per kernel family (spmm_gathered.hip, spmm_warpspec.hip, spmm_densestage.hip, spmm_unified.hip,
-// spmm_skinny.hip); hipErrorInvalidValue for an id of another family
+// spmm_skinny.hip, spmm_pingpong.hip); hipErrorInvalidValue for an id of another family
 hipError_t launch_gathered(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 hipError_t launch_warpspec(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 hipError_t launch_densestage(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 hipError_t launch_unified(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 hipError_t launch_skinny_family(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
+hipError_t launch_pingpong(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
                        int m, int v, int ksp, int S, int half_tiles, uint16_t* apack, uint32_t* rowtab, hipStream_t stream);

@@ -309,8 +309,6 @@ hipError_t launch_unified(int variant, int out_layout, const SpmmParams& p, hipS
     const bool t = out_layout == SPATHA_OUT_TRANSPOSED;
     if (p.fuse) return hipErrorNotSupported;
     switch (variant) {
-        case SPMM_VARIANT_DU512x128_S4:
-            return t ? launch_du<SPATHA_OUT_TRANSPOSED, false>(p, stream) : launch_du<SPATHA_OUT_ROW_MAJOR, false>(p, stream);
         case SPMM_VARIANT_DU512x128_M16:
             return t ? launch_du<SPATHA_OUT_TRANSPOSED, false, 16>(p, stream) : launch_du<SPATHA_OUT_ROW_MAJOR, false, 16>(p, stream);
         default: return hipErrorInvalidValue;

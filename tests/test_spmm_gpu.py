@@ -156,8 +156,10 @@ FUSED_CASES = [
     # rows, cols, N, m, v
     (256, 512, 264, 8, 64),       # dense-staged kernels + gathered 64-row tiles, ragged N
     (256, 1024, 200, 8, 128),     # 128-row tiles: wave-specialised and tall consumers
-    (512, 325, 136, 5, 128),
+    (512, 325, 136, 5, 128),      # ... and the unified kernel in two phase groups (rows % 512 == 0, m <= 8)
     (256, 512, 136, 16, 64),
+    (512, 512, 264, 8, 64),
+    (512, 512, 136, 16, 64),      # unified kernel for 8 < m <= 16
 ]
 
 
@@ -184,6 +186,7 @@ def test_fused_bias_and_activation(gpu, rows, cols, N, m, v, transposed, activat
         want = fn(pre.astype(np.float64)).astype(np.float16)
     plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
     ran = 0
+    unified = 18 if m <= 8 else 19 if m <= 16 else None        # the unified kernels apply bias / activation themselves
     for variant in range(spatha.num_variants()):
         if plan.kernel_name(N, 1 if transposed else 0, variant) is None:
             continue
@@ -191,6 +194,7 @@ def test_fused_bias_and_activation(gpu, rows, cols, N, m, v, transposed, activat
             got = plan.run(_dev(B, gpu), bias=_dev(bias, gpu), transposed_out=transposed, variant=variant, activation=activation)
         except RuntimeError as e:
             assert "no kernel" in str(e)            # this kernel has no fused write-out: refused, not ignored
+            assert not (rows % 512 == 0 and v % 64 == 0 and variant == unified), variant
             continue
         torch.cuda.synchronize()
         ran += 1

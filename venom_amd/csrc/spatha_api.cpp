@@ -31,6 +31,7 @@ bool variant_has_fused_writeout(int variant) {
         case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_R64x256_S3:
         case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x256_S3: case SPMM_VARIANT_W64x256_S3:
         case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DSH256x128_S3_C8:
+        case SPMM_VARIANT_UP512x128_S3: case SPMM_VARIANT_DU512x128_M16:
             return true;
         default:
             return false;
@@ -68,8 +69,7 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = f
         // four 64-row blocks per tile; all 16*m dense rows of a k-step must fit one stage
         if (plan->geo.v % 64 != 0 || plan->geo.m > 8 || plan->geo.rows % 256 != 0 || !plan->gtab) return false;
     } else if (unified) {
-        // no fused write-out (that instantiation would need scratch memory)
-        if (plan->geo.v % 64 != 0 || plan->geo.rows % 512 != 0 || !plan->gtab || plan->half_tiles || fused) return false;
+        if (plan->geo.v % 64 != 0 || plan->geo.rows % 512 != 0 || !plan->gtab || plan->half_tiles) return false;
         if (variant == SPMM_VARIANT_DU512x128_M16 ? (plan->geo.m <= 8 || plan->geo.m > 16) : plan->geo.m > 8) return false;
         if (plan->gtab_bytes >= 0xE0000000ull) return false;
     } else if (plan->geo.v % bm != 0) {
@@ -188,7 +188,7 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
     // of the dense-staged kernel when its tiles fill whole rounds of the CUs (BERT-large layer shapes at N = 16384,
     // V = 64 and 128, m = 8 and 4: 256, 768, 1024 tiles), 10-20 % behind at 320 or 384 tiles (1.25 / 1.5 rounds) and up to
     // 2x behind with fewer tiles than CUs; transposed output with 256 tiles of 8 k-steps measures 2-3 % behind.
-    if (!fused && plan->geo.m <= 8 && variant_ok(plan, N, SPMM_VARIANT_UP512x128_S3, fused)) {
+    if (plan->geo.m <= 8 && variant_ok(plan, N, SPMM_VARIANT_UP512x128_S3, fused)) {
         const int64_t du_tiles = (int64_t)(plan->geo.rows / 512) * ((N + 127) / 128);
         const int64_t cus = plan->cus > 0 ? plan->cus : 256;
         const int64_t rounds = (du_tiles + cus - 1) / cus;
@@ -200,7 +200,7 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
     // Its form for 8 < m <= 16 (64 KB stages, two of them): V a multiple of 64 only - 7-26 % ahead of the gathered
     // 64 x 256 tiles on the BERT-large layer shapes at N = 16384 (64:2:16 and 64:2:10, both layouts); with V % 128 == 0
     // the gathered 128 x 256 tiles share their B rows over 128 rows and are equal or up to 15 % ahead.
-    if (!fused && plan->geo.m > 8 && plan->geo.v % 128 != 0 && variant_ok(plan, N, SPMM_VARIANT_DU512x128_M16, fused)) {
+    if (plan->geo.m > 8 && plan->geo.v % 128 != 0 && variant_ok(plan, N, SPMM_VARIANT_DU512x128_M16, fused)) {
         const int64_t du_tiles = (int64_t)(plan->geo.rows / 512) * ((N + 127) / 128);
         const int64_t cus = plan->cus > 0 ? plan->cus : 256;
         const int64_t rounds = (du_tiles + cus - 1) / cus;

@@ -161,6 +161,31 @@ __device__ __forceinline__ void fused_bias_act_impl(float4_t (&acc)[4][4], const
         }
     }
 }
+// The same with the choice of the activation inside the loop (one uniform branch per group of four values): the two
+// paths then join on four registers, not on the 64 of the whole block - for kernels that have no registers to spare
+// for the copies such a join can cost.
+__device__ __forceinline__ void fused_bias_act_narrow(float4_t (&acc)[4][4], const uint16_t* bias, int64_t row16, int act) {
+#pragma unroll
+    for (int mb = 0; mb < 4; mb++) {
+        half4_t bv = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+        if (bias) bv = *(const half4_t*)(bias + row16 + 4 * mb);
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+            float4_t v = acc[mb][nb];
+#pragma unroll
+            for (int r = 0; r < 4; r++) v[r] = (float)((_Float16)v[r] + bv[r]);
+            if (act == SPATHA_ACT_GELU) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) v[r] = act_gelu_erf(v[r]);
+            } else if (act == SPATHA_ACT_GELU_TANH) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) v[r] = act_gelu_tanh(v[r]);
+            }
+            acc[mb][nb] = v;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
 __device__ __forceinline__ void fused_bias_act(float4_t (&acc)[4][4], const uint16_t* bias, int64_t row16, int act) {
     if (act == SPATHA_ACT_GELU) fused_bias_act_impl<SPATHA_ACT_GELU>(acc, bias, row16);
     else if (act == SPATHA_ACT_GELU_TANH) fused_bias_act_impl<SPATHA_ACT_GELU_TANH>(acc, bias, row16);
@@ -687,10 +712,9 @@ struct UpCfg {
     static constexpr int BM = 512, BN = 128, M = 8, NS = 3;
     static constexpr int NB = 4;                   // DMA instructions per wave and stage (4 rows x 256 B each)
     static constexpr int STAGE_BYTES = 16 * M * BN * 2;
-    static constexpr int SLAB_BYTES = TT_SLAB_BYTES;
-    static_assert(SLAB_BYTES >= TR8_SLAB_BYTES + 128, "slab");
+    static constexpr int WAVE_EPI = WAVE_EPI_BYTES;            // four write-out slabs per wave
     static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
-    static constexpr int LDS_BYTES = NS * STAGE_BYTES + 8 * SLAB_BYTES;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES + 8 * WAVE_EPI;
     static constexpr int THREADS = 512;
 };
 

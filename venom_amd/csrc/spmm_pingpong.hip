@@ -19,27 +19,38 @@
 //   Y, step q: burst = operands of step q + 2 (into the set step q just used)  + this wave's share of stage q + 2
 // Stage q + 2 goes into the slot stage q - 1 occupied, which every wave has left when it passed barrier q: three stages.
 // The wait sits ahead of a tile's stores: a wait behind them would wait for the stores too (same counter).
+// A finished tile leaves through four LDS slabs per wave (a 64 x 64 block in two LDS round trips); LDS: 3 x 32 KB of
+// stages + 8 x 4.6 KB of slabs.
 
 #include "spmm_device.h"
+
+// Development switches, compiled in with -DSPATHA_UP_KNOBS=<bits> for timing experiments only (0 in the library; the
+// results are then wrong on purpose):  1 no B stages (matrix phases on whatever the LDS holds)   2 no write-out
+//   4 the late group skips its matrix phases   8 a second barrier in the middle of a step   16 no A operands (only
+//   the gather table is loaded)   32 write-out without its global stores
+#ifndef SPATHA_UP_KNOBS
+#define SPATHA_UP_KNOBS 0
+#endif
 
 namespace spatha {
 
 namespace {
+constexpr int UP_KNOBS = SPATHA_UP_KNOBS;
 __device__ __forceinline__ void pload_b128(u32x4& r, uint32_t voff, i32x4 rsrc, uint32_t soff) {
-    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "+v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 __device__ __forceinline__ void pload_b32(uint32_t& r, uint32_t voff, i32x4 rsrc, uint32_t soff) {
-    asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "+v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    asm volatile("buffer_load_dword %0, %1, %2, %3 offen" : "=&v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 __device__ __forceinline__ void pload_b64(u32x2& r, uint32_t voff, i32x4 rsrc, uint32_t soff) {
-    asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "+v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+    asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "=&v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 }  // namespace
 
 // The whole life of one wave.  LATE is the wave's phase group (false: X, true: Y), a template argument so that each group
 // runs straight-line code of its own: an operand set that is in flight must never meet, at a join of two paths, a
 // version of itself that is not (the register copy the compiler may place there would copy a value that has not arrived).
-template <int OUT_LAYOUT, bool LATE>
+template <int OUT_LAYOUT, bool FUSE, bool LATE>
 __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& walk, char* smem, uint32_t smem_base, int wave,
                                         int lane) {
     using Cfg = UpCfg;
@@ -69,6 +80,7 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
     set_voff();
     int issued = 0;
     auto issue_stage = [&]() {
+        if (UP_KNOBS & 1) return;
         if (issued >= Q) return;
         ++issued;
         const uint32_t dst = smem_base + is_stage + wave * (NB * 1024);
@@ -111,6 +123,7 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
             }
         }
         pload_b64(y.g, gvoff, rsrc_g, goff);
+        if (UP_KNOBS & 16) return;
 #pragma unroll
         for (int k = 0; k < 4; k++) pload_b128(y.a[k], lane16, rsrc_a, soff + k * 1024);
         pload_b32(y.i0, lane4, rsrc_a, soff + 4096);
@@ -195,27 +208,44 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
         if constexpr (!LATE) {
             load_set(other);    // operands of step q + 1
             issue_stage();      // share of stage q + 2
+            if (UP_KNOBS & 8) __syncthreads();
         }
-        matrix_phase(cur);
+        if (!(LATE && (UP_KNOBS & 4))) matrix_phase(cur);
         c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
         // Everything this wave has in flight, issued one matrix phase ago: X, its burst of this step (operands of step
         // q + 1, share of stage q + 2); Y, its burst of the step before (operands of step q + 1, share of stage q + 1).
         // Always here, never under a condition, and ahead of the tile's stores, which a later wait would sit out too.
         SPATHA_UP_WAIT_ALL();
         if constexpr (LATE) {
+            if (UP_KNOBS & 8) __syncthreads();
             load_set(cur);      // operands of step q + 2
             issue_stage();      // share of stage q + 2
         }
         if (++c_step == S) {
             c_step = 0;
             const int cm0 = c_tm * BM + wave * 64, cn0 = c_tn * BN;
-            char* stg = smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES;
+            char* stg = smem + Cfg::EPI_BASE + wave * Cfg::WAVE_EPI;
+            if (UP_KNOBS & 2) {     // keep the accumulators alive without storing them
+                float t = 0.f;
 #pragma unroll
-            for (int wn = 0; wn < 2; wn++) {
-                if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
-                    store_block_transposed_slab<true>(acc[wn], stg, p.C, p.bias, (int64_t)cm0, cn0 + wn * 64, p.rows, N, lane, true);
-                else
-                    store_block_row_major_tr<true>(acc[wn], stg, p.C, (int64_t)cm0, cn0 + wn * 64, N, lane, true);
+                for (int h = 0; h < 2; h++)
+#pragma unroll
+                    for (int a = 0; a < 4; a++)
+#pragma unroll
+                        for (int b = 0; b < 4; b++) t += acc[h][a][b][0] + acc[h][a][b][1] + acc[h][a][b][2] + acc[h][a][b][3];
+                if (t == 12345.678f) p.C[lane] = 1;
+            } else {
+#pragma unroll
+                for (int wn = 0; wn < 2; wn++) {
+                    // fused: bias and activation first, always and on one path (a path that skipped them would join this
+                    // one on all 64 accumulator registers of the block); the write-out itself is then the plain one
+                    if constexpr (FUSE) fused_bias_act_narrow(acc[wn], p.bias, (int64_t)cm0 + (lane >> 4) * 16, p.act);
+                    if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
+                        store_block_transposed_slab4(acc[wn], stg, p.C, FUSE ? nullptr : p.bias, (int64_t)cm0, cn0 + wn * 64, p.rows, N,
+                                                     lane, !(UP_KNOBS & 32));
+                    else
+                        store_block_row_major_tr4<false>(acc[wn], stg, p.C, (int64_t)cm0, cn0 + wn * 64, N, lane, !(UP_KNOBS & 32), nullptr);
+                }
             }
             zero_acc();
             walk.next(c_tm, c_tn);
@@ -228,7 +258,7 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
 #undef SPATHA_UP_WAIT_ALL
 }
 
-template <int OUT_LAYOUT>
+template <int OUT_LAYOUT, bool FUSE>
 __global__ __launch_bounds__(512) void spmm_up_kernel(SpmmParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
@@ -237,16 +267,16 @@ __global__ __launch_bounds__(512) void spmm_up_kernel(SpmmParams p) {
     TileWalk walk;
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
-    if (wave >= 4) up_wave<OUT_LAYOUT, true>(p, walk, smem, smem_base, wave, lane);
-    else up_wave<OUT_LAYOUT, false>(p, walk, smem, smem_base, wave, lane);
+    if (wave >= 4) up_wave<OUT_LAYOUT, FUSE, true>(p, walk, smem, smem_base, wave, lane);
+    else up_wave<OUT_LAYOUT, FUSE, false>(p, walk, smem, smem_base, wave, lane);
 }
 
-template <int OUT_LAYOUT>
+template <int OUT_LAYOUT, bool FUSE>
 static hipError_t launch_up(const SpmmParams& p, hipStream_t stream) {
     constexpr int lds = UpCfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static int cus = 0;
-    void (*kern)(SpmmParams) = spmm_up_kernel<OUT_LAYOUT>;
+    void (*kern)(SpmmParams) = spmm_up_kernel<OUT_LAYOUT, FUSE>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         // the kernel's register loads complete asynchronously into named variables: an instantiation that keeps
@@ -273,9 +303,12 @@ static hipError_t launch_up(const SpmmParams& p, hipStream_t stream) {
 
 hipError_t launch_pingpong(int variant, int out_layout, const SpmmParams& p, hipStream_t stream) {
     if (variant != SPMM_VARIANT_UP512x128_S3) return hipErrorInvalidValue;
-    if (p.fuse) return hipErrorNotSupported;
-    return out_layout == SPATHA_OUT_TRANSPOSED ? launch_up<SPATHA_OUT_TRANSPOSED>(p, stream)
-                                               : launch_up<SPATHA_OUT_ROW_MAJOR>(p, stream);
+    // (the plain instantiations carry nothing of the fused write-out)
+    if (p.fuse)
+        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_up<SPATHA_OUT_TRANSPOSED, true>(p, stream)
+                                                   : launch_up<SPATHA_OUT_ROW_MAJOR, true>(p, stream);
+    return out_layout == SPATHA_OUT_TRANSPOSED ? launch_up<SPATHA_OUT_TRANSPOSED, false>(p, stream)
+                                               : launch_up<SPATHA_OUT_ROW_MAJOR, false>(p, stream);
 }
 
 }  // namespace spatha

@@ -249,16 +249,14 @@ __global__ __launch_bounds__(512) void spmm_du_kernel(SpmmParams p) {
             const int cm0 = c_tm * BM + wave * 64, cn0 = c_tn * BN;
             char* stg = smem + Cfg::EPI_BASE + wave * Cfg::SLAB_BYTES;
             const int ib = lane >> 4;
-            // a bias alone rides in the row-major write-out itself (packed fp16 additions); anything else goes first
-            const bool pre = FUSE && (p.act != SPATHA_ACT_NONE || OUT_LAYOUT == SPATHA_OUT_TRANSPOSED);
 #pragma unroll
             for (int wn = 0; wn < 2; wn++) {
-                if (FUSE && pre) fused_bias_act(acc[wn], p.bias, (int64_t)cm0 + ib * 16, p.act);
+                // fused: bias and activation first, always and on one path (a path that skipped them would join this one
+                // on all 64 accumulator registers of the block); the write-out itself is then the plain one
+                if constexpr (FUSE) fused_bias_act_narrow(acc[wn], p.bias, (int64_t)cm0 + ib * 16, p.act);
                 if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED)
                     store_block_transposed_slab<true>(acc[wn], stg, p.C, FUSE ? nullptr : p.bias, (int64_t)cm0, cn0 + wn * 64, p.rows,
                                                       N, lane, true);
-                else if (FUSE && !pre && p.bias)
-                    store_block_row_major_tr<true, true>(acc[wn], stg, p.C, (int64_t)cm0, cn0 + wn * 64, N, lane, true, p.bias);
                 else
                     store_block_row_major_tr<true>(acc[wn], stg, p.C, (int64_t)cm0, cn0 + wn * 64, N, lane, true);
             }
@@ -304,12 +302,12 @@ static hipError_t launch_du(const SpmmParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
-// (no fused write-out: that instantiation needs scratch memory, which the kernel's asynchronous register loads rule out)
 hipError_t launch_unified(int variant, int out_layout, const SpmmParams& p, hipStream_t stream) {
     const bool t = out_layout == SPATHA_OUT_TRANSPOSED;
-    if (p.fuse) return hipErrorNotSupported;
     switch (variant) {
         case SPMM_VARIANT_DU512x128_M16:
+            if (p.fuse)
+                return t ? launch_du<SPATHA_OUT_TRANSPOSED, true, 16>(p, stream) : launch_du<SPATHA_OUT_ROW_MAJOR, true, 16>(p, stream);
             return t ? launch_du<SPATHA_OUT_TRANSPOSED, false, 16>(p, stream) : launch_du<SPATHA_OUT_ROW_MAJOR, false, 16>(p, stream);
         default: return hipErrorInvalidValue;
     }

@@ -30,8 +30,12 @@ SMFMAC_PEAK_TFLOPS = 5033.0    # fp16 MFMA with 2:4 structured sparsity (dense f
 MEASURED_TRAFFIC = {
     ("smfmac16x16x64_warpspec_densestage_tile256x128_3stage_8consumers", 4096, 1024, 16384, 8, 64):
         (194_615_000, "profiles/spmm_ds_kernel_tile256x128_ffn_up_64-2-8.md"),
-    ("smfmac16x16x64_unified_densestage_aregs_tile512x128_4stage", 4096, 1024, 16384, 8, 64):
-        (199_275_000, "profiles/spmm_du_kernel_tile512x128_ffn_up_64-2-8.md"),
+    ("smfmac16x16x64_unified_pingpong_densestage_aregs_tile512x128_3stage", 4096, 1024, 16384, 8, 64):
+        (199_214_000, "profiles/spmm_up_kernel_tile512x128_ffn_up_64-2-8.md"),
+    ("smfmac16x16x64_unified_pingpong_densestage_aregs_tile512x128_3stage", 4096, 1024, 16384, 4, 128):
+        (323_090_000, "profiles/spmm_up_kernel_tile512x128_ffn_up_2-4.md"),
+    ("smfmac16x16x64_warpspec_tall_tile128x256_3stage", 49152, 12288, 2048, 16, 128):
+        (2_202_100_000, "profiles/spmm_wst_kernel_tile128x256_gpt3_ffn_n2048.md"),
 }
 
 
@@ -183,7 +187,9 @@ def main():
         by = algorithmic_bytes(r2, c2, n2, m2, v2, w2["geo"].ksp)
         fl = 2.0 * r2 * n2 * 2 * w2["geo"].ksp
         t_hbm, t_mma = by / (HBM_PEAK_GBS * 1e9), fl / (SMFMAC_PEAK_TFLOPS * 1e12)
+        tr, src = MEASURED_TRAFFIC.get((w2["plan"].kernel_name(n2, 0, 0), r2, c2, n2, m2, v2), (None, None))
         return {"shape": "%dx%dx%d %d:2:%d" % (r2, c2, n2, v2, m2), "kernel": w2["plan"].kernel_name(n2, 0, 0),
+                "algorithmic_bytes": by, "traffic": tr, "traffic_source": src,
                 "us": round(k2 * 1e3, 2), "dense_equiv_tflops": round(2.0 * r2 * c2 * n2 / (k2 * 1e-3) / 1e12, 1),
                 "hbm_gbs": round(by / (k2 * 1e-3) / 1e9, 1), "hbm_frac": round(by / (k2 * 1e-3) / 1e9 / HBM_PEAK_GBS, 3),
                 "pct_smfmac_peak": round(100 * fl / (k2 * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2),

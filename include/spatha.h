@@ -27,7 +27,7 @@ typedef enum spatha_status {
     SPATHA_OK = 0,
     SPATHA_ERR_BAD_ARGUMENT = 1,   /* null pointer, negative size, n != 2, ...              */
     SPATHA_ERR_BAD_SHAPE = 2,      /* rows % V, V % 32, m < 4, N alignment, ...             */
-    SPATHA_ERR_UNSUPPORTED = 3,    /* valid format, but no kernel for it (rows % 64 != 0)   */
+    SPATHA_ERR_UNSUPPORTED = 3,    /* valid format, but no kernel for the request          */
     SPATHA_ERR_HIP = 4,            /* a HIP runtime call failed; see spatha_last_hip_error  */
     SPATHA_ERR_NO_DEVICE = 5,      /* no HIP device visible                                 */
     SPATHA_ERR_TOO_LARGE = 6,      /* beyond a fixed capacity of the entry point            */

@@ -37,7 +37,6 @@ def test_spmm_entry_points_reject_bad_arguments_without_a_gpu():
     assert L.spatha_spmm_plan_create(128, 128, 2, 8, 64, None, None, None, None, ctypes.byref(handle)) == 1
     # shape errors come before any device work
     assert L.spatha_spmm_plan_create(100, 128, 2, 8, 64, 1, 1, 1, None, ctypes.byref(handle)) == 2
-    assert L.spatha_spmm_plan_create(96, 128, 2, 8, 32, 16, 16, 16, None, ctypes.byref(handle)) == 3   # rows % 64: no kernel
     assert L.spatha_spmm_run(None, None, 8, None, None, 0, 0, None) == 1
     assert L.spatha_spmm_plan_destroy(None) == 0
     assert L.spatha_dense_gemm_f16(None, None, 8, 8, 8, None, None) == 1

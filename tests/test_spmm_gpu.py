@@ -272,8 +272,6 @@ def test_reference_encoded_matrices(gpu, path):
     z = np.load(path)
     n, m, v = int(z["n"]), int(z["m"]), int(z["v"])
     rows, cols = z["dense"].shape
-    if rows % 64:
-        pytest.skip("the kernels own 64-row tiles")
     vals = z["values"].astype(np.float16)
     rng = np.random.default_rng(1)
     N = 72
@@ -285,6 +283,47 @@ def test_reference_encoded_matrices(gpu, path):
     assert err.max() <= REL_TOL
     want = oracle.spmm(vals, z["metadata"].view(np.uint32), z["columns"].astype(np.uint32), rows, cols, n, m, v, B)
     assert np.abs(got - want.astype(np.float64)).max() <= REL_TOL * np.maximum(np.abs(exact), 1.0).max()
+
+
+HALF_TILE_ROWS_CASES = [
+    # rows, cols, N, m, v: rows % 64 == 32 (V a multiple of 32 only): the last 64-row wave tile is half padding
+    (32, 256, 136, 8, 32),
+    (96, 512, 264, 8, 32),
+    (160, 325, 72, 5, 32),
+    (96, 512, 520, 16, 96),
+    (480, 1024, 136, 32, 160),
+]
+
+
+@pytest.mark.parametrize("rows,cols,N,m,v", HALF_TILE_ROWS_CASES)
+def test_rows_not_a_multiple_of_64(gpu, rows, cols, N, m, v):
+    """Every kernel that takes such a plan, both layouts, with bias: bit-exact against the oracle, and nothing written
+    outside the rows x N (N x rows) output (the buffers carry a guard band)."""
+    print("case", rows, cols, N, m, v, flush=True)
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=rows + m, integer_values=True)
+    rng = np.random.default_rng(rows)
+    B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+    bias = rng.integers(-8, 9, size=rows).astype(np.float16)
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B)
+    want_t = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias, transposed_out=True)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    dB, dbias = _dev(B, gpu), _dev(bias, gpu)
+    guard = 4096
+    ran = 0
+    for variant in range(spatha.num_variants()):
+        if plan.kernel_name(N, 0, variant) is None:
+            continue
+        ran += 1
+        for transposed in (False, True):
+            buf = torch.full((rows * N + 2 * guard,), 7.0, dtype=torch.float16, device=gpu)
+            out = buf[guard:guard + rows * N].view((N, rows) if transposed else (rows, N))
+            plan.run(dB, bias=dbias if transposed else None, transposed_out=transposed, variant=variant, out=out)
+            torch.cuda.synchronize()
+            got = out.cpu().numpy()
+            ref = want_t if transposed else want
+            assert np.array_equal(got.view(np.uint16), ref.view(np.uint16)), (variant, transposed)
+            assert bool((buf[:guard] == 7.0).all()) and bool((buf[guard + rows * N:] == 7.0).all()), (variant, transposed)
+    assert ran >= 2
 
 
 def test_config1_gaussian_within_tolerance(gpu):

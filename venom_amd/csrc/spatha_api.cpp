@@ -222,7 +222,7 @@ int note_hip_error(hipError_t e) { return hip_fail(e); }
 void plan_layout(int rows, int m, int v, int ksp, PlanLayout* out) {
     out->S = (ksp + 31) / 32;
     out->half_tiles = (v % 64 != 0);      // V = 32, 96, ...: a wave tile spans two V blocks
-    out->apack_bytes = (size_t)(rows / 64) * out->S * APACK_BLOCK;
+    out->apack_bytes = (size_t)((rows + 63) / 64) * out->S * APACK_BLOCK;    // rows % 64 == 32: V a multiple of 32 only
     out->rowtab_bytes = (size_t)(rows / v) * out->S * 64 * 4;
     out->gtab_bytes = 0;
     if ((m <= 8 && rows % 256 == 0) || (m <= 16 && rows % 512 == 0 && !out->half_tiles)) {
@@ -365,7 +365,6 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
     int st = spatha::geometry_init(rows, cols, n, m, v, &geo);
     if (st) return st;
     if (!values_dev || !metadata_dev || !columns_dev) return SPATHA_ERR_BAD_ARGUMENT;
-    if (rows % 64 != 0) return SPATHA_ERR_UNSUPPORTED;   // kernels own 64-row wave tiles
     int ndev = 0;
     hipError_t e = hipGetDeviceCount(&ndev);
     if (e != hipSuccess || ndev == 0) { g_last_hip_error = (int)e; return SPATHA_ERR_NO_DEVICE; }
@@ -389,6 +388,12 @@ int spatha_spmm_plan_create(int rows, int cols, int n, int m, int v, const uint1
         (e = hipMemsetAsync(plan->zeros, 0, 1024, (hipStream_t)stream)) != hipSuccess ||
         (lay.gtab_bytes && (e = hipMalloc((void**)&plan->gtab, lay.gtab_bytes)) != hipSuccess) ||
         (e = spatha::plan_pack(plan, values_dev, metadata_dev, columns_dev, (hipStream_t)stream)) != hipSuccess) {
+        spatha_spmm_plan_destroy(plan);
+        return hip_fail(e);
+    }
+    // the derived copies are complete before the plan is handed out: a later run on another stream has nothing to order
+    // itself against
+    if ((e = hipStreamSynchronize((hipStream_t)stream)) != hipSuccess) {
         spatha_spmm_plan_destroy(plan);
         return hip_fail(e);
     }
@@ -430,7 +435,7 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
     p.gtab_bytes = (uint32_t)plan->gtab_bytes;
     p.rows = plan->geo.rows; p.cols = plan->geo.cols; p.N = N; p.S = plan->S; p.v = plan->geo.v; p.m = plan->geo.m;
     const int bm = spatha::spmm_variant_bm(var), bn = spatha::spmm_variant_bn(var);
-    p.tiles_m = plan->geo.rows / bm;
+    p.tiles_m = (plan->geo.rows + bm - 1) / bm;     // (only the half-tile kernels see rows % 64 != 0: a padded last tile)
     p.tiles_n = (N + bn - 1) / bn;
     p.b_bytes = (uint32_t)((uint64_t)plan->geo.cols * (uint64_t)N * 2u);     // only read by variants that passed variant_ok
     p.apack_bytes = (uint32_t)plan->apack_bytes;

@@ -485,9 +485,10 @@ __global__ __launch_bounds__(WN * 64) void spmm_half_kernel(SpmmParams p) {
     {
         const uint32_t* rt0 = p.rowtab + (int64_t)(m0 / p.v) * S * 64;
         const uint32_t* rt1 = p.rowtab + (int64_t)((m0 + 32) / p.v) * S * 64;
+        const bool second_half = m0 + 32 < p.rows;      // rows % 64 == 32: the last tile's second half is padding
         for (int i = tid; i < S * 128; i += WN * 64) {
             const int s = i >> 7, rho = i & 63;
-            const uint32_t r = ((i & 64) ? rt1 : rt0)[s * 64 + rho];
+            const uint32_t r = (i & 64) ? (second_half ? rt1[s * 64 + rho] : 0xffffffffu) : rt0[s * 64 + rho];
             lds_rt[i] = (r == 0xffffffffu) ? (uint16_t)0xffffu : (uint16_t)r;
         }
     }
@@ -536,10 +537,11 @@ __global__ __launch_bounds__(WN * 64) void spmm_half_kernel(SpmmParams p) {
     if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
         // per output column the lane holds rows 8*ib .. +7 (instructions 0, 1) and 32 + 8*ib .. +7 (2, 3)
         const int64_t row_lo = (int64_t)m0 + ib * 8, row_hi = row_lo + 32;
-        half8_t bias_lo, bias_hi;
+        const bool hi_rows = m0 + 32 < p.rows;
+        half8_t bias_lo, bias_hi = {};
         if (p.bias) {
             bias_lo = *(const half8_t*)(p.bias + row_lo);
-            bias_hi = *(const half8_t*)(p.bias + row_hi);
+            if (hi_rows) bias_hi = *(const half8_t*)(p.bias + row_hi);
         }
 #pragma unroll
         for (int nb = 0; nb < 4; nb++) {
@@ -559,7 +561,7 @@ __global__ __launch_bounds__(WN * 64) void spmm_half_kernel(SpmmParams p) {
             if (col < N) {
                 uint16_t* dst = p.C + (int64_t)col * p.rows;
                 *(half8_t*)(dst + row_lo) = lo;
-                *(half8_t*)(dst + row_hi) = hi;
+                if (hi_rows) *(half8_t*)(dst + row_hi) = hi;
             }
         }
     } else {
@@ -583,7 +585,7 @@ __global__ __launch_bounds__(WN * 64) void spmm_half_kernel(SpmmParams p) {
             const int row = 32 * (Lr >> 5) + 8 * (Lr & 3) + 4 * ((Lr >> 4) & 1) + ((Lr >> 2) & 3);
             const int col = n0 + wn * 64 + ch * 8;
             u32x4 v = *(const u32x4*)(stg + Lr * PITCH_C + ch * 16);
-            if (col < N) store_c16(p.C + ((int64_t)m0 + row) * N + col, v);
+            if (col < N && m0 + row < p.rows) store_c16(p.C + ((int64_t)m0 + row) * N + col, v);
         }
     }
 }

@@ -11,7 +11,8 @@ namespace spatha {
 // ---------------------------------------------------------------------------
 __global__ void pack_a_kernel(const uint16_t* __restrict__ values, const uint32_t* __restrict__ metadata, int rows,
                               int ksp, int S, int half_tiles, uint16_t* __restrict__ apack) {
-    const int64_t total = (int64_t)(rows / 64) * S * 4 * 64;
+    // (rows % 64 == 32 with V a multiple of 32 only: the last wave tile's second half is padding, packed as zeros)
+    const int64_t total = (int64_t)((rows + 63) / 64) * S * 4 * 64;
     const int ngroups = ksp / 2;
     for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x) {
         int lane = (int)(t & 63);
@@ -33,7 +34,7 @@ __global__ void pack_a_kernel(const uint16_t* __restrict__ values, const uint32_
             int fb = (kq >> 1) * 2 + (gp & 1);
             int kb = (kq & 1) * 2 + (gp >> 1);
             int g = s * 16 + fb * 4 + kb;                 // global group
-            if (g < ngroups) {
+            if (g < ngroups && r < rows) {
                 int tt = g >> 2, u = g & 3;
                 int64_t vi = R16 * 16 * (int64_t)ksp + (int64_t)tt * 128 + q * 32 + u * 8 + p * 4 + sbit * 2;
                 vals[2 * gp] = values[vi];
@@ -108,7 +109,7 @@ hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int
 
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
                        int m, int v, int ksp, int S, int half_tiles, uint16_t* apack, uint32_t* rowtab, hipStream_t stream) {
-    int64_t total_a = (int64_t)(rows / 64) * S * 256;
+    int64_t total_a = (int64_t)((rows + 63) / 64) * S * 256;
     int blocks_a = (int)((total_a + 255) / 256);
     if (blocks_a > 65535 * 8) blocks_a = 65535 * 8;
     hipLaunchKernelGGL(pack_a_kernel, dim3(blocks_a), dim3(256), 0, stream, values, metadata, rows, ksp, S, half_tiles, apack);

@@ -56,7 +56,6 @@ extern "C" int spatha_spmm_run_noalloc(int rows, int cols, int n, int m, int v, 
     int st = spatha_vnm_geometry_init(rows, cols, n, m, v, &geo);
     if (st) return st;
     if (!values_dev || !metadata_dev || !columns_dev) return SPATHA_ERR_BAD_ARGUMENT;
-    if (rows % 64 != 0) return SPATHA_ERR_UNSUPPORTED;
     spatha::PlanLayout lay;
     spatha::plan_layout(rows, m, v, geo.ksp, &lay);
     // [zeros 1 KiB][packed operands][row table][gather table], each at a multiple of 256 bytes

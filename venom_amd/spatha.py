@@ -95,6 +95,8 @@ class SpmmPlan:
                                                             None if bias is None else bias.data_ptr(), out.data_ptr(),
                                                             layout, _ACTIVATIONS[activation], variant,
                                                             _stream_ptr(self.device)), "spatha_spmm_run_fused")
+        # the kernel wrote through a raw pointer: tell torch, so that caches keyed on the tensor's version see the change
+        torch.autograd.graph.increment_version(out)
         return out
 
     def time(self, B, out, bias=None, transposed_out=False, variant=0, warmup=10, iters=100):

@@ -122,8 +122,11 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         // 128 x 128 tiles; 1024 x 4096, 512 tiles of 16 k-steps, 3 % slower).  m >= 16: the producer/consumer kernel with
         // 64 x 64 consumer blocks leads the tall-consumer form by 1-13 % up to 16 k-steps per tile (BERT-large, GPT-2-large
         // layers) and trails it by 1-3 % on long k-loops (GPT-3 layers).
-        const bool wide = wide_tiles >= 512 && (wide_tiles >= 1024 || plan->S >= 8);
-        const bool ws_wide = plan->geo.m >= 16 && plan->S <= 16;
+        // (every kernel id on the BERT layer shapes x N = 2048 .. 8192 x 2:10 .. 2:100: the 256-wide tile leads from 1024 tiles on,
+        // from 768 with two or more k-steps, from 512 with eight or more, and from 192 with a dozen or more)
+        const bool wide = wide_tiles >= 1024 || (wide_tiles >= 768 && plan->S >= 2) || (wide_tiles >= 512 && plan->S >= 8) ||
+                          (wide_tiles >= 192 && plan->S >= 12);
+        const bool ws_wide = plan->geo.m >= 16 && plan->S <= 16 && wide_tiles >= 768;    // (fewer tiles: the tall form, 8-10 % ahead)
         if (wide) {
             order[0] = ws_wide ? SPMM_VARIANT_W128x256_S3 : SPMM_VARIANT_T128x256_S3;
             order[1] = ws_wide ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x256_S3;
@@ -131,6 +134,15 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         } else {
             order[0] = SPMM_VARIANT_W128x128_S3;
             order[1] = SPMM_VARIANT_P128x128_S3;
+            // more than one round of 128 x 128 tiles but at most two, few k-steps: the same number of 64 x 256 tiles runs as
+            // one round of two co-resident workgroups per CU (768 x 768 x 8192, 3072 x 768 x 2048, 1024 x 1024 x 8192,
+            // 4096 x 1024 x 2048 at 128:2:10 .. 128:2:100: 5-30 % ahead)
+            const int64_t tiles128 = (int64_t)(plan->geo.rows / 128) * ((N + 127) / 128);
+            const int64_t cus = plan->cus > 0 ? plan->cus : 256;
+            if (plan->geo.m > 8 && tiles128 > cus && tiles128 <= 2 * cus && plan->S <= 8 && out_layout == SPATHA_OUT_ROW_MAJOR) {
+                order[1] = order[0];
+                order[0] = SPMM_VARIANT_P64x256_S2;
+            }
         }
         // m <= 8: dense staging leads the gathered tiles by 5-35 % as soon as its 256 x 128 tiles fill three quarters of
         // the CUs (BERT layer shapes, N = 2048 .. 16384; from 160 tiles on the GPT-2-large ones); with fewer tiles the 128 x 128
@@ -154,8 +166,9 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
             } else {
                 // m >= 16: 128 x 256 tiles at any tile count (5-15 % ahead of 128 x 128 on the BERT-large and GPT-2-large
                 // layer shapes, N = 4096 and 16384)
-                order[0] = ws_wide ? SPMM_VARIANT_W128x256_S3 : SPMM_VARIANT_T128x256_S3;
-                order[1] = ws_wide ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x256_S3;
+                const bool ws_wide_t = plan->geo.m >= 16 && plan->S <= 16;
+                order[0] = ws_wide_t ? SPMM_VARIANT_W128x256_S3 : SPMM_VARIANT_T128x256_S3;
+                order[1] = ws_wide_t ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x256_S3;
                 order[2] = SPMM_VARIANT_W128x128_S3;
             }
         }
@@ -173,7 +186,11 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         const int64_t tiles = (int64_t)(plan->geo.rows / 64) * ((N + 255) / 256);
         const bool long_k = plan->S >= 32 && (tiles >= 2048 || tiles <= 256);
         const bool ws_short = plan->geo.m >= 32 && out_layout != SPATHA_OUT_TRANSPOSED && tiles >= 2048 && plan->S <= 8;
-        order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : (ws_short ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_P64x256_S2);
+        // at most one tile per CU with a dozen or more k-steps: producer/consumer kernel (768 x 3072 / 1024 x 4096 x 4096 at 64:2:10
+        // and 64:2:20: 10-17 % ahead of the per-tile pipeline)
+        const int64_t cus64 = plan->cus > 0 ? plan->cus : 256;
+        const bool ws_one_round = !long_k && tiles <= cus64 && plan->S >= 12 && out_layout == SPATHA_OUT_ROW_MAJOR;
+        order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : ((ws_short || ws_one_round) ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_P64x256_S2);
         // 16 <= m < 32, many tiles, few k-steps, plain row-major output: the producer/consumer kernel with the write-out
         // deferred into the next tile's steps leads the pipeline by 5-8 % (3072 / 4096 x 1024 x 16384 at 64:2:16)
         if (!long_k && !ws_short && !fused && out_layout == SPATHA_OUT_ROW_MAJOR && plan->geo.m >= 16 && tiles >= 3072 &&
@@ -192,7 +209,8 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         const int64_t du_tiles = (int64_t)(plan->geo.rows / 512) * ((N + 127) / 128);
         const int64_t cus = plan->cus > 0 ? plan->cus : 256;
         const int64_t rounds = (du_tiles + cus - 1) / cus;
-        const bool whole_rounds = du_tiles >= cus && du_tiles * 10 >= rounds * cus * 9;
+        // (a single round three quarters full is enough: 3072 x 768 x 4096, 192 tiles, 10-12 % ahead of the 256 x 128 tiles)
+        const bool whole_rounds = rounds == 1 ? du_tiles * 4 >= cus * 3 : du_tiles * 10 >= rounds * cus * 9;
         const bool layout_ok = out_layout == SPATHA_OUT_ROW_MAJOR || du_tiles >= 2 * cus || plan->S >= 16;
         // (the form in two phase groups leads the one-group form by 3-8 % on every shape of that sweep)
         if (whole_rounds && layout_ok) return SPMM_VARIANT_UP512x128_S3;
@@ -206,8 +224,8 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         const int64_t rounds = (du_tiles + cus - 1) / cus;
         // long k-loops (GPT-3 projections at 64:2:16, 48 k-steps and more): ahead of every gathered form at 1.5 rounds too
         // (12288 x 12288 x 2048: 177 us against 188 us for the best of them and 262 us for the per-tile pipeline)
-        const bool whole_rounds = du_tiles * 10 >= rounds * cus * 9;
-        if (du_tiles >= cus && (whole_rounds || plan->S >= 32)) return SPMM_VARIANT_DU512x128_M16;
+        const bool whole_rounds = rounds == 1 ? du_tiles * 4 >= cus * 3 : du_tiles * 10 >= rounds * cus * 9;
+        if (whole_rounds || (du_tiles >= cus && plan->S >= 32)) return SPMM_VARIANT_DU512x128_M16;
     }
     for (int i = 0; i < 4; i++)
         if (variant_ok(plan, N, order[i], fused)) return order[i];

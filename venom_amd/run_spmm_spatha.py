@@ -7,6 +7,11 @@ instead).  Writes the driver's CSV rows (the reference's 24 columns, then micros
 reference's header.
 
     python -m venom_amd.run_spmm_spatha [--out spmm_bert_spatha.csv] [--tokens 4096,8192] [--v 64,128] [--all-variants]
+
+`--compare-kernels` answers a different question on the same points, in this process and with Gaussian data: how far is
+the library's automatic choice from the fastest kernel id that accepts the shape?  It times every id on every point
+(HIP events, 2 x 40 launches each), writes one JSON line per point to --out and prints the points where the choice is
+more than 5 % behind, then the geometric mean of automatic / best.
 """
 import argparse
 import os
@@ -60,6 +65,54 @@ def run_point(rows, cols, tokens, v, m, all_variants=False, num_variants=64):
     return (best[1], "") if best else (None, message or "no kernel accepted the shape")
 
 
+def compare_kernels(out_path, tokens, vs, ms):
+    """Automatic choice against the best kernel id, per point; returns the list of automatic / best ratios."""
+    import json
+    import math
+
+    import numpy as np
+    import torch
+
+    from . import format as F
+    from . import spatha
+
+    ratios = []
+    with open(out_path, "w") as f:
+        for rows, cols in LAYERS:
+            for v in vs:
+                if rows % v:
+                    continue
+                for m in ms:
+                    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=0, value_std=0.02)
+                    plan = spatha.SpmmPlan(torch.from_numpy(vals).cuda(), torch.from_numpy(meta.view(np.int32)).cuda(),
+                                           torch.from_numpy(columns.view(np.int32)).cuda(), rows, cols, 2, m, v)
+                    for N in tokens:
+                        gen = torch.Generator(device="cuda")
+                        gen.manual_seed(0)
+                        B = torch.randn((cols, N), generator=gen, device="cuda").half()
+                        out = torch.empty((rows, N), dtype=torch.float16, device="cuda")
+                        auto = plan.kernel_name(N, 0, 0)
+                        plan.time(B, out, warmup=30, iters=30)
+                        times = {}
+                        for variant in range(1, spatha.num_variants()):
+                            name = plan.kernel_name(N, 0, variant)
+                            if name is not None:
+                                times[name] = min(plan.time(B, out, variant=variant, warmup=5, iters=40) for _ in range(2)) * 1e3
+                        best = min(times, key=times.get)
+                        ratio = times[auto] / times[best]
+                        ratios.append(ratio)
+                        f.write(json.dumps({"rows": rows, "cols": cols, "N": N, "v": v, "m": m, "auto": auto, "best": best,
+                                            "ratio": round(ratio, 3), "us": {k: round(t, 2) for k, t in times.items()}}) + "\n")
+                        f.flush()
+                        if ratio > 1.05:
+                            print("%dx%dx%d %d:2:%d: %s %.2f us, best %s %.2f us (%.3f)" %
+                                  (rows, cols, N, v, m, auto, times[auto], best, times[best], ratio), flush=True)
+    print("%d points: automatic / best, geometric mean %.4f; within 5 %%: %d, within 10 %%: %d, worst %.3f" %
+          (len(ratios), math.exp(sum(math.log(r) for r in ratios) / len(ratios)), sum(r <= 1.05 for r in ratios),
+           sum(r <= 1.10 for r in ratios), max(ratios)), flush=True)
+    return ratios
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--out", default="spmm_bert_spatha.csv")
@@ -67,7 +120,14 @@ def main(argv=None):
     ap.add_argument("--v", default="64,128")
     ap.add_argument("--m", default=",".join(str(x) for x in M_VALUES))
     ap.add_argument("--all-variants", action="store_true")
+    ap.add_argument("--compare-kernels", action="store_true",
+                    help="time every kernel id on every point in this process (Gaussian data) and compare with the automatic choice")
     args = ap.parse_args(argv)
+    if args.compare_kernels:
+        compare_kernels(args.out if args.out != "spmm_bert_spatha.csv" else "spmm_bert_kernels.jsonl",
+                        [int(x) for x in args.tokens.split(",")], [int(x) for x in args.v.split(",")],
+                        [int(x) for x in args.m.split(",")])
+        return 0
     failures = 0
     with open(args.out, "w") as f:
         f.write(HEADER + "\n")

@@ -72,3 +72,17 @@ def test_unified_kernels_use_no_scratch_memory(tmp_path):
                 found[name] = int(line.split(":", 1)[1])
     assert len(found) >= 4, found                 # two output layouts x (m <= 8 in two phase groups, 8 < m <= 16)
     assert all(size == 0 for size in found.values()), found
+
+
+def test_torch_extension_exposes_the_operator():
+    """The PyTorch C++ extension is built in place and names the reference operator's fifteen arguments in order
+    (end2end/spatha_mod/block_sparse/api/spatha.cu:41-65); calling it needs a GPU and is left to the GPU tests."""
+    from venom_amd import spatha
+    ext = spatha._extension()
+    doc = ext.spmm.__doc__
+    names = ["A_metadata", "A_indices", "A_values", "rhs_matrix", "bias", "A_num_rows", "A_num_cols", "B_num_cols",
+             "vec_length", "n", "m", "nnz", "seed", "mbrow", "brow"]
+    at = [doc.index(name + ":") for name in names]
+    assert at == sorted(at)
+    assert ext.plan_cache_size() == 0
+    ext.clear_plan_cache()

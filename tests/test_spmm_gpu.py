@@ -468,6 +468,37 @@ def test_spmm_operator_signature(gpu):
     assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))
 
 
+def test_operator_plan_cache_follows_the_weights(gpu):
+    """The extension keeps one plan per (weights, version): a second call reuses it, an in-place update of the values
+    gets a new one, and the results follow the update."""
+    rows, cols, N, m, v = 128, 256, 72, 8, 64
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=21, integer_values=True)
+    B = np.random.default_rng(21).integers(-4, 5, size=(cols, N)).astype(np.float16)
+    spatha.clear_plan_cache()
+    ext = spatha._extension()
+    dv, dm, dc, dB = _dev(vals, gpu), _dev(meta, gpu), _dev(columns, gpu), _dev(B, gpu)
+    a = spatha.spmm(dm, dc, dv, dB, None, rows, cols, N, v, 2, m)
+    b = spatha.spmm(dm, dc, dv, dB, None, rows, cols, N, v, 2, m)
+    assert ext.plan_cache_size() == 1 and torch.equal(a, b)
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, transposed_out=True)
+    assert np.array_equal(a.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    dv.mul_(2)                                   # in place: same address, new version
+    c = spatha.spmm(dm, dc, dv, dB, None, rows, cols, N, v, 2, m)
+    assert ext.plan_cache_size() == 2
+    want2 = oracle.spmm((vals * 2).astype(np.float16), meta, columns, rows, cols, 2, m, v, B, transposed_out=True)
+    assert np.array_equal(c.cpu().numpy().view(np.uint16), want2.view(np.uint16))
+    # the fused operator: same plan, row-major output with bias
+    bias = np.random.default_rng(22).integers(-3, 4, size=rows).astype(np.float16)
+    d = spatha.spmm_fused(dm, dc, dv, dB, _dev(bias, gpu), rows, cols, v, 2, m)
+    assert ext.plan_cache_size() == 2 and tuple(d.shape) == (rows, N)
+    want3 = oracle.spmm((vals * 2).astype(np.float16), meta, columns, rows, cols, 2, m, v, B, bias=bias, transposed_out=True)
+    assert np.array_equal(d.cpu().numpy().view(np.uint16), np.ascontiguousarray(want3.T).view(np.uint16))
+    with pytest.raises(RuntimeError):
+        spatha.spmm(dm, dc, dv, dB, None, rows, cols, N, v, 2, m, 0, 0, 16, 4)       # only mbrow 32 / brow 4 exist
+    spatha.clear_plan_cache()
+    assert ext.plan_cache_size() == 0
+
+
 def test_bias_rounding_is_one_fp16_add(gpu):
     rows, cols, N, m, v = 128, 256, 64, 8, 64
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=9, value_std=1.0)

@@ -17,6 +17,7 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "build")
 LIB = os.path.join(LIBDIR, "libspatha.so")
 BENCH = os.path.join(LIBDIR, "benchmark_spmm")
+TORCH_EXT = os.path.join(HERE, "_spatha_torch.so")       # the PyTorch C++ extension (operator `spmm`), importable in place
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
@@ -47,10 +48,36 @@ def _compile_all(jobs, verbose):
             f.result()
 
 
-def build(verbose=False, with_driver=True, with_out_32b=False):
+def _torch_ext_compile():
+    """g++ command for the PyTorch extension's only source (csrc/spatha_torch.cpp): written against the ROCm build of
+    PyTorch directly, so it goes through the host compiler as it is."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+    incs = cpp_extension.include_paths() + [sysconfig.get_paths()["include"], "/opt/rocm/include"]
+    return (["g++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+             "-DTORCH_EXTENSION_NAME=_spatha_torch", "-DTORCH_API_INCLUDE_EXTENSION_H",
+             "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)] +
+            ["-isystem" + i for i in incs] +
+            ["-c", os.path.join(CSRC, "spatha_torch.cpp"), "-o", os.path.join(OBJDIR, "spatha_torch.cpp.o")])
+
+
+def _torch_ext_link(verbose):
+    from torch.utils import cpp_extension
+    libdirs = cpp_extension.library_paths()
+    _run(["g++", "-shared", "-fPIC", "-o", TORCH_EXT, os.path.join(OBJDIR, "spatha_torch.cpp.o"), "-L" + LIBDIR, "-lspatha",
+          "-Wl,-rpath,$ORIGIN/lib"] + ["-L" + d for d in libdirs] + ["-Wl,-rpath," + d for d in libdirs] +
+         ["-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python"], verbose)
+    return TORCH_EXT
+
+
+def build(verbose=False, with_driver=True, with_out_32b=False, with_torch_ext=True):
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
     objs, jobs = [], []
+    if with_torch_ext:
+        jobs.append(_torch_ext_compile())
     for src in CXX_SOURCES:
         obj = os.path.join(OBJDIR, src + ".o")
         jobs.append(["g++"] + CXX_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
@@ -71,6 +98,8 @@ def build(verbose=False, with_driver=True, with_out_32b=False):
         _run([HIPCC] + HIP_FLAGS + [os.path.join(CSRC, "benchmark_spmm.cpp"), os.path.join(CSRC, "vendor_gemm.cpp"), "-o", BENCH,
                                     "-L" + LIBDIR, "-lspatha", "-Wl,-rpath,$ORIGIN", "-L/opt/rocm/lib", "-lhipblaslt", "-lgomp"],
              verbose)
+    if with_torch_ext:
+        _torch_ext_link(verbose)
     return LIB
 
 

@@ -1,0 +1,180 @@
+// PyTorch C++ extension for the operator (end2end/spatha_mod/block_sparse/api/spatha.cu:41-65 in the reference:
+// `spmm(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_cols, B_num_cols, vec_length, n, m, nnz,
+// seed, mbrow, brow) -> Tensor`, bound with pybind11 under the name `spmm`).  Same argument order and meaning; the work
+// itself goes through the C ABI of include/spatha.h on torch's current HIP stream.  Written against the ROCm build of
+// PyTorch directly (c10/hip, ATen/hip), not passed through a source translator.
+//
+// The reference packs nothing per call (its kernel reads the canonical arrays); here the derived operand copies live
+// in a plan, so the extension keeps a cache of plans keyed by the identity and version of the three weight tensors.
+// An entry holds the tensors, so an address cannot be recycled under a stale plan.
+
+#include <torch/extension.h>
+
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+
+#include <list>
+#include <mutex>
+#include <stdexcept>
+#include <string>
+#include <tuple>
+#include <unordered_map>
+
+#include "../../include/spatha.h"
+
+namespace {
+
+struct PlanKey {
+    const void *values, *metadata, *columns;
+    uint32_t v_values, v_metadata, v_columns;
+    int rows, cols, n, m, v, device;
+    bool operator==(const PlanKey& o) const {
+        return values == o.values && metadata == o.metadata && columns == o.columns && v_values == o.v_values &&
+               v_metadata == o.v_metadata && v_columns == o.v_columns && rows == o.rows && cols == o.cols && n == o.n &&
+               m == o.m && v == o.v && device == o.device;
+    }
+};
+struct PlanKeyHash {
+    size_t operator()(const PlanKey& k) const {
+        size_t h = std::hash<const void*>()(k.values);
+        auto mix = [&h](size_t x) { h ^= x + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2); };
+        mix(std::hash<const void*>()(k.metadata));
+        mix(std::hash<const void*>()(k.columns));
+        mix(((size_t)k.v_values << 32) ^ ((size_t)k.v_metadata << 16) ^ k.v_columns);
+        mix(((size_t)k.rows << 32) ^ (size_t)k.cols);
+        mix(((size_t)k.m << 40) ^ ((size_t)k.v << 20) ^ ((size_t)k.n << 8) ^ (size_t)k.device);
+        return h;
+    }
+};
+struct PlanEntry {
+    PlanKey key;
+    spatha_spmm_plan* plan;
+    torch::Tensor values, metadata, columns;      // kept alive for the plan's lifetime
+};
+
+constexpr size_t kMaxPlans = 1024;
+std::mutex g_lock;
+std::list<PlanEntry> g_lru;                                                           // most recently used first
+std::unordered_map<PlanKey, std::list<PlanEntry>::iterator, PlanKeyHash> g_index;
+
+void check(int status, const char* what) {
+    if (status != SPATHA_OK)
+        throw std::runtime_error(std::string(what) + ": " + spatha_status_string(status) +
+                                 (status == SPATHA_ERR_HIP ? " (HIP error " + std::to_string(spatha_last_hip_error()) + ")" : ""));
+}
+
+void check_weight(const torch::Tensor& t, c10::ScalarType a, c10::ScalarType b, const char* name) {
+    TORCH_CHECK(t.is_cuda(), name, " must live on the GPU");
+    TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+    TORCH_CHECK(t.scalar_type() == a || t.scalar_type() == b, name, " has the wrong dtype");
+}
+
+uint32_t version_of(const torch::Tensor& t) { return (uint32_t)t.unsafeGetTensorImpl()->version_counter().current_version(); }
+
+spatha_spmm_plan* plan_for(const torch::Tensor& values, const torch::Tensor& metadata, const torch::Tensor& columns, int rows,
+                           int cols, int n, int m, int v, hipStream_t stream) {
+    PlanKey key{values.data_ptr(), metadata.data_ptr(), columns.data_ptr(), version_of(values), version_of(metadata),
+                version_of(columns), rows, cols, n, m, v, (int)values.get_device()};
+    std::lock_guard<std::mutex> guard(g_lock);
+    auto hit = g_index.find(key);
+    if (hit != g_index.end()) {
+        g_lru.splice(g_lru.begin(), g_lru, hit->second);
+        return hit->second->plan;
+    }
+    spatha_spmm_plan* plan = nullptr;
+    check(spatha_spmm_plan_create(rows, cols, n, m, v, (const uint16_t*)values.data_ptr(), (const uint32_t*)metadata.data_ptr(),
+                                  (const uint32_t*)columns.data_ptr(), stream, &plan),
+          "spatha_spmm_plan_create");
+    g_lru.push_front(PlanEntry{key, plan, values, metadata, columns});
+    g_index[key] = g_lru.begin();
+    while (g_lru.size() > kMaxPlans) {
+        PlanEntry& old = g_lru.back();
+        spatha_spmm_plan_destroy(old.plan);
+        g_index.erase(old.key);
+        g_lru.pop_back();
+    }
+    return plan;
+}
+
+torch::Tensor run(const torch::Tensor& A_metadata, const torch::Tensor& A_indices, const torch::Tensor& A_values,
+                  const torch::Tensor& rhs_matrix, const c10::optional<torch::Tensor>& bias, int rows, int cols, int v, int n, int m,
+                  bool transposed_out, int activation, bool fused) {
+    check_weight(A_values, torch::kFloat16, torch::kFloat16, "A_values");
+    check_weight(A_metadata, torch::kInt32, torch::kInt32, "A_metadata");
+    check_weight(A_indices, torch::kInt32, torch::kInt32, "A_indices");
+    check_weight(rhs_matrix, torch::kFloat16, torch::kFloat16, "rhs_matrix");
+    TORCH_CHECK(rhs_matrix.dim() == 2 && rhs_matrix.size(0) == cols, "rhs_matrix must be [A_num_cols, tokens]");
+    TORCH_CHECK(rhs_matrix.get_device() == A_values.get_device(), "operands live on different devices");
+    const uint16_t* bias_ptr = nullptr;
+    if (bias.has_value() && bias->defined()) {
+        check_weight(*bias, torch::kFloat16, torch::kFloat16, "bias");
+        TORCH_CHECK(bias->numel() == rows, "bias must have A_num_rows elements");
+        bias_ptr = (const uint16_t*)bias->data_ptr();
+    }
+    const int tokens = (int)rhs_matrix.size(1);
+    const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(A_values.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(A_values.get_device()).stream();
+    spatha_spmm_plan* plan = plan_for(A_values.detach(), A_metadata, A_indices, rows, cols, n, m, v, stream);
+    torch::Tensor out = torch::empty(transposed_out ? std::vector<int64_t>{tokens, rows} : std::vector<int64_t>{rows, tokens},
+                                     rhs_matrix.options());
+    const int layout = transposed_out ? SPATHA_OUT_TRANSPOSED : SPATHA_OUT_ROW_MAJOR;
+    if (fused)
+        check(spatha_spmm_run_fused(plan, (const uint16_t*)rhs_matrix.data_ptr(), tokens, bias_ptr, (uint16_t*)out.data_ptr(), layout,
+                                    activation, 0, stream),
+              "spatha_spmm_run_fused");
+    else
+        check(spatha_spmm_run(plan, (const uint16_t*)rhs_matrix.data_ptr(), tokens, bias_ptr, (uint16_t*)out.data_ptr(), layout, 0,
+                              stream),
+              "spatha_spmm_run");
+    return out;
+}
+
+// out[B_num_cols, A_num_rows] = (A_vnm @ rhs_matrix).T + bias, fp16: the reference operator.  vec_length is V and is
+// honoured at run time; nnz and seed are accepted and unused, as there; mbrow / brow must be 32 / 4, the only layout the
+// format defines.
+torch::Tensor spmm(torch::Tensor A_metadata, torch::Tensor A_indices, torch::Tensor A_values, torch::Tensor rhs_matrix,
+                   c10::optional<torch::Tensor> bias, int A_num_rows, int A_num_cols, int B_num_cols, int vec_length, int n, int m,
+                   int nnz, int seed, int mbrow, int brow) {
+    (void)nnz;
+    (void)seed;
+    TORCH_CHECK(mbrow == 32 && brow == 4, "only mbrow=32, brow=4 is defined for the V:N:M layout");
+    TORCH_CHECK(rhs_matrix.dim() == 2 && rhs_matrix.size(1) == B_num_cols, "B_num_cols does not match rhs_matrix");
+    return run(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_cols, vec_length, n, m, true, SPATHA_ACT_NONE,
+               false);
+}
+
+// act((A_vnm @ rhs_matrix) + bias) as [A_num_rows, tokens] (ready to be the rhs of the next spmm) or, with
+// transposed_out, as [tokens, A_num_rows]; activation: 0 none, 1 GELU (erf), 2 GELU (tanh)
+torch::Tensor spmm_fused(torch::Tensor A_metadata, torch::Tensor A_indices, torch::Tensor A_values, torch::Tensor rhs_matrix,
+                         c10::optional<torch::Tensor> bias, int A_num_rows, int A_num_cols, int vec_length, int n, int m,
+                         int activation, bool transposed_out) {
+    return run(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_cols, vec_length, n, m, transposed_out,
+               activation, true);
+}
+
+void clear_plan_cache() {
+    std::lock_guard<std::mutex> guard(g_lock);
+    for (PlanEntry& e : g_lru) spatha_spmm_plan_destroy(e.plan);
+    g_lru.clear();
+    g_index.clear();
+}
+
+int64_t plan_cache_size() {
+    std::lock_guard<std::mutex> guard(g_lock);
+    return (int64_t)g_lru.size();
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
+    mod.def("spmm", &spmm, "V:N:M SpMM: (A_vnm @ rhs).T + bias", py::arg("A_metadata"), py::arg("A_indices"), py::arg("A_values"),
+            py::arg("rhs_matrix"), py::arg("bias"), py::arg("A_num_rows"), py::arg("A_num_cols"), py::arg("B_num_cols"),
+            py::arg("vec_length"), py::arg("n"), py::arg("m"), py::arg("nnz") = 0, py::arg("seed") = 0, py::arg("mbrow") = 32,
+            py::arg("brow") = 4);
+    mod.def("spmm_fused", &spmm_fused, "V:N:M SpMM with bias and activation in the write-out", py::arg("A_metadata"),
+            py::arg("A_indices"), py::arg("A_values"), py::arg("rhs_matrix"), py::arg("bias"), py::arg("A_num_rows"),
+            py::arg("A_num_cols"), py::arg("vec_length"), py::arg("n"), py::arg("m"), py::arg("activation") = 0,
+            py::arg("transposed_out") = false);
+    mod.def("clear_plan_cache", &clear_plan_cache, "drop every cached plan");
+    mod.def("plan_cache_size", &plan_cache_size, "number of cached plans");
+}

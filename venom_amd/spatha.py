@@ -4,7 +4,6 @@ libspatha.so through its C ABI.  torch is used for device memory and the
 current stream only."""
 import ctypes
 import weakref
-from collections import OrderedDict
 
 import torch
 
@@ -111,29 +110,20 @@ class SpmmPlan:
         return ms.value
 
 
-# plans of matrices already seen by spmm(), keyed by the identity and version of
-# the three tensors; the entry keeps the tensors alive so that an address cannot
-# be recycled under a stale plan
-_PLAN_CACHE = OrderedDict()
-_PLAN_CACHE_MAX = 1024
-
-
-def _plan_for(values, metadata, columns, rows, cols, n, m, v):
-    key = (values.data_ptr(), metadata.data_ptr(), columns.data_ptr(), values._version, metadata._version,
-           columns._version, rows, cols, n, m, v)
-    hit = _PLAN_CACHE.get(key)
-    if hit is not None:
-        _PLAN_CACHE.move_to_end(key)
-        return hit[0]
-    plan = SpmmPlan(values, metadata, columns, rows, cols, n, m, v)
-    _PLAN_CACHE[key] = (plan, values, metadata, columns)
-    while len(_PLAN_CACHE) > _PLAN_CACHE_MAX:
-        _PLAN_CACHE.popitem(last=False)
-    return plan
+def _extension():
+    """The PyTorch C++ extension that holds the operator (csrc/spatha_torch.cpp, built in place by `python -m
+    venom_amd.build`): `spmm` with the reference's signature, `spmm_fused`, and the cache of plans of the matrices they
+    have seen.  There is no fallback: without it the operator raises."""
+    try:
+        from . import _spatha_torch
+    except ImportError as e:
+        raise RuntimeError("the PyTorch extension venom_amd/_spatha_torch.so is not built or does not load (%s): run "
+                           "`python -m venom_amd.build`" % e)
+    return _spatha_torch
 
 
 def clear_plan_cache():
-    _PLAN_CACHE.clear()
+    _extension().clear_plan_cache()
 
 
 def transpose(x):
@@ -178,21 +168,19 @@ def spmm(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_co
          nnz=0, seed=0, mbrow=32, brow=4):
     """out[B_num_cols, A_num_rows] = (A_vnm @ rhs_matrix).T + bias, fp16.
 
-    Same argument order and meaning as the reference operator
-    (end2end/bert_pytorch.py:89-104).  vec_length is V and is honoured at run
-    time; nnz and seed are accepted and unused, as there; mbrow/brow must be
-    32/4, the only layout the format defines.  Runs on torch's current stream."""
-    if mbrow != 32 or brow != 4:
-        raise ValueError("only mbrow=32, brow=4 is defined for the V:N:M layout")
-    if rhs_matrix.shape[1] != B_num_cols:
-        raise ValueError("B_num_cols does not match rhs_matrix")
-    plan = _plan_for(A_values.detach(), A_metadata, A_indices, A_num_rows, A_num_cols, n, m, vec_length)
-    return plan.run(rhs_matrix, bias=bias, transposed_out=True)
+    Same argument order and meaning as the reference operator (end2end/bert_pytorch.py:89-104), and like it a
+    function of a PyTorch C++ extension (end2end/spatha_mod/block_sparse/api/spatha.cu:41-65).  vec_length is V and
+    is honoured at run time; nnz and seed are accepted and unused, as there; mbrow/brow must be 32/4, the only layout
+    the format defines.  Runs on torch's current stream."""
+    return _extension().spmm(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_cols, B_num_cols, vec_length,
+                             n, m, nnz, seed, mbrow, brow)
 
 
 def spmm_fused(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_cols, vec_length, n, m,
                activation="none", transposed_out=False):
     """act((A_vnm @ rhs_matrix) + bias), fp16, as [A_num_rows, tokens] (default: ready to be the rhs of the next
     spmm without a transposed copy) or, with transposed_out, as [tokens, A_num_rows] like `spmm`."""
-    plan = _plan_for(A_values.detach(), A_metadata, A_indices, A_num_rows, A_num_cols, n, m, vec_length)
-    return plan.run(rhs_matrix, bias=bias, transposed_out=transposed_out, activation=activation)
+    if activation not in _ACTIVATIONS:
+        raise ValueError("unknown activation %r" % (activation,))
+    return _extension().spmm_fused(A_metadata, A_indices, A_values, rhs_matrix, bias, A_num_rows, A_num_cols, vec_length, n, m,
+                                   _ACTIVATIONS[activation], transposed_out)

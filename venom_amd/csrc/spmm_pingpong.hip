@@ -4,8 +4,8 @@
 // wave's rows go from L2 straight into its registers, only the dense B stage (32 KB) lives in LDS and serves all eight
 // 64-row blocks, every wave issues an eighth of each stage's DMA.  What differs is WHEN a wave issues its vector-memory
 // instructions.  There, all eight waves spread their loads between their groups of matrix instructions; a load whose
-// issue blocks (the memory pipeline is the busiest unit of this kernel: 88 wave-instructions of 1 KB per step, 16 clocks
-// each) then stops that wave's matrix instructions, and since the waves run in lockstep between two barriers, the other
+// issue blocks (the memory pipeline is the busiest unit of this kernel: 88 wave-instructions, 72 KB per step, through a path that
+// delivers about 53 B per clock) then stops that wave's matrix instructions, and since the waves run in lockstep between two barriers, the other
 // wave of the SIMD is blocked in the same place.  Here the two waves of a SIMD belong to different phase groups:
 //   group X (waves 0-3):  barrier | burst of the step's 11 loads | matrix phase (8 x 4 instructions, reads interleaved)
 //   group Y (waves 4-7):  barrier | matrix phase                 | burst
@@ -30,6 +30,28 @@
 //   the gather table is loaded)   32 write-out without its global stores
 #ifndef SPATHA_UP_KNOBS
 #define SPATHA_UP_KNOBS 0
+#endif
+
+// Development-only cycle accounting (-DSPATHA_DEV_PROFILE): every wave sums the s_memtime ticks it spends (0) issuing its
+// bursts, (1) in matrix phases, (2) in the wait for its loads, (3) at the step barrier, (4) in write-outs; lane 0 writes the
+// five sums to prof[(workgroup * 8 + wave) * 8 ..].
+#ifdef SPATHA_DEV_PROFILE
+#define SPATHA_UP_PROF_DECL long long up_prof_t = __builtin_readcyclecounter(), up_prof_sum[5] = {0, 0, 0, 0, 0};
+#define SPATHA_UP_PROF_MARK(SLOT)                                \
+    {                                                            \
+        const long long now = __builtin_readcyclecounter();      \
+        up_prof_sum[SLOT] += now - up_prof_t;                    \
+        up_prof_t = now;                                         \
+    }
+#define SPATHA_UP_PROF_FLUSH                                                              \
+    if (p.prof && lane == 0) {                                                            \
+        long long* dst = p.prof + ((int64_t)blockIdx.x * 8 + wave) * 8;                   \
+        for (int k = 0; k < 5; k++) dst[k] = up_prof_sum[k];                              \
+    }
+#else
+#define SPATHA_UP_PROF_DECL
+#define SPATHA_UP_PROF_MARK(SLOT)
+#define SPATHA_UP_PROF_FLUSH
 #endif
 
 namespace spatha {
@@ -159,9 +181,9 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
     uint32_t c_stage = 0;
 
     // The matrix phase of one k-step: 8 fragments of B (4 transposing reads each), 4 matrix instructions per fragment.
-    // Fine interleave: behind every matrix instruction of fragment f goes one read (address + ds_read) of fragment
-    // f + 2, so that the wave's address arithmetic and LDS issue run in the shadow of its own matrix instructions
-    // (a matrix instruction occupies the unit for 16 clocks and its issue for 4).  Three fragment buffers in rotation.
+    // Fine interleave: behind every matrix instruction of fragment f goes one read of fragment f + 2, so that the
+    // wave's LDS issue runs in the shadow of its own matrix instructions (a matrix instruction occupies the unit for
+    // 16 clocks and its issue for 4).  Three fragment buffers in rotation.
     auto matrix_phase = [&](const ASet& x) {
         const uint32_t st = smem_base + c_stage;
         uint32_t base[4];
@@ -174,9 +196,17 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
         for (int mb = 0; mb < 4; mb++) a_cur[mb] = __builtin_bit_cast(half8_t, x.a[mb]);
         const uint32_t ix[2] = {x.i0, x.i1};
         half16_t bf[3];
-        auto read_part = [&](half16_t& dst, int nb8, int fb) {
-            const uint32_t addr = base[fb] ^ (uint32_t)(nb8 << 5);
-            short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)addr);
+        // The four read addresses of a fragment are computed together, ahead of the four matrix instructions they follow:
+        // a vector ALU instruction BETWEEN two matrix instructions holds the second one back (measured on the matrix
+        // phase alone, one wave per SIMD: 952 clocks per step with an xor ahead of every read, 760 with the xors in
+        // groups, 640 with none), an LDS instruction does not.
+        uint32_t ad[4];
+        auto addresses = [&](int nb8) {
+#pragma unroll
+            for (int fb = 0; fb < 4; fb++) ad[fb] = base[fb] ^ (uint32_t)(nb8 << 5);
+        };
+        auto read_part = [&](half16_t& dst, int fb) {
+            short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)ad[fb]);
             half4_t h4 = __builtin_bit_cast(half4_t, t4);
             dst[fb * 4 + 0] = h4[0];
             dst[fb * 4 + 1] = h4[1];
@@ -184,42 +214,52 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
             dst[fb * 4 + 3] = h4[3];
         };
 #pragma unroll
-        for (int k = 0; k < 2; k++)
+        for (int k = 0; k < 2; k++) {
+            addresses(k);
 #pragma unroll
-            for (int fb = 0; fb < 4; fb++) read_part(bf[k], k, fb);
+            for (int fb = 0; fb < 4; fb++) read_part(bf[k], fb);
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int nb8 = 0; nb8 < 8; nb8++) {
+            if (nb8 + 2 < 8) addresses(nb8 + 2);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int mb = 0; mb < 4; mb++) {
                 float4_t& c = acc[nb8 >> 2][mb][nb8 & 3];
                 if (mb & 1) c = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[mb], bf[nb8 % 3], c, (int)ix[mb >> 1], 0, 1);
                 else c = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[mb], bf[nb8 % 3], c, (int)ix[mb >> 1], 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                if (nb8 + 2 < 8) read_part(bf[(nb8 + 2) % 3], nb8 + 2, mb);
+                if (nb8 + 2 < 8) read_part(bf[(nb8 + 2) % 3], mb);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
 
     // one k-step; `cur` holds its operands, `other` is the wave's second set
+    SPATHA_UP_PROF_DECL
     auto do_step = [&](ASet& cur, ASet& other) {
         __syncthreads();        // stage q has landed for every wave; every wave has left stage q - 1
+        SPATHA_UP_PROF_MARK(3)
         if constexpr (!LATE) {
             load_set(other);    // operands of step q + 1
             issue_stage();      // share of stage q + 2
             if (UP_KNOBS & 8) __syncthreads();
+            SPATHA_UP_PROF_MARK(0)
         }
         if (!(LATE && (UP_KNOBS & 4))) matrix_phase(cur);
+        SPATHA_UP_PROF_MARK(1)
         c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
         // Everything this wave has in flight, issued one matrix phase ago: X, its burst of this step (operands of step
         // q + 1, share of stage q + 2); Y, its burst of the step before (operands of step q + 1, share of stage q + 1).
         // Always here, never under a condition, and ahead of the tile's stores, which a later wait would sit out too.
         SPATHA_UP_WAIT_ALL();
+        SPATHA_UP_PROF_MARK(2)
         if constexpr (LATE) {
             if (UP_KNOBS & 8) __syncthreads();
             load_set(cur);      // operands of step q + 2
             issue_stage();      // share of stage q + 2
+            SPATHA_UP_PROF_MARK(0)
         }
         if (++c_step == S) {
             c_step = 0;
@@ -249,12 +289,14 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
             }
             zero_acc();
             walk.next(c_tm, c_tn);
+            SPATHA_UP_PROF_MARK(4)
         }
     };
     for (int q = 0; q < Q; q += 2) {
         do_step(s0, s1);
         if (q + 1 < Q) do_step(s1, s0);
     }
+    SPATHA_UP_PROF_FLUSH
 #undef SPATHA_UP_WAIT_ALL
 }
 

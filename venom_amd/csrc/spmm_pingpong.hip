@@ -72,7 +72,7 @@ __device__ __forceinline__ void pload_b64(u32x2& r, uint32_t voff, i32x4 rsrc, u
 // The whole life of one wave.  LATE is the wave's phase group (false: X, true: Y), a template argument so that each group
 // runs straight-line code of its own: an operand set that is in flight must never meet, at a join of two paths, a
 // version of itself that is not (the register copy the compiler may place there would copy a value that has not arrived).
-template <int OUT_LAYOUT, bool FUSE, bool LATE>
+template <int OUT_LAYOUT, bool FUSE, bool GROUPED, bool LATE>
 __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& walk, char* smem, uint32_t smem_base, int wave,
                                         int lane) {
     using Cfg = UpCfg;
@@ -196,17 +196,22 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
         for (int mb = 0; mb < 4; mb++) a_cur[mb] = __builtin_bit_cast(half8_t, x.a[mb]);
         const uint32_t ix[2] = {x.i0, x.i1};
         half16_t bf[3];
-        // The four read addresses of a fragment are computed together, ahead of the four matrix instructions they follow:
-        // a vector ALU instruction BETWEEN two matrix instructions holds the second one back (measured on the matrix
-        // phase alone, one wave per SIMD: 952 clocks per step with an xor ahead of every read, 760 with the xors in
-        // groups, 640 with none), an LDS instruction does not.
+        // Where the read addresses are computed is a template argument.  A vector ALU instruction BETWEEN two matrix
+        // instructions holds the second one back (measured on the matrix phase alone, one wave per SIMD: 952 clocks per
+        // step with an xor ahead of every read, 760 with the xors in groups of four, 640 with none), an LDS instruction
+        // does not.  GROUPED computes a fragment's four addresses together, ahead of the four matrix instructions its
+        // reads follow: 3-4 % faster wherever the clock holds (2:4, 2:5, integer-valued operands).  With Gaussian
+        // operands at m >= 7 it does not: the denser matrix phases run into the GPU's power management, launches
+        // take anything from 54 to 72 us and the sustained mean is 65-68 us against a steady 58 us with the xors left
+        // between the matrix instructions - so that form stays for m > 5 (chosen at launch).
         uint32_t ad[4];
         auto addresses = [&](int nb8) {
 #pragma unroll
             for (int fb = 0; fb < 4; fb++) ad[fb] = base[fb] ^ (uint32_t)(nb8 << 5);
         };
-        auto read_part = [&](half16_t& dst, int fb) {
-            short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)ad[fb]);
+        auto read_part = [&](half16_t& dst, int nb8, int fb) {
+            const uint32_t addr = GROUPED ? ad[fb] : base[fb] ^ (uint32_t)(nb8 << 5);
+            short4_t t4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)addr);
             half4_t h4 = __builtin_bit_cast(half4_t, t4);
             dst[fb * 4 + 0] = h4[0];
             dst[fb * 4 + 1] = h4[1];
@@ -215,14 +220,14 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
         };
 #pragma unroll
         for (int k = 0; k < 2; k++) {
-            addresses(k);
+            if (GROUPED) addresses(k);
 #pragma unroll
-            for (int fb = 0; fb < 4; fb++) read_part(bf[k], fb);
+            for (int fb = 0; fb < 4; fb++) read_part(bf[k], k, fb);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int nb8 = 0; nb8 < 8; nb8++) {
-            if (nb8 + 2 < 8) addresses(nb8 + 2);
+            if (GROUPED && nb8 + 2 < 8) addresses(nb8 + 2);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int mb = 0; mb < 4; mb++) {
@@ -230,7 +235,7 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
                 if (mb & 1) c = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[mb], bf[nb8 % 3], c, (int)ix[mb >> 1], 0, 1);
                 else c = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[mb], bf[nb8 % 3], c, (int)ix[mb >> 1], 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                if (nb8 + 2 < 8) read_part(bf[(nb8 + 2) % 3], mb);
+                if (nb8 + 2 < 8) read_part(bf[(nb8 + 2) % 3], nb8 + 2, mb);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -300,7 +305,7 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
 #undef SPATHA_UP_WAIT_ALL
 }
 
-template <int OUT_LAYOUT, bool FUSE>
+template <int OUT_LAYOUT, bool FUSE, bool GROUPED>
 __global__ __launch_bounds__(512) void spmm_up_kernel(SpmmParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
@@ -309,16 +314,16 @@ __global__ __launch_bounds__(512) void spmm_up_kernel(SpmmParams p) {
     TileWalk walk;
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
-    if (wave >= 4) up_wave<OUT_LAYOUT, FUSE, true>(p, walk, smem, smem_base, wave, lane);
-    else up_wave<OUT_LAYOUT, FUSE, false>(p, walk, smem, smem_base, wave, lane);
+    if (wave >= 4) up_wave<OUT_LAYOUT, FUSE, GROUPED, true>(p, walk, smem, smem_base, wave, lane);
+    else up_wave<OUT_LAYOUT, FUSE, GROUPED, false>(p, walk, smem, smem_base, wave, lane);
 }
 
-template <int OUT_LAYOUT, bool FUSE>
+template <int OUT_LAYOUT, bool FUSE, bool GROUPED>
 static hipError_t launch_up(const SpmmParams& p, hipStream_t stream) {
     constexpr int lds = UpCfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static int cus = 0;
-    void (*kern)(SpmmParams) = spmm_up_kernel<OUT_LAYOUT, FUSE>;
+    void (*kern)(SpmmParams) = spmm_up_kernel<OUT_LAYOUT, FUSE, GROUPED>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         // the kernel's register loads complete asynchronously into named variables: an instantiation that keeps
@@ -345,12 +350,14 @@ static hipError_t launch_up(const SpmmParams& p, hipStream_t stream) {
 
 hipError_t launch_pingpong(int variant, int out_layout, const SpmmParams& p, hipStream_t stream) {
     if (variant != SPMM_VARIANT_UP512x128_S3) return hipErrorInvalidValue;
-    // (the plain instantiations carry nothing of the fused write-out)
-    if (p.fuse)
-        return out_layout == SPATHA_OUT_TRANSPOSED ? launch_up<SPATHA_OUT_TRANSPOSED, true>(p, stream)
-                                                   : launch_up<SPATHA_OUT_ROW_MAJOR, true>(p, stream);
-    return out_layout == SPATHA_OUT_TRANSPOSED ? launch_up<SPATHA_OUT_TRANSPOSED, false>(p, stream)
-                                               : launch_up<SPATHA_OUT_ROW_MAJOR, false>(p, stream);
+    // (the plain instantiations carry nothing of the fused write-out; the form of the matrix phase follows m, see there)
+    const bool t = out_layout == SPATHA_OUT_TRANSPOSED, grouped = p.m <= 5;
+    if (p.fuse) {
+        if (grouped) return t ? launch_up<SPATHA_OUT_TRANSPOSED, true, true>(p, stream) : launch_up<SPATHA_OUT_ROW_MAJOR, true, true>(p, stream);
+        return t ? launch_up<SPATHA_OUT_TRANSPOSED, true, false>(p, stream) : launch_up<SPATHA_OUT_ROW_MAJOR, true, false>(p, stream);
+    }
+    if (grouped) return t ? launch_up<SPATHA_OUT_TRANSPOSED, false, true>(p, stream) : launch_up<SPATHA_OUT_ROW_MAJOR, false, true>(p, stream);
+    return t ? launch_up<SPATHA_OUT_TRANSPOSED, false, false>(p, stream) : launch_up<SPATHA_OUT_ROW_MAJOR, false, false>(p, stream);
 }
 
 }  // namespace spatha

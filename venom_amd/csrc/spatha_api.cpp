@@ -83,152 +83,156 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = f
     return true;
 }
 
-// Kernel choice.  V a multiple of 128: producer/consumer kernel on 128-row tiles; 256 columns wide
-// with 128 x 64 consumer waves when that still gives every CU at least two tiles, else 128 wide.  Otherwise (V a
-// multiple of 64 only) the 64 x 256 tile whose B rows are gathered per 64-row block.
-int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = false, int out_layout = SPATHA_OUT_ROW_MAJOR) {
-    using namespace spatha;
-    if (variant != SPMM_VARIANT_AUTO) return variant_ok(plan, N, variant, fused) ? variant : -1;
-    const int v = plan->geo.v;
-    int order[4] = {0, 0, 0, 0};
+// ---- Kernel choice ----------------------------------------------------------------------------------------------
+// The automatic choice is a list of rules read top-down: the first rule whose class and condition hold for the shape
+// and whose kernel accepts the plan (variant_ok) names the kernel.  The conditions are measured crossover points on
+// MI355X (BERT-base / BERT-large / GPT-2-large / GPT-3 layer shapes, N = 2048 .. 16384, m = 4 .. 100); each rule's comment
+// says what was measured.  Later rules double as the fall-backs of earlier ones.
+struct Shape {
+    int v, m, rows, N, S;
+    int64_t cus;
+    bool fused, transposed;
+    // tiles of bm x bn in the output (whole row tiles only: the kernels that take a partial row tile are never chosen by count)
+    int64_t tiles(int bm, int bn) const { return (int64_t)(rows / bm) * ((N + bn - 1) / bn); }
+    // the last of `tiles` tiles' rounds over the CUs is at least 90 % full (a single round: 75 %)
+    bool whole_rounds(int64_t t) const {
+        const int64_t rounds = (t + cus - 1) / cus;
+        return rounds == 1 ? t * 4 >= cus * 3 : t * 10 >= rounds * cus * 9;
+    }
+    // 128 x 256 tiles ahead of 128 x 128 ones: from 1024 tiles on, from 768 with two or more k-steps, from 512 with eight or
+    // more, from 192 with a dozen or more (every kernel on the BERT layer shapes x N = 2048 .. 8192 x 2:10 .. 2:100;
+    // 1024 x 1024 x 16384 at 128:2:16, 512 wide tiles of 4 k-steps, runs 19 % faster on 128 x 128 tiles)
+    bool wide() const {
+        const int64_t t = tiles(128, 256);
+        return t >= 1024 || (t >= 768 && S >= 2) || (t >= 512 && S >= 8) || (t >= 192 && S >= 12);
+    }
+    // 64 x 256 tiles with long k-loops and either many rounds or at most one
+    bool long_k() const { const int64_t t = tiles(64, 256); return S >= 32 && (t >= 2048 || t <= 256); }
+    // 64 x 256 tiles: many tiles of few k-steps, m >= 32, row-major
+    bool short_k_many() const { return m >= 32 && !transposed && tiles(64, 256) >= 2048 && S <= 8; }
+};
+
+enum : unsigned { V_HALF = 1u, V_128 = 2u, V_64 = 4u };       // V % 64 != 0 / V % 128 == 0 / V % 64 == 0 only
+
+struct Rule {
+    unsigned v_classes;
+    int variant;
+    bool (*when)(const Shape&);
+};
+
+const Rule kRules[] = {
     // few columns: streaming A is all that matters, one 64-row tile per workgroup with the k-steps split over its waves
     // (N = 32: equal on the GPT-3 FFN matrix, 1.3-1.5x ahead on the BERT-large ones; N = 48, 64: behind the 128-wide tiles)
-    if (N <= 32 && variant_ok(plan, N, SPMM_VARIANT_SKINNY, fused)) return SPMM_VARIANT_SKINNY;
-    if (plan->half_tiles) {
-        // measured (1024 x 4096 x 4096 and 4096 x 1024 x 16384, m = 8..32): the 256-wide tile is never behind the
-        // 128-wide one with two stages by more than 7 %, and up to 2x ahead; three stages of 128 leave two waves per CU
-        // m <= 8: the dense B stage is shared by eight 32-row blocks, the fill does not grow with the smaller V
-        order[0] = SPMM_VARIANT_DSH256x128_S3_C8;
-        order[1] = N > 128 ? SPMM_VARIANT_H64x256_S2 : SPMM_VARIANT_H64x128_S2;
-        order[2] = SPMM_VARIANT_H64x128_S2;
-        order[3] = SPMM_VARIANT_H64x128_S3;
-        for (int i = 0; i < 4; i++)
-            if (variant_ok(plan, N, order[i], fused)) return order[i];
-        return -1;
-    }
-    // Dense-staged 256 x 128 tiles: with at most 768 of them the two-phase-group form leads the eight-consumer form by
-    // 2-5 % (BERT-base / BERT-large layer shapes at N = 2048 .. 8192), beyond that it falls behind; it has no fused
-    // write-out and is measured for row-major output only.
-    const int64_t ds_tiles = (int64_t)(plan->geo.rows / 256) * ((N + 127) / 128);
-    // (not for long k-loops: 12288 x 12288 x 2048 at 64:2:8, 96 k-steps, 255 us against 239 us)
-    const int ds_variant = (ds_tiles <= 768 && plan->S <= 32 && !fused && out_layout == SPATHA_OUT_ROW_MAJOR &&
-                            variant_ok(plan, N, SPMM_VARIANT_DS256x128_S3_PP, fused))
-                               ? SPMM_VARIANT_DS256x128_S3_PP
-                               : SPMM_VARIANT_DS256x128_S3_C8;
-    if (v % 128 == 0) {
-        const int64_t wide_tiles = (int64_t)(plan->geo.rows / 128) * ((N + 255) / 256);
-        // 128 x 256 tiles once there is work for two rounds of them, or for four with few k-steps per tile (measured on
-        // the BERT-large layer shapes, N = 16384: 1024 x 1024 at 128:2:16, 512 wide tiles of 4 k-steps, runs 19 % faster on
-        // 128 x 128 tiles; 1024 x 4096, 512 tiles of 16 k-steps, 3 % slower).  m >= 16: the producer/consumer kernel with
-        // 64 x 64 consumer blocks leads the tall-consumer form by 1-13 % up to 16 k-steps per tile (BERT-large, GPT-2-large
-        // layers) and trails it by 1-3 % on long k-loops (GPT-3 layers).
-        // (every kernel id on the BERT layer shapes x N = 2048 .. 8192 x 2:10 .. 2:100: the 256-wide tile leads from 1024 tiles on,
-        // from 768 with two or more k-steps, from 512 with eight or more, and from 192 with a dozen or more)
-        const bool wide = wide_tiles >= 1024 || (wide_tiles >= 768 && plan->S >= 2) || (wide_tiles >= 512 && plan->S >= 8) ||
-                          (wide_tiles >= 192 && plan->S >= 12);
-        const bool ws_wide = plan->geo.m >= 16 && plan->S <= 16 && wide_tiles >= 768;    // (fewer tiles: the tall form, 8-10 % ahead)
-        if (wide) {
-            order[0] = ws_wide ? SPMM_VARIANT_W128x256_S3 : SPMM_VARIANT_T128x256_S3;
-            order[1] = ws_wide ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x256_S3;
-            order[2] = SPMM_VARIANT_W128x128_S3;
-        } else {
-            order[0] = SPMM_VARIANT_W128x128_S3;
-            order[1] = SPMM_VARIANT_P128x128_S3;
-            // more than one round of 128 x 128 tiles but at most two, few k-steps: the same number of 64 x 256 tiles runs as
-            // one round of two co-resident workgroups per CU (768 x 768 x 8192, 3072 x 768 x 2048, 1024 x 1024 x 8192,
-            // 4096 x 1024 x 2048 at 128:2:10 .. 128:2:100: 5-30 % ahead)
-            const int64_t tiles128 = (int64_t)(plan->geo.rows / 128) * ((N + 127) / 128);
-            const int64_t cus = plan->cus > 0 ? plan->cus : 256;
-            if (plan->geo.m > 8 && tiles128 > cus && tiles128 <= 2 * cus && plan->S <= 8 && out_layout == SPATHA_OUT_ROW_MAJOR) {
-                order[1] = order[0];
-                order[0] = SPMM_VARIANT_P64x256_S2;
-            }
-        }
-        // m <= 8: dense staging leads the gathered tiles by 5-35 % as soon as its 256 x 128 tiles fill three quarters of
-        // the CUs (BERT layer shapes, N = 2048 .. 16384; from 160 tiles on the GPT-2-large ones); with fewer tiles the 128 x 128
-        // tile's finer split wins
-        if (plan->geo.m <= 8 && plan->geo.rows % 256 == 0 && ds_tiles >= 160 && plan->S <= 64 &&
-            out_layout == SPATHA_OUT_ROW_MAJOR) {
-            order[1] = order[0];
-            order[0] = ds_variant;
-        }
-        if (out_layout == SPATHA_OUT_TRANSPOSED) {
-            // measured with transposed output + bias on the BERT-large layer shapes (N = 16384): the kernels that write
-            // through the 8-column slab (dense-staged, tall) lead by 10-25 % once there is enough work per tile column
-            if (plan->geo.m <= 8) {
-                // not for long k-loops: with many k-steps per tile the gathered 128 x 256 tile moves fewer bytes per
-                // output element (GPT-3 block at 128:2:8, 96 k-steps: 6.95 ms against 8.26 ms with dense staging; GPT-2-large
-                // FFN-down, 40 k-steps: dense staging 20 % ahead)
-                if (plan->S <= 40) {
-                    order[1] = order[0];
-                    order[0] = SPMM_VARIANT_DS256x128_S3_C8;
-                }
-            } else {
-                // m >= 16: 128 x 256 tiles at any tile count (5-15 % ahead of 128 x 128 on the BERT-large and GPT-2-large
-                // layer shapes, N = 4096 and 16384)
-                const bool ws_wide_t = plan->geo.m >= 16 && plan->S <= 16;
-                order[0] = ws_wide_t ? SPMM_VARIANT_W128x256_S3 : SPMM_VARIANT_T128x256_S3;
-                order[1] = ws_wide_t ? SPMM_VARIANT_T128x256_S3 : SPMM_VARIANT_W128x256_S3;
-                order[2] = SPMM_VARIANT_W128x128_S3;
-            }
-        }
-        if (order[2] == 0) order[2] = SPMM_VARIANT_P128x128_S3;
-        order[3] = SPMM_VARIANT_128x128;
-    } else if (v % 64 == 0) {
-        // m <= 8: staging the dense B rows once for four 64-row blocks halves the L2 -> LDS traffic
-        order[0] = ds_variant;
-        // m > 8: gathered 64 x 256 tiles.  Per-tile pipeline with two stages (two workgroups per CU) unless there is
-        // work for many rounds: then, with 32 or more k-steps per tile, the persistent pipeline (which keeps loading
-        // across tile boundaries) leads (GPT-3 layers at 64:2:16; at 64:2:32, 24 k-steps, the per-tile pipeline is
-        // 10-20 % ahead), and for m >= 32 with few k-steps and row-major output the producer/consumer kernel leads by
-        // 5-10 % (transposed: the pipeline leads by 6-8 %).  With one tile per CU or less the persistent kernel's third
-        // stage still gives long k-loops 5-15 %.
-        const int64_t tiles = (int64_t)(plan->geo.rows / 64) * ((N + 255) / 256);
-        const bool long_k = plan->S >= 32 && (tiles >= 2048 || tiles <= 256);
-        const bool ws_short = plan->geo.m >= 32 && out_layout != SPATHA_OUT_TRANSPOSED && tiles >= 2048 && plan->S <= 8;
-        // at most one tile per CU with a dozen or more k-steps: producer/consumer kernel (768 x 3072 / 1024 x 4096 x 4096 at 64:2:10
-        // and 64:2:20: 10-17 % ahead of the per-tile pipeline)
-        const int64_t cus64 = plan->cus > 0 ? plan->cus : 256;
-        const bool ws_one_round = !long_k && tiles <= cus64 && plan->S >= 12 && out_layout == SPATHA_OUT_ROW_MAJOR;
-        order[1] = long_k ? SPMM_VARIANT_R64x256_S3 : ((ws_short || ws_one_round) ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_P64x256_S2);
-        // 16 <= m < 32, many tiles, few k-steps, plain row-major output: the producer/consumer kernel with the write-out
-        // deferred into the next tile's steps leads the pipeline by 5-8 % (3072 / 4096 x 1024 x 16384 at 64:2:16)
-        if (!long_k && !ws_short && !fused && out_layout == SPATHA_OUT_ROW_MAJOR && plan->geo.m >= 16 && tiles >= 3072 &&
-            plan->S <= 8 && variant_ok(plan, N, SPMM_VARIANT_D64x256_S3, fused))
-            order[1] = SPMM_VARIANT_D64x256_S3;
-        order[2] = long_k ? SPMM_VARIANT_W64x256_S3 : SPMM_VARIANT_R64x256_S3;
-        order[3] = SPMM_VARIANT_64x256;
-    } else {
-        return -1;
-    }
-    // Unified 512 x 128 kernel (m <= 8, rows % 512 == 0, no fused write-out): 3-13 % ahead of the producer/consumer forms
-    // of the dense-staged kernel when its tiles fill whole rounds of the CUs (BERT-large layer shapes at N = 16384,
-    // V = 64 and 128, m = 8 and 4: 256, 768, 1024 tiles), 10-20 % behind at 320 or 384 tiles (1.25 / 1.5 rounds) and up to
-    // 2x behind with fewer tiles than CUs; transposed output with 256 tiles of 8 k-steps measures 2-3 % behind.
-    if (plan->geo.m <= 8 && variant_ok(plan, N, SPMM_VARIANT_UP512x128_S3, fused)) {
-        const int64_t du_tiles = (int64_t)(plan->geo.rows / 512) * ((N + 127) / 128);
-        const int64_t cus = plan->cus > 0 ? plan->cus : 256;
-        const int64_t rounds = (du_tiles + cus - 1) / cus;
-        // (a single round three quarters full is enough: 3072 x 768 x 4096, 192 tiles, 10-12 % ahead of the 256 x 128 tiles)
-        const bool whole_rounds = rounds == 1 ? du_tiles * 4 >= cus * 3 : du_tiles * 10 >= rounds * cus * 9;
-        const bool layout_ok = out_layout == SPATHA_OUT_ROW_MAJOR || du_tiles >= 2 * cus || plan->S >= 16;
-        // (the form in two phase groups leads the one-group form by 3-8 % on every shape of that sweep)
-        if (whole_rounds && layout_ok) return SPMM_VARIANT_UP512x128_S3;
-    }
-    // Its form for 8 < m <= 16 (64 KB stages, two of them): V a multiple of 64 only - 7-26 % ahead of the gathered
-    // 64 x 256 tiles on the BERT-large layer shapes at N = 16384 (64:2:16 and 64:2:10, both layouts); with V % 128 == 0
-    // the gathered 128 x 256 tiles share their B rows over 128 rows and are equal or up to 15 % ahead.
-    if (plan->geo.m > 8 && plan->geo.v % 128 != 0 && variant_ok(plan, N, SPMM_VARIANT_DU512x128_M16, fused)) {
-        const int64_t du_tiles = (int64_t)(plan->geo.rows / 512) * ((N + 127) / 128);
-        const int64_t cus = plan->cus > 0 ? plan->cus : 256;
-        const int64_t rounds = (du_tiles + cus - 1) / cus;
-        // long k-loops (GPT-3 projections at 64:2:16, 48 k-steps and more): ahead of every gathered form at 1.5 rounds too
-        // (12288 x 12288 x 2048: 177 us against 188 us for the best of them and 262 us for the per-tile pipeline)
-        const bool whole_rounds = rounds == 1 ? du_tiles * 4 >= cus * 3 : du_tiles * 10 >= rounds * cus * 9;
-        if (whole_rounds || (du_tiles >= cus && plan->S >= 32)) return SPMM_VARIANT_DU512x128_M16;
-    }
-    for (int i = 0; i < 4; i++)
-        if (variant_ok(plan, N, order[i], fused)) return order[i];
+    {V_HALF | V_128 | V_64, spatha::SPMM_VARIANT_SKINNY, [](const Shape& s) { return s.N <= 32; }},
+
+    // -- V % 64 != 0 (1024 x 4096 x 4096 and 4096 x 1024 x 16384, m = 8 .. 32) --
+    // m <= 8: the dense B stage is shared by eight 32-row blocks, the fill does not grow with the smaller V
+    {V_HALF, spatha::SPMM_VARIANT_DSH256x128_S3_C8, [](const Shape&) { return true; }},
+    // the 256-wide tile is never behind the 128-wide one with two stages by more than 7 %, and up to 2x ahead
+    {V_HALF, spatha::SPMM_VARIANT_H64x256_S2, [](const Shape& s) { return s.N > 128; }},
+    // (three stages of 128 leave two waves per CU)
+    {V_HALF, spatha::SPMM_VARIANT_H64x128_S2, [](const Shape&) { return true; }},
+    {V_HALF, spatha::SPMM_VARIANT_H64x128_S3, [](const Shape&) { return true; }},
+
+    // -- unified 512 x 128 tiles --
+    // m <= 8, two phase groups: 3-13 % ahead of the dense-staged 256 x 128 tiles when its tiles fill whole rounds of the CUs
+    // (BERT-large layer shapes at N = 16384, V = 64 and 128, m = 8 and 4: 256, 768, 1024 tiles; 3072 x 768 x 4096, 192
+    // tiles: 10-12 % ahead), 10-20 % behind at 320 or 384 tiles and up to 2x behind with fewer tiles than CUs;
+    // transposed output with 256 tiles of 8 k-steps measures 2-3 % behind
+    {V_128 | V_64, spatha::SPMM_VARIANT_UP512x128_S3,
+     [](const Shape& s) {
+         const int64_t t = s.tiles(512, 128);
+         return s.m <= 8 && s.whole_rounds(t) && (!s.transposed || t >= 2 * s.cus || s.S >= 16);
+     }},
+    // 8 < m <= 16, one phase group with two 64 KB stages: 7-26 % ahead of the gathered 64 x 256 tiles on the BERT-large
+    // layer shapes at N = 16384 (64:2:16 and 64:2:10, both layouts); on long k-loops ahead at 1.5 rounds too (12288 x 12288
+    // x 2048 at 64:2:16: 177 us against 188 us for the best gathered form).  With V % 128 == 0 the gathered 128 x 256
+    // tiles share their B rows over 128 rows and are equal or up to 15 % ahead.
+    {V_64, spatha::SPMM_VARIANT_DU512x128_M16,
+     [](const Shape& s) {
+         const int64_t t = s.tiles(512, 128);
+         return s.m > 8 && (s.whole_rounds(t) || (t >= s.cus && s.S >= 32));
+     }},
+
+    // -- V % 128 == 0 --
+    // transposed output, m <= 8: the kernels that write through the 8-column slab lead by 10-25 % (BERT-large layer shapes,
+    // N = 16384, with bias); not on long k-loops, where the gathered 128 x 256 tile moves fewer bytes per output element
+    // (GPT-3 block at 128:2:8, 96 k-steps: 6.95 ms against 8.26 ms; GPT-2-large FFN-down, 40 k-steps: dense staging 20 % ahead)
+    {V_128, spatha::SPMM_VARIANT_DS256x128_S3_C8, [](const Shape& s) { return s.transposed && s.m <= 8 && s.S <= 40; }},
+    // row-major, m <= 8: dense staging leads the gathered tiles by 5-35 % as soon as its 256 x 128 tiles fill three quarters
+    // of the CUs (BERT layer shapes, N = 2048 .. 16384; from 160 tiles on the GPT-2-large ones).  Up to 768 tiles the form in
+    // two phase groups leads the eight-consumer form by 2-5 %; it has no fused write-out, and falls behind on long k-loops
+    // (12288 x 12288 x 2048 at 64:2:8, 96 k-steps: 255 us against 239 us)
+    {V_128, spatha::SPMM_VARIANT_DS256x128_S3_PP,
+     [](const Shape& s) {
+         const int64_t t = s.tiles(256, 128);
+         return !s.transposed && !s.fused && s.m <= 8 && s.rows % 256 == 0 && t >= 160 && t <= 768 && s.S <= 32;
+     }},
+    {V_128, spatha::SPMM_VARIANT_DS256x128_S3_C8,
+     [](const Shape& s) { return !s.transposed && s.m <= 8 && s.rows % 256 == 0 && s.tiles(256, 128) >= 160 && s.S <= 64; }},
+    // transposed output, m > 8: 128 x 256 tiles at any tile count (5-15 % ahead of 128 x 128 on the BERT-large and
+    // GPT-2-large layer shapes, N = 4096 and 16384); 64 x 64 consumer blocks up to 16 k-steps, else the tall consumers
+    {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.m >= 16 && s.S <= 16; }},
+    {V_128, spatha::SPMM_VARIANT_T128x256_S3, [](const Shape& s) { return s.transposed && s.m > 8; }},
+    {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.m > 8; }},
+    // 128 x 256 tiles, m >= 16: the 64 x 64 consumer blocks lead the tall-consumer form by 1-13 % up to 16 k-steps per tile
+    // (BERT-large, GPT-2-large layers) from 768 tiles on (fewer: the tall form is 8-10 % ahead) and trail it by 1-3 % on
+    // long k-loops (GPT-3 layers)
+    {V_128, spatha::SPMM_VARIANT_W128x256_S3,
+     [](const Shape& s) { return s.wide() && s.m >= 16 && s.S <= 16 && s.tiles(128, 256) >= 768; }},
+    {V_128, spatha::SPMM_VARIANT_T128x256_S3, [](const Shape& s) { return s.wide(); }},
+    {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.wide(); }},
+    // more than one round of 128 x 128 tiles but at most two, few k-steps: the same number of 64 x 256 tiles runs as one
+    // round of two co-resident workgroups per CU (768 x 768 x 8192, 3072 x 768 x 2048, 1024 x 1024 x 8192, 4096 x 1024 x
+    // 2048 at 128:2:10 .. 128:2:100: 5-30 % ahead)
+    {V_128, spatha::SPMM_VARIANT_P64x256_S2,
+     [](const Shape& s) {
+         const int64_t t = s.tiles(128, 128);
+         return !s.transposed && s.m > 8 && t > s.cus && t <= 2 * s.cus && s.S <= 8;
+     }},
+    {V_128, spatha::SPMM_VARIANT_W128x128_S3, [](const Shape&) { return true; }},
+    {V_128, spatha::SPMM_VARIANT_P128x128_S3, [](const Shape&) { return true; }},
+    {V_128, spatha::SPMM_VARIANT_128x128, [](const Shape&) { return true; }},
+
+    // -- V a multiple of 64 only --
+    // m <= 8: staging the dense B rows once for four 64-row blocks halves the L2 -> LDS traffic; the two forms as above
+    {V_64, spatha::SPMM_VARIANT_DS256x128_S3_PP,
+     [](const Shape& s) { return !s.transposed && !s.fused && s.tiles(256, 128) <= 768 && s.S <= 32; }},
+    {V_64, spatha::SPMM_VARIANT_DS256x128_S3_C8, [](const Shape&) { return true; }},
+    // m > 8, gathered 64 x 256 tiles.  32 or more k-steps per tile and many rounds: the persistent pipeline, which keeps
+    // loading across tile boundaries, leads (GPT-3 layers at 64:2:16; at 64:2:32, 24 k-steps, the per-tile pipeline is
+    // 10-20 % ahead); with one tile per CU or less its third stage still gives long k-loops 5-15 %
+    {V_64, spatha::SPMM_VARIANT_R64x256_S3, [](const Shape& s) { return s.long_k(); }},
+    {V_64, spatha::SPMM_VARIANT_W64x256_S3, [](const Shape& s) { return s.long_k(); }},
+    // 16 <= m, 3072 tiles or more of few k-steps, plain row-major output: the producer/consumer kernel with the write-out
+    // deferred into the next tile's steps leads the pipeline by 5-8 % (3072 / 4096 x 1024 x 16384 at 64:2:16)
+    {V_64, spatha::SPMM_VARIANT_D64x256_S3,
+     [](const Shape& s) {
+         return !s.long_k() && !s.short_k_many() && !s.fused && !s.transposed && s.m >= 16 && s.tiles(64, 256) >= 3072 && s.S <= 8;
+     }},
+    // producer/consumer kernel: m >= 32 with many tiles of few k-steps, row-major, 5-10 % ahead (transposed: the pipeline
+    // leads by 6-8 %); at most one tile per CU with a dozen or more k-steps, 10-17 % ahead of the per-tile pipeline
+    // (768 x 3072 / 1024 x 4096 x 4096 at 64:2:10 and 64:2:20)
+    {V_64, spatha::SPMM_VARIANT_W64x256_S3,
+     [](const Shape& s) {
+         return !s.long_k() && (s.short_k_many() || (!s.transposed && s.tiles(64, 256) <= s.cus && s.S >= 12));
+     }},
+    // else the per-tile pipeline with two stages (two workgroups per CU)
+    {V_64, spatha::SPMM_VARIANT_P64x256_S2, [](const Shape& s) { return !s.long_k(); }},
+    {V_64, spatha::SPMM_VARIANT_R64x256_S3, [](const Shape&) { return true; }},
+    {V_64, spatha::SPMM_VARIANT_64x256, [](const Shape&) { return true; }},
+};
+
+int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = false, int out_layout = SPATHA_OUT_ROW_MAJOR) {
+    if (variant != spatha::SPMM_VARIANT_AUTO) return variant_ok(plan, N, variant, fused) ? variant : -1;
+    Shape s;
+    s.v = plan->geo.v; s.m = plan->geo.m; s.rows = plan->geo.rows; s.N = N; s.S = plan->S;
+    s.cus = plan->cus > 0 ? plan->cus : 256;
+    s.fused = fused;
+    s.transposed = out_layout == SPATHA_OUT_TRANSPOSED;
+    const unsigned v_class = plan->half_tiles ? V_HALF : s.v % 128 == 0 ? V_128 : s.v % 64 == 0 ? V_64 : 0u;
+    for (const Rule& r : kRules)
+        if ((r.v_classes & v_class) && r.when(s) && variant_ok(plan, N, r.variant, fused)) return r.variant;
     return -1;
 }
 }  // namespace

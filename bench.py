@@ -7,12 +7,17 @@ One step = one SpMM  C[4096 x 16384] = A_vnm[4096 x 1024] * B[1024 x 16384]  (fp
 fp32 accumulation, fp16 result) with every operand already resident in HBM.  Prints ONE JSON
 line: dense-equivalent TFLOPS (2*M*K*N / t), microseconds per SpMM, the roofline of the SpMM
 kernel (HBM bound for this shape) and the CPU baseline (the CPU oracle's SpMM on a bounded
-sample of the same workload, timed on this host's cores)."""
+sample of the same workload, timed on this host's cores) and, where `amd-smi` answers, the socket power and graphics clock
+under a sustained run of the same launches (`power`): on MI355X this kernel runs at the socket's power limit, which is what
+sets its clock."""
 import argparse
 import ctypes
 import json
 import os
+import re
+import subprocess
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -37,6 +42,61 @@ MEASURED_TRAFFIC = {
     ("smfmac16x16x64_warpspec_tall_tile128x256_3stage", 49152, 12288, 2048, 16, 128):
         (2_202_100_000, "profiles/spmm_wst_kernel_tile128x256_gpt3_ffn_n2048.md"),
 }
+
+
+def smi_sample():
+    """(socket power in W, mean graphics clock over the XCDs in MHz) from `amd-smi metric --power --clock --json`, or None."""
+    try:
+        r = subprocess.run(["amd-smi", "metric", "--power", "--clock", "--json"], capture_output=True, text=True, timeout=10)
+    except (OSError, subprocess.SubprocessError):
+        return None
+    watts = re.search(r'"socket_power": \{\s*"value": (\d+)', r.stdout)
+    clocks = re.findall(r'"gfx_\d+": \{\s*"clk": \{\s*"value": (\d+)', r.stdout)
+    if r.returncode != 0 or not watts or not clocks:
+        return None
+    return int(watts.group(1)), sum(map(int, clocks)) / len(clocks)
+
+
+def under_profiler():
+    """A profiler's preloaded library would load into the sampling tool as well: no power sampling under one."""
+    return "rocprof" in os.environ.get("LD_PRELOAD", "") or any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ)
+
+
+def sustained(launch, sync, us_estimate, seconds):
+    """Back-to-back launches for `seconds` (after a quarter of that to settle) with `amd-smi` sampled from a second thread;
+    returns (microseconds per launch by wall clock, mean socket W, mean gfx MHz, samples used) - power and clock None if
+    the tool does not answer."""
+    chunk = max(1, int(20e3 / max(us_estimate, 1.0)))          # synchronize every ~20 ms of queued work
+    t_end = time.perf_counter() + seconds / 4
+    while time.perf_counter() < t_end:
+        for _ in range(chunk):
+            launch()
+        sync()
+    samples, stop = [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            got = smi_sample()
+            if got is None:
+                return
+            samples.append((time.perf_counter(),) + got)
+            stop.wait(0.15)
+
+    th = threading.Thread(target=sampler)
+    th.start()
+    n, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(chunk):
+            launch()
+        sync()
+        n += chunk
+    t1 = time.perf_counter()
+    stop.set()
+    th.join()
+    used = [x for x in samples if t0 + min(0.8, seconds / 3) < x[0] < t1]      # the tool's reading lags by a few 100 ms
+    if not used:
+        return (t1 - t0) * 1e6 / n, None, None, 0
+    return (t1 - t0) * 1e6 / n, sum(x[1] for x in used) / len(used), sum(x[2] for x in used) / len(used), len(used)
 
 
 def algorithmic_bytes(rows, cols, N, m, v, ksp):
@@ -71,6 +131,13 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="before the benchmark, run 5 plain device copies of 256 MiB (a kernel of known HBM traffic, "
                          "for scaling the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
+    ap.add_argument("--no-power", action="store_true",
+                    help="skip the sustained run with `amd-smi` power / clock sampling that follows the timed region ('power')")
+    ap.add_argument("--power-seconds", type=float, default=2.0, help="length of that sustained run")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run the machine calibration kernels (venom_amd/csrc/calibrate.hip) under the same sampling: a "
+                         "write of C alone, and sparse matrix instructions alone on Gaussian / small-integer / zero operands "
+                         "('calibration')")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the SpMM path has no multi-GPU part); run with --gpus 1",
@@ -89,6 +156,8 @@ def main():
                                env=dict(os.environ, SPATHA_LIBRARY=alt), stdout=subprocess.PIPE, text=True)
             if r.returncode == 0 and r.stdout.strip():
                 out32 = json.loads(r.stdout.strip().splitlines()[-1])["roofline"]["kernel_us"]
+
+    idle = None if args.no_power or under_profiler() else smi_sample()
 
     import numpy as np
     import torch
@@ -182,6 +251,74 @@ def main():
                      "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes": nbytes, "kernel_us": round(ms_kernel * 1e3, 3)},
     }
+
+    if idle is not None:
+        # Sustained run of the same launches with the socket power and graphics clock sampled beside it.  (The idle
+        # reading was taken before this process touched the GPU.)
+        stream = torch.cuda.current_stream(dev)
+        sp = ctypes.c_void_p(stream.cuda_stream)
+        plan, B, C = w["plan"], w["B"], w["C"]
+        us_s, watts, mhz, n_s = sustained(
+            lambda: _lib.check(L.spatha_spmm_run(plan._handle, B.data_ptr(), N, None, C.data_ptr(), 0, args.variant, sp), "run"),
+            torch.cuda.synchronize, ms_kernel * 1e3, args.power_seconds)
+        out["power"] = {"socket_w": None if watts is None else round(watts, 1), "gfx_mhz": None if mhz is None else round(mhz, 1),
+                        "idle_socket_w": idle[0], "us_per_spmm_sustained": round(us_s, 3),
+                        "mj_per_spmm": None if watts is None else round(watts * us_s * 1e-3, 2), "samples": n_s,
+                        "source": "amd-smi metric --power --clock, sampled over %.1f s of back-to-back launches after the timed "
+                                  "region" % args.power_seconds}
+    else:
+        out["power"] = None
+
+    if args.calibrate:
+        cal = ctypes.CDLL(os.path.join(ROOT, "venom_amd", "lib", "libspatha_calibrate.so"))
+        cal.spatha_calibrate_store.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+        cal.spatha_calibrate_smfmac.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                                ctypes.c_void_p]
+        stream = torch.cuda.current_stream(dev)
+        sp = ctypes.c_void_p(stream.cuda_stream)
+        wgs = torch.cuda.get_device_properties(dev).multi_processor_count
+        calib = {}
+
+        def run_cal(name, launch, us_guess, describe):
+            us_c, watts, mhz, n_c = sustained(launch, torch.cuda.synchronize, us_guess, args.power_seconds)
+            calib[name] = dict(describe(us_c), us=round(us_c, 2), socket_w=None if watts is None else round(watts, 1),
+                               gfx_mhz=None if mhz is None else round(mhz, 1), samples=n_c)
+
+        def check_hip(rc):
+            if rc != 0:
+                raise RuntimeError("calibration kernel: HIP error %d" % rc)
+
+        c_rows, c_n = (rows // 512) * 512, (N // 128) * 128
+        if c_rows and c_n:
+            Cc = torch.empty((c_rows, c_n), dtype=torch.float16, device=dev)
+            seed = [0]
+
+            def launch_store():
+                seed[0] += 1
+                check_hip(cal.spatha_calibrate_store(Cc.data_ptr(), c_rows, c_n, wgs, seed[0], sp))
+
+            run_cal("store_c_alone", launch_store, 20.0,
+                    lambda us_c: {"bytes": 2 * c_rows * c_n, "tb_per_s": round(2 * c_rows * c_n / us_c * 1e-6, 2)})
+            del Cc
+        threads, passes = wgs * 512, 100
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(1)
+        out_c = torch.empty(threads, dtype=torch.float32, device=dev)
+        operand_sets = {
+            "smfmac_alone_gaussian": (torch.randn(threads * 32, generator=gen, device=dev) * 0.02,
+                                      torch.randn(threads * 128, generator=gen, device=dev)),
+            "smfmac_alone_integers": (torch.randint(-4, 5, (threads * 32,), generator=gen, device=dev).float(),
+                                      torch.randint(-4, 5, (threads * 128,), generator=gen, device=dev).float()),
+            "smfmac_alone_zeros": (torch.zeros(threads * 32, device=dev), torch.zeros(threads * 128, device=dev)),
+        }
+        for name, (a32, b32) in operand_sets.items():
+            a16, b16 = a32.to(torch.float16), b32.to(torch.float16)
+            n_inst = wgs * 8 * passes * 32
+            run_cal(name, lambda: check_hip(cal.spatha_calibrate_smfmac(a16.data_ptr(), b16.data_ptr(), out_c.data_ptr(), wgs, passes, sp)),
+                    60.0, lambda us_c: {"wave_instructions": n_inst,
+                                        "dense_equiv_tflops": round(n_inst * 16 * 16 * 64 * 2 / us_c * 1e-6, 1),
+                                        "pct_smfmac_peak": round(100 * n_inst * 16 * 16 * 64 * 2 / us_c * 1e-6 / SMFMAC_PEAK_TFLOPS, 1)})
+        out["calibration"] = calib
 
     def side_figures(r2, c2, n2, m2, v2, w2, k2):
         by = algorithmic_bytes(r2, c2, n2, m2, v2, w2["geo"].ksp)

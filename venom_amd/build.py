@@ -100,7 +100,32 @@ def build(verbose=False, with_driver=True, with_out_32b=False, with_torch_ext=Tr
              verbose)
     if with_torch_ext:
         _torch_ext_link(verbose)
+    build_calibrate(verbose)
     return LIB
+
+
+def build_calibrate(verbose=False):
+    """The machine calibration kernels of `bench.py --calibrate` (csrc/calibrate.hip): a library of their own,
+    venom_amd/lib/libspatha_calibrate.so, so that the SpMM library exports the SpMM interface only."""
+    lib = os.path.join(LIBDIR, "libspatha_calibrate.so")
+    _run([HIPCC] + HIP_FLAGS + ["-x", "hip", "-shared", os.path.join(CSRC, "calibrate.hip"), "-o", lib], verbose)
+    return lib
+
+
+def build_variant(tag, defines, verbose=False, only=None):
+    """A development build of the library with extra -D switches on the kernel sources (e.g. the timing knobs of
+    spmm_pingpong.hip, SPATHA_UP_KNOBS=<bits>) -> venom_amd/lib/libspatha_<tag>.so; `SPATHA_LIBRARY=<that file>` makes the
+    Python binding and bench.py load it.  Needs the objects of a normal build.  Such builds compute wrong results on
+    purpose (a knob removes part of the kernel's work) and are for timing and power measurements only.  `only` names the
+    kernel sources that see the switches (default: all of them)."""
+    sources = [src for src in KERNEL_SOURCES if not only or src in only]
+    jobs = [[HIPCC] + HIP_FLAGS + ["-D" + d for d in defines] +
+            ["-x", "hip", "-c", os.path.join(CSRC, src), "-o", os.path.join(OBJDIR, "%s.%s.o" % (src, tag))] for src in sources]
+    _compile_all(jobs, verbose)
+    lib = os.path.join(LIBDIR, "libspatha_%s.so" % tag)
+    objs = [os.path.join(OBJDIR, s + (".%s.o" % tag if s in sources else ".o")) for s in CXX_SOURCES + HIP_SOURCES]
+    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", lib] + objs + ["-lgomp"], verbose)
+    return lib
 
 
 def build_out_32b(verbose=False):
@@ -124,5 +149,12 @@ def _out_32b_link(verbose):
 
 
 if __name__ == "__main__":
-    build(verbose=True, with_out_32b="--ablation" in sys.argv[1:])
+    # python -m venom_amd.build [--ablation]            the library, the driver, the PyTorch extension (+ the OUT_32B build)
+    # python -m venom_amd.build --variant TAG [--only SRC.hip] -DX=1 ...  a development build libspatha_TAG.so (after a normal build)
+    argv = sys.argv[1:]
+    if "--variant" in argv:
+        only = [argv[i + 1] for i, a in enumerate(argv) if a == "--only"]
+        build_variant(argv[argv.index("--variant") + 1], [a[2:] for a in argv if a.startswith("-D")], verbose=True, only=only)
+    else:
+        build(verbose=True, with_out_32b="--ablation" in argv)
     sys.exit(0)

@@ -27,7 +27,7 @@
 // Development switches, compiled in with -DSPATHA_UP_KNOBS=<bits> for timing experiments only (0 in the library; the
 // results are then wrong on purpose):  1 no B stages (matrix phases on whatever the LDS holds)   2 no write-out
 //   4 the late group skips its matrix phases   8 a second barrier in the middle of a step   16 no A operands (only
-//   the gather table is loaded)   32 write-out without its global stores
+//   the gather table is loaded)   32 write-out without its global stores   64 no matrix instructions
 #ifndef SPATHA_UP_KNOBS
 #define SPATHA_UP_KNOBS 0
 #endif
@@ -232,7 +232,8 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
 #pragma unroll
             for (int mb = 0; mb < 4; mb++) {
                 float4_t& c = acc[nb8 >> 2][mb][nb8 & 3];
-                if (mb & 1) c = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[mb], bf[nb8 % 3], c, (int)ix[mb >> 1], 0, 1);
+                if (UP_KNOBS & 64) asm volatile("" ::"v"(bf[nb8 % 3]), "v"(a_cur[mb]), "v"(ix[mb >> 1]));
+                else if (mb & 1) c = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[mb], bf[nb8 % 3], c, (int)ix[mb >> 1], 0, 1);
                 else c = __builtin_amdgcn_smfmac_f32_16x16x64_f16(a_cur[mb], bf[nb8 % 3], c, (int)ix[mb >> 1], 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
                 if (nb8 + 2 < 8) read_part(bf[(nb8 + 2) % 3], nb8 + 2, mb);
@@ -348,10 +349,15 @@ static hipError_t launch_up(const SpmmParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// largest m that runs the grouped form of the matrix phase
+#ifndef SPATHA_UP_GROUPED_MAX_M
+#define SPATHA_UP_GROUPED_MAX_M 5
+#endif
+
 hipError_t launch_pingpong(int variant, int out_layout, const SpmmParams& p, hipStream_t stream) {
     if (variant != SPMM_VARIANT_UP512x128_S3) return hipErrorInvalidValue;
     // (the plain instantiations carry nothing of the fused write-out; the form of the matrix phase follows m, see there)
-    const bool t = out_layout == SPATHA_OUT_TRANSPOSED, grouped = p.m <= 5;
+    const bool t = out_layout == SPATHA_OUT_TRANSPOSED, grouped = p.m <= SPATHA_UP_GROUPED_MAX_M;
     if (p.fuse) {
         if (grouped) return t ? launch_up<SPATHA_OUT_TRANSPOSED, true, true>(p, stream) : launch_up<SPATHA_OUT_ROW_MAJOR, true, true>(p, stream);
         return t ? launch_up<SPATHA_OUT_TRANSPOSED, true, false>(p, stream) : launch_up<SPATHA_OUT_ROW_MAJOR, true, false>(p, stream);

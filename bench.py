@@ -50,9 +50,14 @@ def smi_sample():
         r = subprocess.run(["amd-smi", "metric", "--power", "--clock", "--json"], capture_output=True, text=True, timeout=10)
     except (OSError, subprocess.SubprocessError):
         return None
-    watts = re.search(r'"socket_power": \{\s*"value": (\d+)', r.stdout)
-    clocks = re.findall(r'"gfx_\d+": \{\s*"clk": \{\s*"value": (\d+)', r.stdout)
-    if r.returncode != 0 or not watts or not clocks:
+    return parse_smi(r.stdout) if r.returncode == 0 else None
+
+
+def parse_smi(text):
+    """The two figures out of the tool's JSON text (one "socket_power" value, one "clk" value per "gfx_<n>" entry), or None."""
+    watts = re.search(r'"socket_power": \{\s*"value": (\d+)', text)
+    clocks = re.findall(r'"gfx_\d+": \{\s*"clk": \{\s*"value": (\d+)', text)
+    if not watts or not clocks:
         return None
     return int(watts.group(1)), sum(map(int, clocks)) / len(clocks)
 

@@ -102,9 +102,10 @@ struct Shape {
     // 128 x 256 tiles ahead of 128 x 128 ones: from 1024 tiles on, from 768 with two or more k-steps, from 512 with eight or
     // more, from 192 with a dozen or more (every kernel on the BERT layer shapes x N = 2048 .. 8192 x 2:10 .. 2:100;
     // 1024 x 1024 x 16384 at 128:2:16, 512 wide tiles of 4 k-steps, runs 19 % faster on 128 x 128 tiles)
+    // (never for a single, half-empty column tile: GPT-3 FFN matrix at 128 tokens, 46.5 us on 128 x 128 against 61.5 us)
     bool wide() const {
         const int64_t t = tiles(128, 256);
-        return t >= 1024 || (t >= 768 && S >= 2) || (t >= 512 && S >= 8) || (t >= 192 && S >= 12);
+        return N > 128 && (t >= 1024 || (t >= 768 && S >= 2) || (t >= 512 && S >= 8) || (t >= 192 && S >= 12));
     }
     // 64 x 256 tiles with long k-loops and either many rounds or at most one
     bool long_k() const { const int64_t t = tiles(64, 256); return S >= 32 && (t >= 2048 || t <= 256); }
@@ -170,11 +171,11 @@ const Rule kRules[] = {
      }},
     {V_128, spatha::SPMM_VARIANT_DS256x128_S3_C8,
      [](const Shape& s) { return !s.transposed && s.m <= 8 && s.rows % 256 == 0 && s.tiles(256, 128) >= 160 && s.S <= 64; }},
-    // transposed output, m > 8: 128 x 256 tiles at any tile count (5-15 % ahead of 128 x 128 on the BERT-large and
+    // transposed output, m > 8, more than one 128-column tile: 128 x 256 tiles at any tile count (5-15 % ahead of 128 x 128 on the BERT-large and
     // GPT-2-large layer shapes, N = 4096 and 16384); 64 x 64 consumer blocks up to 16 k-steps, else the tall consumers
-    {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.m >= 16 && s.S <= 16; }},
-    {V_128, spatha::SPMM_VARIANT_T128x256_S3, [](const Shape& s) { return s.transposed && s.m > 8; }},
-    {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.m > 8; }},
+    {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m >= 16 && s.S <= 16; }},
+    {V_128, spatha::SPMM_VARIANT_T128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m > 8; }},
+    {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m > 8; }},
     // 128 x 256 tiles, m >= 16: the 64 x 64 consumer blocks lead the tall-consumer form by 1-13 % up to 16 k-steps per tile
     // (BERT-large, GPT-2-large layers) from 768 tiles on (fewer: the tall form is 8-10 % ahead) and trail it by 1-3 % on
     // long k-loops (GPT-3 layers)

@@ -258,8 +258,9 @@ def main():
     }
 
     if idle is not None:
-        # Sustained run of the same launches with the socket power and graphics clock sampled beside it.  (The idle
-        # reading was taken before this process touched the GPU.)
+        # Sustained run of the same launches with the socket power and graphics clock sampled beside it.
+        # (socket_w_at_start: the reading before this process touched the GPU - idle power, unless another run ended
+        # within the last second or two.)
         stream = torch.cuda.current_stream(dev)
         sp = ctypes.c_void_p(stream.cuda_stream)
         plan, B, C = w["plan"], w["B"], w["C"]
@@ -267,7 +268,7 @@ def main():
             lambda: _lib.check(L.spatha_spmm_run(plan._handle, B.data_ptr(), N, None, C.data_ptr(), 0, args.variant, sp), "run"),
             torch.cuda.synchronize, ms_kernel * 1e3, args.power_seconds)
         out["power"] = {"socket_w": None if watts is None else round(watts, 1), "gfx_mhz": None if mhz is None else round(mhz, 1),
-                        "idle_socket_w": idle[0], "us_per_spmm_sustained": round(us_s, 3),
+                        "socket_w_at_start": idle[0], "us_per_spmm_sustained": round(us_s, 3),
                         "mj_per_spmm": None if watts is None else round(watts * us_s * 1e-3, 2), "samples": n_s,
                         "source": "amd-smi metric --power --clock, sampled over %.1f s of back-to-back launches after the timed "
                                   "region" % args.power_seconds}

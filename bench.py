@@ -279,7 +279,7 @@ def main():
         cal = ctypes.CDLL(os.path.join(ROOT, "venom_amd", "lib", "libspatha_calibrate.so"))
         cal.spatha_calibrate_store.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
         cal.spatha_calibrate_smfmac.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
-                                                ctypes.c_void_p]
+                                                ctypes.c_int, ctypes.c_void_p]
         stream = torch.cuda.current_stream(dev)
         sp = ctypes.c_void_p(stream.cuda_stream)
         wgs = torch.cuda.get_device_properties(dev).multi_processor_count
@@ -319,11 +319,14 @@ def main():
         }
         for name, (a32, b32) in operand_sets.items():
             a16, b16 = a32.to(torch.float16), b32.to(torch.float16)
-            n_inst = wgs * 8 * passes * 32
-            run_cal(name, lambda: check_hip(cal.spatha_calibrate_smfmac(a16.data_ptr(), b16.data_ptr(), out_c.data_ptr(), wgs, passes, sp)),
-                    60.0, lambda us_c: {"wave_instructions": n_inst,
-                                        "dense_equiv_tflops": round(n_inst * 16 * 16 * 64 * 2 / us_c * 1e-6, 1),
-                                        "pct_smfmac_peak": round(100 * n_inst * 16 * 16 * 64 * 2 / us_c * 1e-6 / SMFMAC_PEAK_TFLOPS, 1)})
+            # the 16 x 16 x 64 instruction the kernels use; for Gaussian operands also 32 x 32 x 32 (half as many instructions)
+            for shape in ((16, 32) if name.endswith("gaussian") else (16,)):
+                n_inst = wgs * 8 * passes * (32 if shape == 16 else 16)
+                flops = wgs * 8 * passes * 32 * 16 * 16 * 64 * 2
+                run_cal(name if shape == 16 else name.replace("smfmac_", "smfmac32x32x32_"),
+                        lambda: check_hip(cal.spatha_calibrate_smfmac(a16.data_ptr(), b16.data_ptr(), out_c.data_ptr(), wgs, passes, shape, sp)),
+                        60.0, lambda us_c: {"wave_instructions": n_inst, "dense_equiv_tflops": round(flops / us_c * 1e-6, 1),
+                                            "pct_smfmac_peak": round(100 * flops / us_c * 1e-6 / SMFMAC_PEAK_TFLOPS, 1)})
         out["calibration"] = calib
 
     def side_figures(r2, c2, n2, m2, v2, w2, k2):

@@ -62,7 +62,8 @@ def test_short_run_prints_one_line_with_roofline_power_and_calibration():
     if out["power"] is not None:
         assert out["power"]["us_per_spmm_sustained"] > 0
     cal = out["calibration"]
-    assert set(cal) == {"store_c_alone", "smfmac_alone_gaussian", "smfmac_alone_integers", "smfmac_alone_zeros"}
+    assert set(cal) == {"store_c_alone", "smfmac_alone_gaussian", "smfmac32x32x32_alone_gaussian", "smfmac_alone_integers",
+                        "smfmac_alone_zeros"}
     assert 1.0 < cal["store_c_alone"]["tb_per_s"] < 20.0
     # zeros are the cheapest operands: never slower than Gaussian ones, and never above the nominal peak
     assert cal["smfmac_alone_gaussian"]["pct_smfmac_peak"] <= cal["smfmac_alone_zeros"]["pct_smfmac_peak"] * 1.05 <= 105.0

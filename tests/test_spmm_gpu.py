@@ -402,6 +402,35 @@ def test_gpt3_ffn_shape_blocks_within_tolerance(gpu, N):
         assert (np.abs(got - want) / np.maximum(np.abs(want), 1.0)).max() <= REL_TOL
 
 
+@pytest.mark.parametrize("transposed", [False, True])
+def test_uneven_last_round_runs_as_two_launches(gpu, transposed):
+    """More 128 x 256 tiles than compute units with a rest of at most half a round: the automatic choice runs the rest's row
+    tiles as a second launch on 128 x 128 tiles.  Both launches together equal the oracle bit for bit (integer operands),
+    also with the bias of the transposed layout and with the fused bias of the row-major one, and equal the one-launch result
+    of the same kernel asked for by id."""
+    cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+    grid = cus // 8 * 8
+    N, m, v, cols = 2048, 16, 128, 3072
+    rows = (grid // 8 + grid // 16) * 128            # 1.5 rounds of 128 x 256 tiles (8 column tiles)
+    print("uneven last round", rows, cols, N, transposed, flush=True)
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=5, integer_values=True)
+    rng = np.random.default_rng(11)
+    B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+    bias = rng.integers(-3, 4, size=rows).astype(np.float16)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    name = plan.kernel_name(N, 1 if transposed else 0, 0)
+    assert name.endswith("+rest_on_tile128x128"), name
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias if transposed else None, transposed_out=transposed)
+    got = plan.run(_dev(B, gpu), bias=_dev(bias, gpu) if transposed else None, transposed_out=transposed)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    one = plan.run(_dev(B, gpu), bias=_dev(bias, gpu) if transposed else None, transposed_out=transposed, variant=10)
+    assert torch.equal(one, got)
+    fused = plan.run(_dev(B, gpu), bias=_dev(bias, gpu), transposed_out=transposed, activation="none")
+    want_b = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias, transposed_out=True)       # [N, rows]
+    want_b = want_b if transposed else np.ascontiguousarray(want_b.T)
+    assert np.array_equal(fused.cpu().numpy().view(np.uint16), want_b.view(np.uint16))
+
+
 K_TAIL_CASES = [
     # rows, cols, N, m, v : cols % (16 m) != 0, so the last k-step of a dense-staged kernel spans rows beyond K
     (1024, 200, 264, 8, 64),

@@ -236,6 +236,23 @@ int pick_variant(const spatha_spmm_plan* plan, int N, int variant, bool fused = 
         if ((r.v_classes & v_class) && r.when(s) && variant_ok(plan, N, r.variant, fused)) return r.variant;
     return -1;
 }
+
+// An uneven last round of 128 x 256 tiles (automatic choice only): when the tiles fill one or more rounds of the CUs and
+// leave a rest of at most half a round, the rest's row tiles run as a second launch on 128 x 128 tiles - twice as many
+// tiles of half the work, so that its one round keeps every CU busy (GPT-3 FFN matrix at 256 tokens: 384 tiles on 256
+// CUs).  Returns the rows of that second launch (the last rows of the matrix), 0 for a single launch.
+int uneven_rest_rows(const spatha_spmm_plan* plan, int N, int requested, int chosen, bool fused) {
+    if (requested != spatha::SPMM_VARIANT_AUTO || plan->cus < 8) return 0;
+    if (chosen != spatha::SPMM_VARIANT_T128x256_S3 && chosen != spatha::SPMM_VARIANT_W128x256_S3) return 0;
+    const int grid = (plan->cus / 8) * 8;       // workgroups of the persistent kernels
+    const int tiles_n = (N + 255) / 256;
+    const int64_t tiles = (int64_t)(plan->geo.rows / 128) * tiles_n, rest = tiles % grid;
+    if (tiles <= grid || rest == 0 || rest % tiles_n != 0) return 0;
+    const int rest_rows = (int)(rest / tiles_n) * 128;
+    if ((int64_t)(rest_rows / 128) * ((N + 127) / 128) > grid) return 0;        // more than half a round: one launch
+    if ((plan->geo.rows - rest_rows) % plan->geo.v != 0) return 0;
+    return variant_ok(plan, N, spatha::SPMM_VARIANT_W128x128_S3, fused) ? rest_rows : 0;
+}
 }  // namespace
 
 namespace spatha {
@@ -471,6 +488,25 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
     { const char* d = std::getenv("SPATHA_SKEW"); p.skew = d ? std::atoi(d) : 0; }
     { const char* d = std::getenv("SPATHA_PROF_PTR"); if (d) p.prof = (long long*)std::strtoull(d, nullptr, 0); }
 #endif
+    if (const int rest_rows = uneven_rest_rows(plan, N, variant, var, fuse)) {
+        const int main_rows = plan->geo.rows - rest_rows;
+        spatha::SpmmParams head = p, tail = p;
+        head.tiles_m = main_rows / 128;
+        const size_t a_off = (size_t)(main_rows / 64) * plan->S * spatha::APACK_BLOCK;
+        const size_t rt_off = (size_t)(main_rows / plan->geo.v) * plan->S * 64 * 4;
+        tail.apack = (const uint16_t*)((const char*)plan->apack + a_off);
+        tail.apack_bytes = (uint32_t)(plan->apack_bytes - a_off);
+        tail.rowtab = (const uint32_t*)((const char*)plan->rowtab + rt_off);
+        tail.rowtab_bytes = (uint32_t)(plan->rowtab_bytes - rt_off);
+        if (bias_dev) tail.bias = bias_dev + main_rows;
+        // (p.rows stays the full row count: these kernels use it as the row stride of the transposed layout only)
+        tail.C = out_layout == SPATHA_OUT_TRANSPOSED ? out_dev + main_rows : out_dev + (size_t)main_rows * N;
+        tail.tiles_m = rest_rows / 128;
+        tail.tiles_n = (N + 127) / 128;
+        hipError_t e2 = spatha::launch_spmm(var, out_layout, head, (hipStream_t)stream);
+        if (e2 == hipSuccess) e2 = spatha::launch_spmm(spatha::SPMM_VARIANT_W128x128_S3, out_layout, tail, (hipStream_t)stream);
+        return e2 == hipSuccess ? SPATHA_OK : hip_fail(e2);
+    }
     hipError_t e = spatha::launch_spmm(var, out_layout, p, (hipStream_t)stream);
     return e == hipSuccess ? SPATHA_OK : hip_fail(e);
 }
@@ -492,7 +528,11 @@ int spatha_spmm_num_variants(void) { return spatha::SPMM_VARIANT_COUNT; }
 const char* spatha_spmm_kernel_name(const spatha_spmm_plan* plan, int N, int out_layout, int variant) {
     if (!plan) return nullptr;
     int var = pick_variant(plan, N, variant, false, out_layout);
-    return var < 0 ? nullptr : spatha::spmm_variant_name(var);
+    if (var < 0) return nullptr;
+    if (uneven_rest_rows(plan, N, variant, var, false))     // two launches: the rest of an uneven last round on 128 x 128 tiles
+        return var == spatha::SPMM_VARIANT_T128x256_S3 ? "smfmac16x16x64_warpspec_tall_tile128x256_3stage+rest_on_tile128x128"
+                                                       : "smfmac16x16x64_warpspec_tile128x256_3stage+rest_on_tile128x128";
+    return spatha::spmm_variant_name(var);
 }
 
 int spatha_spmm_time(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,

@@ -127,8 +127,9 @@ const Rule kRules[] = {
     {V_HALF | V_128 | V_64, spatha::SPMM_VARIANT_SKINNY, [](const Shape& s) { return s.N <= 32; }},
     // V a multiple of 64 only, m <= 8, up to 48 columns: still 9-22 % ahead of the dense-staged 256 x 128 tiles (4096 x 1024 and
     // 12288 x 12288 at 64:2:8; at 64 columns ahead on the larger matrix only).  With V % 128 == 0 the 128 x 128 tiles lead it by
-    // 5-10 % from 40 columns on (m = 4 .. 32).
-    {V_64, spatha::SPMM_VARIANT_SKINNY, [](const Shape& s) { return s.N <= 48 && s.m <= 8; }},
+    // 5-10 % from 40 columns on (m = 4 .. 32).  m > 8 with a dozen or more k-steps: up to 64 columns, 15-22 % ahead of the
+    // gathered 64 x 256 tiles (1024 x 4096 and 768 x 3072 at 64:2:16; with fewer k-steps 11-30 % behind them).
+    {V_64, spatha::SPMM_VARIANT_SKINNY, [](const Shape& s) { return s.m <= 8 ? s.N <= 48 : (s.N <= 64 && s.S >= 12); }},
 
     // -- V % 64 != 0 (1024 x 4096 x 4096 and 4096 x 1024 x 16384, m = 8 .. 32) --
     // m <= 8: the dense B stage is shared by eight 32-row blocks, the fill does not grow with the smaller V

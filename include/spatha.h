@@ -200,7 +200,9 @@ int spatha_spmm_run_noalloc(int rows, int cols, int n, int m, int v, const uint1
 int spatha_spmm_num_variants(void);
 
 /* Name / tile shape of the kernel `variant` (or of the automatic choice for N
- * when variant == 0) would use, for logs; returns NULL if unsupported. */
+ * when variant == 0) would use, for logs; returns NULL if unsupported.  The
+ * automatic choice may be two launches (the row tiles of an uneven last round of
+ * 128 x 256 tiles on 128 x 128 tiles): the name then ends in "+rest_on_tile128x128". */
 const char* spatha_spmm_kernel_name(const spatha_spmm_plan* plan, int N, int out_layout, int variant);
 
 /* Times `iters` back-to-back launches with HIP events on `stream` after

@@ -431,6 +431,38 @@ def test_uneven_last_round_runs_as_two_launches(gpu, transposed):
     assert np.array_equal(fused.cpu().numpy().view(np.uint16), want_b.view(np.uint16))
 
 
+@pytest.mark.parametrize("rows,cols,N,m,v", [(1024, 512, 256, 8, 64),        # unified 512 x 128 kernel
+                                            (512, 2048, 520, 16, 128),       # producer/consumer kernel, ragged N
+                                            (256, 1024, 16, 16, 128)])       # skinny kernel
+def test_run_recorded_into_a_graph_replays_with_new_operands(gpu, rows, cols, N, m, v):
+    """`spatha_spmm_run` allocates nothing, clears nothing and waits for nothing: a caller can record it into a HIP graph.
+    Three replays with new contents of B, eager launches and synchronisations between them, each replay equal to the oracle
+    and to the eager result."""
+    print("graph", rows, cols, N, m, v, flush=True)
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=3, integer_values=True)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    rng = np.random.default_rng(7)
+    dB = _dev(rng.integers(-4, 5, size=(cols, N)).astype(np.float16), gpu)
+    out = torch.empty((rows, N), dtype=torch.float16, device=gpu)
+    plan.run(dB, out=out)              # first launch outside the capture: kernel attributes are set once per process
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.run(dB, out=out)
+    for rep in range(3):
+        B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+        dB.copy_(_dev(B, gpu))
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B)
+        assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16)), rep
+        eager = plan.run(dB)
+        torch.cuda.synchronize()
+        assert torch.equal(eager, out), rep
+
+
 K_TAIL_CASES = [
     # rows, cols, N, m, v : cols % (16 m) != 0, so the last k-step of a dense-staged kernel spans rows beyond K
     (1024, 200, 264, 8, 64),

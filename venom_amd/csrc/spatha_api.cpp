@@ -31,7 +31,7 @@ bool variant_has_fused_writeout(int variant) {
         case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_R64x256_S3:
         case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x256_S3: case SPMM_VARIANT_W64x256_S3:
         case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DSH256x128_S3_C8:
-        case SPMM_VARIANT_UP512x128_S3: case SPMM_VARIANT_DU512x128_M16:
+        case SPMM_VARIANT_UP512x128_S3: case SPMM_VARIANT_DU512x128_M16: case SPMM_VARIANT_WS128x128_S3:
             return true;
         default:
             return false;
@@ -76,6 +76,7 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = f
         return false;
     }
     if (variant == SPMM_VARIANT_SKINNY && N > 64) return false;
+    if (variant == SPMM_VARIANT_WS128x128_S3 && plan->S < 2) return false;    // its tile hand-over needs two k-steps per tile
     if (spmm_variant_lds(variant, plan->S) > 160 * 1024) return false;      // row table kept in LDS
     if (variant_uses_buffer_descriptors(variant) &&
         (b_bytes >= 0xE0000000ull || plan->apack_bytes >= 0xE0000000ull || plan->rowtab_bytes >= 0xE0000000ull))
@@ -181,6 +182,12 @@ const Rule kRules[] = {
     {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m >= 16 && s.S <= 16; }},
     {V_128, spatha::SPMM_VARIANT_T128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m > 8; }},
     {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m > 8; }},
+    // row-major, two or three k-steps per tile and more than two rounds of 128 x 128 tiles: the kernel with store waves (a finished tile
+    // leaves while the next one's k-loop runs) leads the 128 x 256 tiles by 7-18 % and the plain 128 x 128 ones by 14-23 %
+    // (4096 x 1024 x 16384 at 128:2:32, 3072 x 768 x 8192 at 128:2:40, 1024 x 1024 x 16384 at 128:2:32); with transposed output
+    // it is level with the plain kernel and behind the 128 x 256 tiles
+    {V_128, spatha::SPMM_VARIANT_WS128x128_S3,
+     [](const Shape& s) { return !s.transposed && s.m > 8 && s.S >= 2 && s.S <= 3 && s.tiles(128, 128) > 2 * s.cus; }},
     // 128 x 256 tiles, m >= 16: the 64 x 64 consumer blocks lead the tall-consumer form by 1-13 % up to 16 k-steps per tile
     // (BERT-large, GPT-2-large layers) from 768 tiles on (fewer: the tall form is 8-10 % ahead) and trail it by 1-3 % on
     // long k-loops (GPT-3 layers)
@@ -195,6 +202,15 @@ const Rule kRules[] = {
      [](const Shape& s) {
          const int64_t t = s.tiles(128, 128);
          return !s.transposed && s.m > 8 && t > s.cus && t <= 2 * s.cus && s.S <= 8;
+     }},
+    // ... and wherever the 128 x 256 tiles do not lead and every CU has a tile: 5-13 % ahead of the plain 128 x 128 kernel
+    // (1024 x 1024 x 16384 at 128:2:16, 4096 x 1024 x 4096 at 128:2:20, 5120 x 1280 x 4096 at 128:2:16, 1024 x 4096 x 4096 at
+    // 128:2:7 .. 128:2:40), level with it on long k-loops with many tiles; 5-7 % behind with fewer tiles than CUs, and with
+    // exactly one short tile per CU (1024 x 1024 x 4096 at 128:2:40)
+    {V_128, spatha::SPMM_VARIANT_WS128x128_S3,
+     [](const Shape& s) {
+         const int64_t t = s.tiles(128, 128);
+         return !s.transposed && s.S >= 2 && t >= s.cus && (t > s.cus || s.S >= 4);
      }},
     {V_128, spatha::SPMM_VARIANT_W128x128_S3, [](const Shape&) { return true; }},
     {V_128, spatha::SPMM_VARIANT_P128x128_S3, [](const Shape&) { return true; }},

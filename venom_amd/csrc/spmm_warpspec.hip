@@ -20,7 +20,7 @@ namespace spatha {
 // it comes to which DMA instructions of a stage it issues.
 // ---------------------------------------------------------------------------
 
-template <class Cfg, int NP, int PR>
+template <class Cfg, int NP, int PR, bool FINAL_BARRIER = false>
 __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk& walk, char* smem, uint32_t smem_base,
                                             int lane) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1, PA = Cfg::PA;
@@ -149,6 +149,7 @@ __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk&
         wait_stages<LOADS, PA - 1>(Q - 1 - q);
         __syncthreads();
     }
+    if (FINAL_BARRIER) __syncthreads();     // (kernels with store waves: the last tile's hand-over)
 }
 
 template <class Cfg, int WN, int OUT_LAYOUT>
@@ -522,6 +523,233 @@ static hipError_t launch_ws(const SpmmParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// 128 x 128 tiles with a third role: store waves.  A consumer wave that has finished a tile rounds its 64 x 64 block to
+// fp16 (bias / activation applied) and leaves it in an LDS staging buffer that holds the whole tile in output order; it then
+// starts the next tile at once.  Four store waves pick the tile up behind the next step barrier - each a quarter of it, into
+// registers - and write it to C in pieces after the following step barriers, so that the global stores of a tile are spread
+// over the next tile's k-loop and never wait on the waves that issue the matrix instructions.  (The producers cannot
+// take the stores over: stores in flight would sit in the same counter as the loads they wait for.)
+//   consumer: step barriers of tile t | dump t             | step barriers of tile t + 1 | dump t + 1
+//   store wave:                                             barrier 0: read t, store 1/n | barrier 1: store 2/n ...
+// The staging buffer is free again when the consumers dump the next tile: the store waves have read all of it before they
+// join the second step barrier, and a tile has two k-steps or more (the host refuses S = 1 for this kernel).
+// ---------------------------------------------------------------------------
+template <int NS, int NP>
+struct WswCfg {
+    static constexpr int NC = 4, NSW = 4;
+    static constexpr int BM = 128, BN = 128;
+    static constexpr int ROW_BYTES = BN * 2;
+    static constexpr int B_BYTES = 64 * ROW_BYTES;
+    static constexpr int STAGE_BYTES = B_BYTES + 2 * APACK_BLOCK;
+    static constexpr int PA = NS - 1;
+    static constexpr int STG_PITCH = 128 * 2 + 16;                  // a tile row (or, transposed, a tile column) + 16 B
+    static constexpr int EPI_BYTES = 128 * STG_PITCH;               // the staging buffer
+    static constexpr int RT_BYTES = NP * (PA + 1) * 256;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES + EPI_BYTES + RT_BYTES;
+    static constexpr int THREADS = (NC + NP + NSW) * 64;
+    static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
+    static constexpr uint32_t RT_BASE = EPI_BASE + EPI_BYTES;
+};
+
+template <class Cfg, int OUT_LAYOUT>
+__device__ __forceinline__ void wsw_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1, WN = 2;
+    constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES, PITCH = Cfg::STG_PITCH;
+    const int S = p.S;
+    const int wm = wave / WN, wn = wave - wm * WN;
+    float4_t acc[4][4];
+    const int li = lane & 15, kb = lane >> 4;
+    const int rrow = kb * 4 + (li >> 2);
+    const int sw = rrow & 7;
+    int tr_off[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; nb++) {
+        const int ch = (wn * 8 + nb * 2 + ((li & 3) >> 1)) ^ (sw << 1);
+        tr_off[nb] = rrow * ROW_BYTES + ch * 16 + (li & 1) * 8;
+    }
+    const int a_off = B_BYTES + wm * APACK_BLOCK + lane * 16;
+    const int i_off = B_BYTES + wm * APACK_BLOCK + 4096 + lane * 4;
+    const int j16 = lane & 15, ib = lane >> 4;
+    char* stg = smem + Cfg::EPI_BASE;
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    uint32_t c_stage = 0;
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        for (int c_step = 0; c_step < S; c_step++) {
+            __syncthreads();
+            mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {});
+            c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
+        }
+        const int cm0 = c_tm * BM;
+        // lane (j16, ib) holds column nb*16 + j16, rows ib*16 + mb*4 + 0..3 of the wave's block
+        if (p.fuse) fused_bias_act(acc, p.bias, (int64_t)cm0 + wm * 64 + ib * 16, p.act);
+        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+            // staging [tile column][tile row]: four consecutive rows of one column are 8 contiguous bytes
+            const bool with_bias = !p.fuse && p.bias;
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) {
+                const int row = wm * 64 + ib * 16 + mb * 4;
+                half4_t b4 = {0, 0, 0, 0};
+                if (with_bias) b4 = *(const half4_t*)(p.bias + cm0 + row);
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++) {
+                    half4_t h4;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) h4[r] = (_Float16)acc[mb][nb][r];
+                    if (with_bias) h4 = h4 + b4;        // fp16 addition on the rounded product
+                    *(half4_t*)(stg + (wn * 64 + nb * 16 + j16) * PITCH + row * 2) = h4;
+                }
+            }
+        } else {
+            // staging: per consumer block eight slabs of [64 block columns][8 rows] (slab 2*mb + ib/2 holds rows
+            // 16*ib + 4*mb + r of the lane groups ib = 2*(ib/2), 2*(ib/2) + 1), 16 bytes per slab row: a lane's four
+            // rows of one column are one 8-byte write, and a store wave gets row-major pieces back with transposing reads
+            char* blk = stg + wave * 8192;
+#pragma unroll
+            for (int mb = 0; mb < 4; mb++) {
+                char* slab = blk + (mb * 2 + (ib >> 1)) * 1024;
+#pragma unroll
+                for (int nb = 0; nb < 4; nb++) {
+                    half4_t h4;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) h4[r] = (_Float16)acc[mb][nb][r];
+                    *(half4_t*)(slab + (nb * 16 + j16) * 16 + (ib & 1) * 8) = h4;
+                }
+            }
+        }
+        walk.next(c_tm, c_tn);
+    }
+    __syncthreads();        // the last tile's hand-over
+}
+
+template <class Cfg, int OUT_LAYOUT>
+__device__ __forceinline__ void wsw_storer(const SpmmParams& p, const TileWalk& walk, char* smem, int sw, int lane) {
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, PITCH = Cfg::STG_PITCH;
+    const int S = p.S, N = p.N;
+    const char* stg = smem + Cfg::EPI_BASE;
+    // this wave's quarter of the staged tile, 8 pieces of 1 KB (16 bytes per lane).  Transposed output: 32 staging rows
+    // (tile columns), a piece = 4 of them x 256 bytes.  Row-major output: the block of consumer wave `sw`, a piece = one
+    // slab = 8 rows x 128 bytes, read back row-major with transposing reads.
+    const int srow = sw * 32 + (lane >> 4), chunk = lane & 15;
+    const int li = lane & 15, kb = lane >> 4;
+    const int rd_off = (8 * (2 * kb + ((li & 3) >> 1)) + (li >> 2)) * 16 + (li & 1) * 8;
+    const int q_lo = 4 * ((li >> 2) & 1) + (li & 3);
+    const int blk_row0 = (sw >> 1) * 64, blk_col = (sw & 1) * 64 + 8 * (2 * kb + (li >> 3));
+    const int pieces_per_step = S >= 4 ? 2 : (S == 3 ? 3 : 4);
+    // (stores through asm statements: a store the compiler knows of would be waited for at the next step barrier, and every
+    // wave of the workgroup with it)
+    u32x4 held[8];
+    int h_tm = 0, h_tn = 0, next_piece = 8;          // tile held in registers; 8 = nothing left to store
+    auto load_tile = [&](int tm, int tn) {
+        if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) held[i] = *(const u32x4*)(stg + (srow + 4 * i) * PITCH + chunk * 16);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const char* slab = stg + sw * 8192 + i * 1024 + rd_off;
+                const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, slab));
+                const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4_t, slab + 4 * 16));
+                held[i].x = (uint32_t)(uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+                held[i].y = (uint32_t)(uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+                held[i].z = (uint32_t)(uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+                held[i].w = (uint32_t)(uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+            }
+        }
+        h_tm = tm;
+        h_tn = tn;
+        next_piece = 0;
+    };
+    auto store_pieces = [&](int count) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (i >= next_piece && i < next_piece + count) {
+                const int r = srow + 4 * i;         // staging row: a tile row, or (transposed) a tile column
+                if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+                    const int col = h_tn * BN + r;
+                    if (col < N) store_c16<true>(p.C + (int64_t)col * p.rows + h_tm * BM + chunk * 8, held[i]);
+                } else {
+                    const int q = 8 * (i & 1) + q_lo;                  // piece i: slab of mb = i / 2, lane groups 2*(i & 1), + 1
+                    const int row = blk_row0 + 16 * (q >> 2) + 4 * (i >> 1) + (q & 3);
+                    const int col = h_tn * BN + blk_col;
+                    if (col < N) store_c16<true>(p.C + ((int64_t)h_tm * BM + row) * N + col, held[i]);
+                }
+            }
+        }
+        next_piece += count;
+    };
+    int c_tm = walk.tm0, c_tn = walk.tn0;
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+        for (int c_step = 0; c_step < S; c_step++) {
+            __syncthreads();
+            // (the tile before that one is stored by now: its pieces went out over at most four steps, and S >= 2)
+            if (c_step == 0 && c_tile > 0) load_tile(h_tm, h_tn);
+            if (next_piece < 8) store_pieces(pieces_per_step);
+        }
+        // the coordinates of the tile the consumers are about to dump
+        h_tm = c_tm;
+        h_tn = c_tn;
+        walk.next(c_tm, c_tn);
+    }
+    __syncthreads();        // the last tile's hand-over
+    load_tile(h_tm, h_tn);
+    store_pieces(8);
+}
+
+template <int NS, int NP, int OUT_LAYOUT>
+__global__ __launch_bounds__(768) void spmm_wsw_kernel(SpmmParams p) {
+    using Cfg = WswCfg<NS, NP>;
+    static_assert(NP == 4 && Cfg::THREADS == 768, "wave counts");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    TileWalk walk;
+    walk.init(p.tiles_m, p.tiles_n);
+    if (walk.my_tiles == 0) return;
+    if (wave < Cfg::NC) {
+        wsw_consumer<Cfg, OUT_LAYOUT>(p, walk, smem, wave, lane);
+    } else if (wave < Cfg::NC + NP) {
+        const int pr = wave - Cfg::NC;
+        if (pr == 0) ws_producer<Cfg, NP, 0, true>(p, walk, smem, smem_base, lane);
+        else if (pr == 1) ws_producer<Cfg, NP, 1, true>(p, walk, smem, smem_base, lane);
+        else if (pr == 2) ws_producer<Cfg, NP, 2, true>(p, walk, smem, smem_base, lane);
+        else ws_producer<Cfg, NP, 3, true>(p, walk, smem, smem_base, lane);
+    } else {
+        wsw_storer<Cfg, OUT_LAYOUT>(p, walk, smem, wave - Cfg::NC - NP, lane);
+    }
+}
+
+template <int NS, int NP, int OUT_LAYOUT>
+static hipError_t launch_wsw(const SpmmParams& p, hipStream_t stream) {
+    using Cfg = WswCfg<NS, NP>;
+    constexpr int lds = Cfg::LDS_BYTES;
+    static_assert(lds <= 160 * 1024, "LDS budget");
+    if (p.S < 2) return hipErrorInvalidValue;
+    static int cus = 0;
+    auto kern = spmm_wsw_kernel<NS, NP, OUT_LAYOUT>;
+    bool& attr_set = lds_attr_flag((const void*)kern);
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return e;
+        int dev = 0;
+        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
+        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int tiles = p.tiles_m * p.tiles_n;
+    int grid = (cus / 8) * 8;
+    const int need = ((tiles + 7) / 8) * 8;
+    if (grid > need) grid = need;
+    if (grid < 8) grid = 8;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(Cfg::THREADS), lds, stream, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_warpspec(int variant, int out_layout, const SpmmParams& p, hipStream_t stream) {
     const bool t = out_layout == SPATHA_OUT_TRANSPOSED;
     switch (variant) {
@@ -536,6 +764,8 @@ hipError_t launch_warpspec(int variant, int out_layout, const SpmmParams& p, hip
                      : launch_ws<1, 4, 3, 2, SPATHA_OUT_ROW_MAJOR, true>(p, stream);
         case SPMM_VARIANT_T128x256_S3:
             return t ? launch_wst<4, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_wst<4, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
+        case SPMM_VARIANT_WS128x128_S3:
+            return t ? launch_wsw<3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_wsw<3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
         default: return hipErrorInvalidValue;
     }
 }

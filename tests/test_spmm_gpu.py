@@ -465,26 +465,27 @@ def test_run_recorded_into_a_graph_replays_with_new_operands(gpu, rows, cols, N,
 
 @pytest.mark.parametrize("cols", [512, 768, 1280, 2048])      # 2, 3, 5 and 8 k-steps per tile at 2:16
 @pytest.mark.parametrize("transposed", [False, True])
-def test_store_wave_kernel_hands_tiles_over_between_steps(gpu, cols, transposed):
-    """The 128 x 128 kernel with store waves (id 20) on more tiles than workgroups: every workgroup hands finished tiles to
+@pytest.mark.parametrize("variant", [20, 21])
+def test_store_wave_kernel_hands_tiles_over_between_steps(gpu, cols, transposed, variant):
+    """The kernels with store waves (id 20: 128 x 128 tiles, id 21: 64 x 256) on more tiles than workgroups: every workgroup hands finished tiles to
     its store waves while it runs the next one, the pieces of a tile leaving over two, three or four k-steps.  Bit-exact
     against the oracle with ragged N, plain, with the transposed layout's bias and with the fused bias."""
     rows, N, m, v = 2048, 4104, 16, 128
     cus = torch.cuda.get_device_properties(gpu).multi_processor_count
-    assert (rows // 128) * ((N + 127) // 128) > cus
-    print("store waves", rows, cols, N, transposed, flush=True)
+    assert (rows // 128) * ((N + 127) // 128) > cus and (rows // 64) * ((N + 255) // 256) > cus
+    print("store waves", variant, rows, cols, N, transposed, flush=True)
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=cols, integer_values=True)
     rng = np.random.default_rng(cols)
     B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
     bias = rng.integers(-3, 4, size=rows).astype(np.float16)
     plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
-    assert "storewaves" in plan.kernel_name(N, 1 if transposed else 0, 20)
+    assert "storewaves" in plan.kernel_name(N, 1 if transposed else 0, variant)
     if not transposed:
-        assert "storewaves" in plan.kernel_name(N, 0, 0)        # and it is the automatic choice for row-major output here
+        assert "storewaves_tile128x128" in plan.kernel_name(N, 0, 0)    # the automatic choice for row-major output here
     want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias if transposed else None, transposed_out=transposed)
-    got = plan.run(_dev(B, gpu), bias=_dev(bias, gpu) if transposed else None, transposed_out=transposed, variant=20)
+    got = plan.run(_dev(B, gpu), bias=_dev(bias, gpu) if transposed else None, transposed_out=transposed, variant=variant)
     assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16))
-    fused = plan.run(_dev(B, gpu), bias=_dev(bias, gpu), transposed_out=transposed, variant=20, activation="none")
+    fused = plan.run(_dev(B, gpu), bias=_dev(bias, gpu), transposed_out=transposed, variant=variant, activation="none")
     want_b = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias, transposed_out=True)
     want_b = want_b if transposed else np.ascontiguousarray(want_b.T)
     assert np.array_equal(fused.cpu().numpy().view(np.uint16), want_b.view(np.uint16))
@@ -494,7 +495,7 @@ def test_store_wave_kernel_needs_two_k_steps(gpu):
     rows, cols, N, m, v = 256, 256, 256, 16, 128        # Ksp 32: one k-step per tile
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=1, integer_values=True)
     plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
-    assert plan.kernel_name(N, 0, 20) is None and plan.kernel_name(N, 0, 6) is not None
+    assert plan.kernel_name(N, 0, 20) is None and plan.kernel_name(N, 0, 21) is None and plan.kernel_name(N, 0, 6) is not None
 
 
 K_TAIL_CASES = [

@@ -32,6 +32,7 @@ bool variant_has_fused_writeout(int variant) {
         case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x256_S3: case SPMM_VARIANT_W64x256_S3:
         case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DSH256x128_S3_C8:
         case SPMM_VARIANT_UP512x128_S3: case SPMM_VARIANT_DU512x128_M16: case SPMM_VARIANT_WS128x128_S3:
+        case SPMM_VARIANT_WS64x256_S3:
             return true;
         default:
             return false;
@@ -76,7 +77,8 @@ bool variant_ok(const spatha_spmm_plan* plan, int N, int variant, bool fused = f
         return false;
     }
     if (variant == SPMM_VARIANT_SKINNY && N > 64) return false;
-    if (variant == SPMM_VARIANT_WS128x128_S3 && plan->S < 2) return false;    // its tile hand-over needs two k-steps per tile
+    if ((variant == SPMM_VARIANT_WS128x128_S3 || variant == SPMM_VARIANT_WS64x256_S3) && plan->S < 2)
+        return false;       // the tile hand-over to the store waves needs two k-steps per tile
     if (spmm_variant_lds(variant, plan->S) > 160 * 1024) return false;      // row table kept in LDS
     if (variant_uses_buffer_descriptors(variant) &&
         (b_bytes >= 0xE0000000ull || plan->apack_bytes >= 0xE0000000ull || plan->rowtab_bytes >= 0xE0000000ull))
@@ -195,13 +197,14 @@ const Rule kRules[] = {
      [](const Shape& s) { return s.wide() && s.m >= 16 && s.S <= 16 && s.tiles(128, 256) >= 768; }},
     {V_128, spatha::SPMM_VARIANT_T128x256_S3, [](const Shape& s) { return s.wide(); }},
     {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.wide(); }},
-    // more than one round of 128 x 128 tiles but at most two, few k-steps: the same number of 64 x 256 tiles runs as one
+    // more than one round of 128 x 128 tiles but less than two (two full rounds: the kernel with store waves is level or up to 6 %
+    // ahead), few k-steps: the same number of 64 x 256 tiles runs as one
     // round of two co-resident workgroups per CU (768 x 768 x 8192, 3072 x 768 x 2048, 1024 x 1024 x 8192, 4096 x 1024 x
     // 2048 at 128:2:10 .. 128:2:100: 5-30 % ahead)
     {V_128, spatha::SPMM_VARIANT_P64x256_S2,
      [](const Shape& s) {
          const int64_t t = s.tiles(128, 128);
-         return !s.transposed && s.m > 8 && t > s.cus && t <= 2 * s.cus && s.S <= 8;
+         return !s.transposed && s.m > 8 && t > s.cus && t < 2 * s.cus && s.S <= 8;
      }},
     // ... and wherever the 128 x 256 tiles do not lead and every CU has a tile: 5-13 % ahead of the plain 128 x 128 kernel
     // (1024 x 1024 x 16384 at 128:2:16, 4096 x 1024 x 4096 at 128:2:20, 5120 x 1280 x 4096 at 128:2:16, 1024 x 4096 x 4096 at
@@ -221,6 +224,11 @@ const Rule kRules[] = {
     {V_64, spatha::SPMM_VARIANT_DS256x128_S3_PP,
      [](const Shape& s) { return !s.transposed && !s.fused && s.tiles(256, 128) <= 768 && s.S <= 32; }},
     {V_64, spatha::SPMM_VARIANT_DS256x128_S3_C8, [](const Shape&) { return true; }},
+    // m > 8, row-major, two or three k-steps per tile and six rounds or more of 64 x 256 tiles: the producer/consumer kernel
+    // with store waves, 9-10 % ahead of the plain one and of the per-tile pipeline (4096 x 1024 x 16384 at 64:2:32, 3072 x
+    // 768 x 8192 at 64:2:40); level at four rounds, behind with fewer tiles, with four k-steps or more, and with transposed output
+    {V_64, spatha::SPMM_VARIANT_WS64x256_S3,
+     [](const Shape& s) { return !s.transposed && s.m > 8 && s.S >= 2 && s.S <= 3 && s.tiles(64, 256) >= 6 * s.cus; }},
     // m > 8, gathered 64 x 256 tiles.  32 or more k-steps per tile and many rounds: the persistent pipeline, which keeps
     // loading across tile boundaries, leads (GPT-3 layers at 64:2:16; at 64:2:32, 24 k-steps, the per-tile pipeline is
     // 10-20 % ahead); with one tile per CU or less its third stage still gives long k-loops 5-15 %

@@ -535,16 +535,19 @@ static hipError_t launch_ws(const SpmmParams& p, hipStream_t stream) {
 // The staging buffer is free again when the consumers dump the next tile: the store waves have read all of it before they
 // join the second step barrier, and a tile has two k-steps or more (the host refuses S = 1 for this kernel).
 // ---------------------------------------------------------------------------
-template <int NS, int NP>
+template <int WM_, int WN_, int NS, int NP_>
 struct WswCfg {
+    static_assert(WM_ * WN_ == 4, "four consumer waves, four store waves");
+    static constexpr int WM = WM_, WN = WN_, NP = NP_;
     static constexpr int NC = 4, NSW = 4;
-    static constexpr int BM = 128, BN = 128;
+    static constexpr int BM = WM * 64, BN = WN * 64;
     static constexpr int ROW_BYTES = BN * 2;
     static constexpr int B_BYTES = 64 * ROW_BYTES;
-    static constexpr int STAGE_BYTES = B_BYTES + 2 * APACK_BLOCK;
+    static constexpr int STAGE_BYTES = B_BYTES + WM * APACK_BLOCK;
     static constexpr int PA = NS - 1;
-    static constexpr int STG_PITCH = 128 * 2 + 16;                  // a tile row (or, transposed, a tile column) + 16 B
-    static constexpr int EPI_BYTES = 128 * STG_PITCH;               // the staging buffer
+    static constexpr int STG_PITCH = BM * 2 + 16;                   // transposed output: a tile column (BM rows) + 16 B
+    // the staging buffer: row-major output 4 blocks x 8 slabs x 1 KB, transposed output BN tile columns
+    static constexpr int EPI_BYTES = BN * STG_PITCH > 4 * 8192 ? BN * STG_PITCH : 4 * 8192;
     static constexpr int RT_BYTES = NP * (PA + 1) * 256;
     static constexpr int LDS_BYTES = NS * STAGE_BYTES + EPI_BYTES + RT_BYTES;
     static constexpr int THREADS = (NC + NP + NSW) * 64;
@@ -554,7 +557,7 @@ struct WswCfg {
 
 template <class Cfg, int OUT_LAYOUT>
 __device__ __forceinline__ void wsw_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
-    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1, WN = 2;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1, WN = Cfg::WN;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES, PITCH = Cfg::STG_PITCH;
     const int S = p.S;
     const int wm = wave / WN, wn = wave - wm * WN;
@@ -631,14 +634,15 @@ __device__ __forceinline__ void wsw_storer(const SpmmParams& p, const TileWalk& 
     constexpr int BM = Cfg::BM, BN = Cfg::BN, PITCH = Cfg::STG_PITCH;
     const int S = p.S, N = p.N;
     const char* stg = smem + Cfg::EPI_BASE;
-    // this wave's quarter of the staged tile, 8 pieces of 1 KB (16 bytes per lane).  Transposed output: 32 staging rows
-    // (tile columns), a piece = 4 of them x 256 bytes.  Row-major output: the block of consumer wave `sw`, a piece = one
+    // this wave's quarter of the staged tile, 8 pieces of 1 KB (16 bytes per lane).  Transposed output: BN / 4 staging rows
+    // (tile columns of BM rows), a piece = RPP of them.  Row-major output: the block of consumer wave `sw`, a piece = one
     // slab = 8 rows x 128 bytes, read back row-major with transposing reads.
-    const int srow = sw * 32 + (lane >> 4), chunk = lane & 15;
+    constexpr int LPR = BM * 2 / 16, RPP = 64 / LPR;        // lanes per staging row, staging rows per piece
+    const int srow = sw * (BN / 4) + lane / LPR, chunk = lane % LPR;
     const int li = lane & 15, kb = lane >> 4;
     const int rd_off = (8 * (2 * kb + ((li & 3) >> 1)) + (li >> 2)) * 16 + (li & 1) * 8;
     const int q_lo = 4 * ((li >> 2) & 1) + (li & 3);
-    const int blk_row0 = (sw >> 1) * 64, blk_col = (sw & 1) * 64 + 8 * (2 * kb + (li >> 3));
+    const int blk_row0 = (sw / Cfg::WN) * 64, blk_col = (sw % Cfg::WN) * 64 + 8 * (2 * kb + (li >> 3));
     const int pieces_per_step = S >= 4 ? 2 : (S == 3 ? 3 : 4);
     // (stores through asm statements: a store the compiler knows of would be waited for at the next step barrier, and every
     // wave of the workgroup with it)
@@ -647,7 +651,7 @@ __device__ __forceinline__ void wsw_storer(const SpmmParams& p, const TileWalk& 
     auto load_tile = [&](int tm, int tn) {
         if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) held[i] = *(const u32x4*)(stg + (srow + 4 * i) * PITCH + chunk * 16);
+            for (int i = 0; i < 8; i++) held[i] = *(const u32x4*)(stg + (srow + RPP * i) * PITCH + chunk * 16);
         } else {
 #pragma unroll
             for (int i = 0; i < 8; i++) {
@@ -668,9 +672,8 @@ __device__ __forceinline__ void wsw_storer(const SpmmParams& p, const TileWalk& 
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             if (i >= next_piece && i < next_piece + count) {
-                const int r = srow + 4 * i;         // staging row: a tile row, or (transposed) a tile column
                 if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
-                    const int col = h_tn * BN + r;
+                    const int col = h_tn * BN + srow + RPP * i;         // staging row = tile column
                     if (col < N) store_c16<true>(p.C + (int64_t)col * p.rows + h_tm * BM + chunk * 8, held[i]);
                 } else {
                     const int q = 8 * (i & 1) + q_lo;                  // piece i: slab of mb = i / 2, lane groups 2*(i & 1), + 1
@@ -700,10 +703,10 @@ __device__ __forceinline__ void wsw_storer(const SpmmParams& p, const TileWalk& 
     store_pieces(8);
 }
 
-template <int NS, int NP, int OUT_LAYOUT>
-__global__ __launch_bounds__(768) void spmm_wsw_kernel(SpmmParams p) {
-    using Cfg = WswCfg<NS, NP>;
-    static_assert(NP == 4 && Cfg::THREADS == 768, "wave counts");
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT>
+__global__ __launch_bounds__((8 + NP) * 64) void spmm_wsw_kernel(SpmmParams p) {
+    using Cfg = WswCfg<WM, WN, NS, NP>;
+    static_assert((NP == 2 || NP == 4) && Cfg::THREADS == (8 + NP) * 64, "wave counts");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -717,21 +720,21 @@ __global__ __launch_bounds__(768) void spmm_wsw_kernel(SpmmParams p) {
         const int pr = wave - Cfg::NC;
         if (pr == 0) ws_producer<Cfg, NP, 0, true>(p, walk, smem, smem_base, lane);
         else if (pr == 1) ws_producer<Cfg, NP, 1, true>(p, walk, smem, smem_base, lane);
-        else if (pr == 2) ws_producer<Cfg, NP, 2, true>(p, walk, smem, smem_base, lane);
-        else ws_producer<Cfg, NP, 3, true>(p, walk, smem, smem_base, lane);
+        else if (NP > 2 && pr == 2) ws_producer<Cfg, NP, (NP > 2 ? 2 : 0), true>(p, walk, smem, smem_base, lane);
+        else if (NP > 2) ws_producer<Cfg, NP, (NP > 2 ? 3 : 0), true>(p, walk, smem, smem_base, lane);
     } else {
         wsw_storer<Cfg, OUT_LAYOUT>(p, walk, smem, wave - Cfg::NC - NP, lane);
     }
 }
 
-template <int NS, int NP, int OUT_LAYOUT>
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT>
 static hipError_t launch_wsw(const SpmmParams& p, hipStream_t stream) {
-    using Cfg = WswCfg<NS, NP>;
+    using Cfg = WswCfg<WM, WN, NS, NP>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     if (p.S < 2) return hipErrorInvalidValue;
     static int cus = 0;
-    auto kern = spmm_wsw_kernel<NS, NP, OUT_LAYOUT>;
+    auto kern = spmm_wsw_kernel<WM, WN, NS, NP, OUT_LAYOUT>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -765,7 +768,9 @@ hipError_t launch_warpspec(int variant, int out_layout, const SpmmParams& p, hip
         case SPMM_VARIANT_T128x256_S3:
             return t ? launch_wst<4, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_wst<4, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
         case SPMM_VARIANT_WS128x128_S3:
-            return t ? launch_wsw<3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_wsw<3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
+            return t ? launch_wsw<2, 2, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_wsw<2, 2, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
+        case SPMM_VARIANT_WS64x256_S3:
+            return t ? launch_wsw<1, 4, 3, 2, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_wsw<1, 4, 3, 2, SPATHA_OUT_ROW_MAJOR>(p, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -39,6 +39,8 @@ MEASURED_TRAFFIC = {
         (199_214_000, "profiles/spmm_up_kernel_tile512x128_ffn_up_64-2-8.md"),
     ("smfmac16x16x64_unified_pingpong_densestage_aregs_tile512x128_3stage", 4096, 1024, 16384, 4, 128):
         (323_090_000, "profiles/spmm_up_kernel_tile512x128_ffn_up_2-4.md"),
+    ("smfmac16x16x64_warpspec_storewaves_tile128x128_3stage", 4096, 1024, 16384, 32, 128):
+        (172_585_000, "profiles/spmm_wsw_kernel_tile128x128_ffn_up_128-2-32.md"),
     ("smfmac16x16x64_warpspec_tall_tile128x256_3stage", 49152, 12288, 2048, 16, 128):
         (2_202_100_000, "profiles/spmm_wst_kernel_tile128x256_gpt3_ffn_n2048.md"),
 }

@@ -226,9 +226,13 @@ const Rule kRules[] = {
     {V_64, spatha::SPMM_VARIANT_DS256x128_S3_C8, [](const Shape&) { return true; }},
     // m > 8, row-major, two or three k-steps per tile and six rounds or more of 64 x 256 tiles: the producer/consumer kernel
     // with store waves, 9-10 % ahead of the plain one and of the per-tile pipeline (4096 x 1024 x 16384 at 64:2:32, 3072 x
-    // 768 x 8192 at 64:2:40); level at four rounds, behind with fewer tiles, with four k-steps or more, and with transposed output
+    // 768 x 8192 at 64:2:40); level at four rounds, behind with fewer tiles and with four k-steps or more
     {V_64, spatha::SPMM_VARIANT_WS64x256_S3,
-     [](const Shape& s) { return !s.transposed && s.m > 8 && s.S >= 2 && s.S <= 3 && s.tiles(64, 256) >= 6 * s.cus; }},
+     [](const Shape& s) {
+         // (transposed output, where the store waves also add the bias: ahead from twelve rounds on only - 4096 x 1024 x 16384
+         // at 64:2:32 36.3 against 39.8 us for the per-tile pipeline; at six rounds 17.0 against 15.1 us)
+         return s.m > 8 && s.S >= 2 && s.S <= 3 && s.tiles(64, 256) >= (s.transposed ? 12 : 6) * s.cus;
+     }},
     // m > 8, gathered 64 x 256 tiles.  32 or more k-steps per tile and many rounds: the persistent pipeline, which keeps
     // loading across tile boundaries, leads (GPT-3 layers at 64:2:16; at 64:2:32, 24 k-steps, the per-tile pipeline is
     // 10-20 % ahead); with one tile per CU or less its third stage still gives long k-loops 5-15 %

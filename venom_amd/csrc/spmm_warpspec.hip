@@ -591,19 +591,16 @@ __device__ __forceinline__ void wsw_consumer(const SpmmParams& p, const TileWalk
         // lane (j16, ib) holds column nb*16 + j16, rows ib*16 + mb*4 + 0..3 of the wave's block
         if (p.fuse) fused_bias_act(acc, p.bias, (int64_t)cm0 + wm * 64 + ib * 16, p.act);
         if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
-            // staging [tile column][tile row]: four consecutive rows of one column are 8 contiguous bytes
-            const bool with_bias = !p.fuse && p.bias;
+            // staging [tile column][tile row]: four consecutive rows of one column are 8 contiguous bytes.  (The bias of
+            // this layout is added by the store waves: a load from global memory here would sit in the consumers' path.)
 #pragma unroll
             for (int mb = 0; mb < 4; mb++) {
                 const int row = wm * 64 + ib * 16 + mb * 4;
-                half4_t b4 = {0, 0, 0, 0};
-                if (with_bias) b4 = *(const half4_t*)(p.bias + cm0 + row);
 #pragma unroll
                 for (int nb = 0; nb < 4; nb++) {
                     half4_t h4;
 #pragma unroll
                     for (int r = 0; r < 4; r++) h4[r] = (_Float16)acc[mb][nb][r];
-                    if (with_bias) h4 = h4 + b4;        // fp16 addition on the rounded product
                     *(half4_t*)(stg + (wn * 64 + nb * 16 + j16) * PITCH + row * 2) = h4;
                 }
             }
@@ -650,8 +647,17 @@ __device__ __forceinline__ void wsw_storer(const SpmmParams& p, const TileWalk& 
     int h_tm = 0, h_tn = 0, next_piece = 8;          // tile held in registers; 8 = nothing left to store
     auto load_tile = [&](int tm, int tn) {
         if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
+            // a lane's pieces are eight consecutive rows of several columns: one 16-byte piece of the bias serves them all
+            // (fp16 addition on the rounded product, as everywhere)
+            u32x4 b8 = {0, 0, 0, 0};
+            const bool with_bias = !p.fuse && p.bias;
+            if (with_bias) b8 = *(const u32x4*)(p.bias + tm * BM + chunk * 8);
 #pragma unroll
-            for (int i = 0; i < 8; i++) held[i] = *(const u32x4*)(stg + (srow + RPP * i) * PITCH + chunk * 16);
+            for (int i = 0; i < 8; i++) {
+                u32x4 v = *(const u32x4*)(stg + (srow + RPP * i) * PITCH + chunk * 16);
+                if (with_bias) v = __builtin_bit_cast(u32x4, __builtin_bit_cast(half8_t, v) + __builtin_bit_cast(half8_t, b8));
+                held[i] = v;
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < 8; i++) {

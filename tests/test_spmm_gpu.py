@@ -498,6 +498,29 @@ def test_store_wave_kernel_needs_two_k_steps(gpu):
     assert plan.kernel_name(N, 0, 20) is None and plan.kernel_name(N, 0, 21) is None and plan.kernel_name(N, 0, 6) is not None
 
 
+def test_one_plan_on_two_streams_at_once(gpu):
+    """A plan holds no per-launch state: two streams run it concurrently on their own operands (the plan was created on a
+    third one), every result equal to the oracle."""
+    rows, cols, N, m, v = 1024, 1024, 2048, 8, 64
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=9, integer_values=True)
+    rng = np.random.default_rng(9)
+    Bs = [rng.integers(-4, 5, size=(cols, N)).astype(np.float16) for _ in range(2)]
+    wants = [oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B) for B in Bs]
+    with torch.cuda.stream(torch.cuda.Stream(device=gpu)):
+        plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    dBs = [_dev(B, gpu) for B in Bs]
+    outs = [torch.empty((rows, N), dtype=torch.float16, device=gpu) for _ in range(2)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=gpu) for _ in range(2)]
+    for rep in range(20):
+        for k in range(2):
+            with torch.cuda.stream(streams[k]):
+                plan.run(dBs[k], out=outs[k])
+    torch.cuda.synchronize()
+    for k in range(2):
+        assert np.array_equal(outs[k].cpu().numpy().view(np.uint16), wants[k].view(np.uint16)), k
+
+
 K_TAIL_CASES = [
     # rows, cols, N, m, v : cols % (16 m) != 0, so the last k-step of a dense-staged kernel spans rows beyond K
     (1024, 200, 264, 8, 64),

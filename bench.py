@@ -120,8 +120,8 @@ def main():
                     help="before the warm-up launches, keep launching the kernel for this many milliseconds: the GPU's clock "
                          "needs ~50-100 ms of work to settle, whatever --warmup says (reported as settle_ms, separate from warmup)")
     ap.add_argument("--no-extra", action="store_true",
-                    help="skip the two compute-bound workloads (2:4 FFN-up, GPT-3 FFN at 2048 tokens) that the default run "
-                         "reports under 'extra'")
+                    help="skip the other BASELINE workloads that the default run reports under 'extra' (config 1, the 2:4 "
+                         "baseline, the 18 cells of the sparsity sweep, the GPT-3 FFN matrix at 16 / 256 / 2048 tokens)")
     ap.add_argument("--rows", type=int, default=4096)
     ap.add_argument("--cols", type=int, default=1024)
     ap.add_argument("--n", type=int, default=16384, help="columns of B (tokens)")
@@ -129,12 +129,13 @@ def main():
     ap.add_argument("--v", type=int, default=64)
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--extra", action="store_true", help="also time the other BERT-large layer shapes (appended to 'extra')")
+    ap.add_argument("--extra", action="store_true", help="also time three shapes outside BASELINE.json (appended to 'extra')")
     ap.add_argument("--ablation", action="store_true",
                     help="also time the same matrix with identity column-loc (the reference's IDEAL_KERNEL ablation) and, "
                          "if `python -m venom_amd.build --ablation` has been run, the OUT_32B build (4-byte stores of C)")
-    ap.add_argument("--gpt3", action="store_true",
-                    help="also time the GPT-3 FFN shapes (A 49152x12288 128:2:16, N in 16/256/2048; under 'gpt3')")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="skip the BERT-large encoder (BASELINE config 5: dense against 64:2:8 drop-in layers, under 'e2e'; "
+                         "about a minute, most of it building and converting the model on the host)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="before the benchmark, run 5 plain device copies of 256 MiB (a kernel of known HBM traffic, "
                          "for scaling the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
@@ -158,7 +159,7 @@ def main():
         alt = os.path.join(ROOT, "venom_amd", "lib", "libspatha_out32b.so")
         if os.path.exists(alt):
             import subprocess
-            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu-baseline", "--no-extra", "--steps", str(args.steps),
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu-baseline", "--no-extra", "--no-e2e", "--steps", str(args.steps),
                                 "--warmup", str(args.warmup), "--variant", str(args.variant)],
                                env=dict(os.environ, SPATHA_LIBRARY=alt), stdout=subprocess.PIPE, text=True)
             if r.returncode == 0 and r.stdout.strip():
@@ -179,14 +180,18 @@ def main():
     dev = torch.device("cuda:0")
     L = _lib.lib()
 
-    def prepare(rows, cols, N, m, v, seed=0):
-        vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=seed, value_std=0.02)
+    def prepare(rows, cols, N, m, v, seed=0, value_std=0.02, b_uniform=False):
+        """Seeded synthetic operands: A's non-zeros ~ N(0, value_std); B ~ N(0, 1), or U(-1, 1) with b_uniform."""
+        vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=seed, value_std=value_std)
         g = F.geometry(rows, cols, 2, m, v)
         plan = spatha.SpmmPlan(torch.from_numpy(vals).to(dev), torch.from_numpy(meta.view(np.int32)).to(dev),
                                torch.from_numpy(columns.view(np.int32)).to(dev), rows, cols, 2, m, v)
         gen = torch.Generator(device=dev)
         gen.manual_seed(seed)
-        B = torch.randn((cols, N), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+        if b_uniform:
+            B = (torch.rand((cols, N), generator=gen, device=dev, dtype=torch.float32) * 2 - 1).to(torch.float16)
+        else:
+            B = torch.randn((cols, N), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
         C = torch.empty((rows, N), dtype=torch.float16, device=dev)
         return dict(vals=vals, meta=meta, columns=columns, geo=g, plan=plan, B=B, C=C)
 
@@ -331,39 +336,91 @@ def main():
                                             "pct_smfmac_peak": round(100 * flops / us_c * 1e-6 / SMFMAC_PEAK_TFLOPS, 1)})
         out["calibration"] = calib
 
-    def side_figures(r2, c2, n2, m2, v2, w2, k2):
+    def side_figures(r2, c2, n2, m2, v2, w2, k2, config):
         by = algorithmic_bytes(r2, c2, n2, m2, v2, w2["geo"].ksp)
         fl = 2.0 * r2 * n2 * 2 * w2["geo"].ksp
         t_hbm, t_mma = by / (HBM_PEAK_GBS * 1e9), fl / (SMFMAC_PEAK_TFLOPS * 1e12)
         tr, src = MEASURED_TRAFFIC.get((w2["plan"].kernel_name(n2, 0, 0), r2, c2, n2, m2, v2), (None, None))
-        return {"shape": "%dx%dx%d %d:2:%d" % (r2, c2, n2, v2, m2), "kernel": w2["plan"].kernel_name(n2, 0, 0),
+        return {"config": config, "shape": "%dx%dx%d %d:2:%d" % (r2, c2, n2, v2, m2), "kernel": w2["plan"].kernel_name(n2, 0, 0),
                 "algorithmic_bytes": by, "traffic": tr, "traffic_source": src,
                 "us": round(k2 * 1e3, 2), "dense_equiv_tflops": round(2.0 * r2 * c2 * n2 / (k2 * 1e-3) / 1e12, 1),
                 "hbm_gbs": round(by / (k2 * 1e-3) / 1e9, 1), "hbm_frac": round(by / (k2 * 1e-3) / 1e9 / HBM_PEAK_GBS, 3),
                 "pct_smfmac_peak": round(100 * fl / (k2 * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2),
-                "bound": "mfma" if t_mma > t_hbm else "hbm"}
+                "bound": "mfma" if t_mma > t_hbm else "hbm",
+                "frac_of_bound": round(max(t_hbm, t_mma) / (k2 * 1e-3), 3)}
+
+    def power_of(w2, n2, us_guess, seconds=1.5):
+        """Socket power and clock under a sustained run of this workload (the compute-bound ones sit at the power limit)."""
+        if idle is None:
+            return None
+        sp2 = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        plan2, B2, C2 = w2["plan"], w2["B"], w2["C"]
+        us_s, watts, mhz, n_s = sustained(
+            lambda: _lib.check(L.spatha_spmm_run(plan2._handle, B2.data_ptr(), n2, None, C2.data_ptr(), 0, 0, sp2), "run"),
+            torch.cuda.synchronize, us_guess, seconds)
+        return {"socket_w": None if watts is None else round(watts, 1), "gfx_mhz": None if mhz is None else round(mhz, 1),
+                "us_sustained": round(us_s, 2), "samples": n_s}
 
     if not args.no_extra:
-        # the two compute-bound workloads, so that the default line carries them: the 2:4 baseline on the FFN-up shape and
-        # the GPT-3 feed-forward matrix at 2048 tokens (each: 100 ms settle, 10 warm-up, 30 timed launches)
+        # Every other workload BASELINE.json names, so that one default run carries them all (each: 100 ms settle, 10 warm-up,
+        # 30 timed launches, HIP events): config 1 (the reference README's --check case with its own data), config 2 (2:4 on
+        # the FFN-up shape), the 18 cells of config 3's sweep, config 4's three token counts.
         extra = []
-        for (r2, c2, n2, m2, v2) in [(4096, 1024, 16384, 4, 128), (49152, 12288, 2048, 16, 128)]:
-            w2 = prepare(r2, c2, n2, m2, v2)
+        w2 = prepare(1024, 4096, 4096, 8, 128, value_std=1.0, b_uniform=True)
+        _, k2 = timed(w2, 100, 20, settle_ms=100.0)
+        e = side_figures(1024, 4096, 4096, 8, 128, w2, k2, "1: reference README case, A ~N(0,1), B ~U(-1,1)")
+        e["vs_published_rtx3090_209.9us"] = round(209.9 / (k2 * 1e3), 2)
+        extra.append(e)
+        del w2
+        w2 = prepare(4096, 1024, 16384, 4, 128)
+        _, k2 = timed(w2, 30, 10, settle_ms=100.0)
+        e = side_figures(4096, 1024, 16384, 4, 128, w2, k2, "2: plain 2:4 on the FFN-up shape")
+        e["power"] = power_of(w2, 16384, k2 * 1e3)
+        extra.append(e)
+        del w2
+        for (r2, c2) in ((1024, 1024), (4096, 1024), (1024, 4096)):
+            for v2 in (64, 128):
+                for m2 in (8, 16, 32):
+                    if (r2, c2, m2, v2) == (rows, cols, m, v) and N == 16384 and args.variant == 0:
+                        w2, k2 = w, ms_kernel               # the headline cell: measured above
+                    else:
+                        w2 = prepare(r2, c2, 16384, m2, v2)
+                        _, k2 = timed(w2, 30, 10, settle_ms=100.0)
+                    extra.append(side_figures(r2, c2, 16384, m2, v2, w2, k2, "3: sparsity sweep"))
+                    w2 = None
+        r2, c2, m2, v2 = 49152, 12288, 16, 128
+        w2 = prepare(r2, c2, 16, m2, v2)
+        for n2 in (16, 256, 2048):
+            gen = torch.Generator(device=dev)
+            gen.manual_seed(0)
+            w2["B"] = torch.randn((c2, n2), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+            w2["C"] = torch.empty((r2, n2), dtype=torch.float16, device=dev)
             _, k2 = timed(w2, 30, 10, settle_ms=100.0)
-            extra.append(side_figures(r2, c2, n2, m2, v2, w2, k2))
-            del w2
+            e = side_figures(r2, c2, n2, m2, v2, w2, k2, "4: GPT-3 FFN matrix, %d tokens" % n2)
+            if n2 == 2048:
+                e["power"] = power_of(w2, n2, k2 * 1e3)
+            extra.append(e)
+        del w2
         out["extra"] = extra
 
     if args.extra:
         extra = out.get("extra", [])
-        for (r2, c2, n2, m2, v2) in [(1024, 4096, 16384, 8, 64), (1024, 1024, 16384, 8, 64), (4096, 1024, 16384, 8, 128),
-                                     (1024, 4096, 4096, 8, 128), (4096, 1024, 16384, 4, 64),
-                                     (4096, 1024, 16384, 16, 64), (4096, 1024, 16384, 32, 64)]:
+        for (r2, c2, n2, m2, v2) in [(1024, 4096, 4096, 8, 64), (4096, 1024, 16384, 4, 64), (1024, 4096, 4096, 8, 32)]:
             w2 = prepare(r2, c2, n2, m2, v2)
             _, k2 = timed(w2, 100, 20, settle_ms=100.0)
-            extra.append(side_figures(r2, c2, n2, m2, v2, w2, k2))
+            extra.append(side_figures(r2, c2, n2, m2, v2, w2, k2, "other"))
             del w2
         out["extra"] = extra
+
+    if not args.no_e2e:
+        # config 5: the BERT-large encoder, batch 32 x 512 tokens, every encoder Linear in 64:2:8 through the operator
+        # (drop-in layers), against the same model on dense fp16 weights (hipBLASLt through torch)
+        from venom_amd import bert
+        torch.cuda.empty_cache()
+        t_e2e = time.perf_counter()
+        out["e2e"] = dict(bert.measure(n=2, m=8, v=64, repeats=10, warmups=3),
+                          config="5: BERT-large encoder, 24 layers, batch 32 x seq 512, random-init weights, 64:2:8 drop-in layers")
+        out["e2e"]["wall_s_incl_model_build"] = round(time.perf_counter() - t_e2e, 1)
 
     if args.ablation:
         # the reference's IDEAL_KERNEL switch (CMakeLists.txt:25-33, blockwise_kernel.h): column-loc ignored, i.e. the
@@ -376,20 +433,6 @@ def main():
         _, k_nm = timed(w, args.steps, args.warmup, args.variant)
         out["ablation"] = {"column_loc_us": round(k_nm * 1e3, 2), "ideal_identity_column_loc_us": round(k_id * 1e3, 2),
                            "out_32b_stores_us": out32}      # null: libspatha_out32b.so has not been built
-
-    if args.gpt3:
-        r2, c2, m2, v2 = 49152, 12288, 16, 128
-        w2 = prepare(r2, c2, 16, m2, v2)
-        gpt3 = []
-        for n2 in (16, 256, 2048):
-            gen = torch.Generator(device=dev)
-            gen.manual_seed(0)
-            w2["B"] = torch.randn((c2, n2), generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
-            w2["C"] = torch.empty((r2, n2), dtype=torch.float16, device=dev)
-            _, k2 = timed(w2, 50, 20, settle_ms=100.0)
-            gpt3.append(side_figures(r2, c2, n2, m2, v2, w2, k2))
-        del w2
-        out["gpt3"] = gpt3
 
     if not args.no_cpu_baseline:
         import oracle
@@ -416,8 +459,13 @@ def main():
         oracle.encode(dense, w["columns"], 2, m, v)
         t_fmt = time.perf_counter() - t0
         got = w["C"].cpu().numpy()
-        err = float(np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64)) /
-                           np.maximum(np.abs(ref.astype(np.float64)), 1.0)))
+        # |got - ref| / max(|ref|, rms(ref) / 16): relative to the entry unless it is far below the result's typical size
+        err, same = 0.0, 0
+        floor = max(float(np.sqrt(np.mean(ref[:256].astype(np.float64) ** 2))) / 16.0, 2.0 ** -14)
+        for r0 in range(0, rows, 512):
+            g64, r64 = got[r0:r0 + 512].astype(np.float64), ref[r0:r0 + 512].astype(np.float64)
+            err = max(err, float(np.max(np.abs(g64 - r64) / np.maximum(np.abs(r64), floor))))
+            same += int(np.count_nonzero(got[r0:r0 + 512].view(np.uint16) == ref[r0:r0 + 512].view(np.uint16)))
         out["cpu_baseline"] = {
             "value": round(flops_dense / t_spmm / 1e12, 5),
             "unit": "TFLOPS (dense-equivalent)",
@@ -425,8 +473,8 @@ def main():
             "kind": "port",
             "sample": "oracle SpMM (compressed form, fp32 accumulate, OpenMP, %d threads) on the whole workload, mean of %d runs: "
                       "%.3f s per SpMM; 1 thread (timed on %d of %d columns, scaled): %.2f s; host format decode+encode of A, "
-                      "1 thread: %.3f s; max rel err GPU vs oracle over all of C: %.2e"
-                      % (threads, reps, t_spmm, n1, N, t_one, t_fmt, err),
+                      "1 thread: %.3f s; GPU vs oracle over all of C: max rel err %.2e (|d| / max(|ref|, rms/16)), %.4f of the "
+                      "entries bit-identical" % (threads, reps, t_spmm, n1, N, t_one, t_fmt, err, same / float(rows * N)),
         }
     print(json.dumps(out))
 

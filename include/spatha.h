@@ -72,6 +72,15 @@ int spatha_vnm_random_pattern(int rows, int cols, int n, int m, int v, uint32_t*
  * benchmark (src/format/format_sr_nm.cpp:64-68, src/util/matrix_utils.h:88-97). */
 int spatha_fill_rand_small_ints_f16(uint16_t* out, int64_t count);
 
+/* The inputs of one `benchmark_spmm --sparsity-type n-to-m` run, drawn from
+ * rand() in the reference's order: the cols x ncols_b entries of B first
+ * (Dataset's n:m constructor, src/dataset/dataset.cpp:70-90, fills B before it
+ * initialises the format), then the pattern (src/format/format_sr_nm.cpp:62),
+ * then the rows x ksp stored values of A in storage order (:64-68).
+ * metadata / columns must be zero-filled (n_metadata / n_columns words). */
+int spatha_benchmark_inputs_f16(int rows, int cols, int ncols_b, int n, int m, int v, uint16_t* b, uint32_t* metadata,
+                                uint32_t* columns, uint16_t* values);
+
 /* Dense -> V:N:M.  dense is row-major rows x cols; columns holds, per V-row
  * block and per m-column group, the 4 selected column offsets (ascending).
  * mask == NULL: an entry is kept when it is non-zero
@@ -191,7 +200,10 @@ int spatha_spmm_run_fused(const spatha_spmm_plan* plan, const uint16_t* B_dev, i
  * frees nothing: it launches the pack kernels and the SpMM kernel on `stream`.  A matrix whose derived copies exceed
  * the array is refused with SPATHA_ERR_TOO_LARGE (the array holds e.g. 4096 x 1024 or 1024 x 4096 at 2:8 and
  * 4096 x 1024 at 2:4).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two
- * streams, two threads) race; calls ordered on one stream do not. */
+ * streams, two threads) race; calls ordered on one stream do not.  Every argument check and the kernel choice happen
+ * before the first launch, so a refused call has not touched the array.  The first call on a device looks up the
+ * array's address and sets kernel attributes, which a stream capture cannot hold: make one call outside the capture
+ * (any shape that reaches the same kernel) before recording calls into a graph. */
 int spatha_spmm_run_noalloc(int rows, int cols, int n, int m, int v, const uint16_t* values_dev,
                             const uint32_t* metadata_dev, const uint32_t* columns_dev, const uint16_t* B_dev, int N,
                             const uint16_t* bias_dev, uint16_t* out_dev, int out_layout, void* stream);

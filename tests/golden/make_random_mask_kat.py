@@ -14,7 +14,12 @@ the reference's order:
 
 Both arrays persist across draws (they are never reset), which is what makes the stream order observable.
 
-    python tests/golden/make_random_mask_kat.py      # rewrites tests/golden/random_mask_kat.json
+A second file pins the benchmark's fills and the order in which one `benchmark_spmm --sparsity-type n-to-m` run consumes
+the stream: the K x N entries of B first (src/dataset/dataset.cpp:81 -> src/util/matrix_utils.h:88-97), then the pattern
+(src/format/format_sr_nm.cpp:62), then the rows x Ksp stored values of A in storage order (:64-68); every fill entry is
+`rand() % 9 - 4` (C's remainder of a non-negative int, so Python's % agrees).
+
+    python tests/golden/make_random_mask_kat.py      # rewrites tests/golden/random_mask_kat.json and benchmark_draw_order_kat.json
 """
 import json
 import os
@@ -112,7 +117,31 @@ CASES = [
 ]
 
 
+def fill_small_ints(count, stream):
+    return [stream.rand() % 9 - 4 for _ in range(count)]
+
+
+def benchmark_inputs(rows, cols, ncolsB, m, v, stream):
+    """What one run of the reference benchmark draws, in its order: B, pattern, values of A."""
+    B = fill_small_ints(cols * ncolsB, stream)
+    meta, columns = random_mask(rows, cols, m, v, stream)
+    ksp = round_up(-(-cols // m) * 2, 16)
+    values = fill_small_ints(rows * ksp, stream)
+    return dict(rows=rows, cols=cols, ncolsB=ncolsB, m=m, v=v, B=B, metadata=meta, columns=columns, values=values,
+                draws=stream.pos)
+
+
 def main():
+    here = os.path.dirname(os.path.abspath(__file__))
+    d = Stream(1)
+    head = fill_small_ints(6, d)
+    assert head == [-3, 3, -4, 3, 1, 3]       # 1804289383 % 9 - 4, 846930886 % 9 - 4, ...: worked by hand from the stream's head
+    d = Stream(1)
+    runs = [benchmark_inputs(32, 32, 8, 8, 32, d),      # 256 draws for B, 32 words x 8 x 3, 8 groups x 7, 512 values
+            benchmark_inputs(64, 44, 16, 8, 32, d)]     # a second run of the same process: K % m != 0, two V blocks
+    with open(os.path.join(here, "benchmark_draw_order_kat.json"), "w") as f:
+        json.dump(dict(fill_head=head, runs=runs), f, separators=(",", ":"))
+    print("wrote benchmark_draw_order_kat.json", [r["draws"] for r in runs])
     s = Stream(1)
     assert s.values[:4] == [1804289383, 846930886, 1681692777, 1714636915]      # the published head of glibc's stream
     out = []

@@ -9,6 +9,26 @@ import numpy as np
 GOLDEN_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 
+def rel_err(got, exact):
+    """max |got - exact| / max(|exact|, rms(exact) / 16): a true relative error wherever an entry is not far below the
+    typical magnitude of the result (there the error of an fp32-accumulated sum is absolute by nature), so the 1e-2
+    bound means the same on outputs of magnitude 0.3 as on outputs of magnitude 30."""
+    got = np.asarray(got, dtype=np.float64)
+    exact = np.asarray(exact, dtype=np.float64)
+    floor = max(float(np.sqrt(np.mean(exact * exact))) / 16.0, 2.0 ** -14)
+    return float((np.abs(got - exact) / np.maximum(np.abs(exact), floor)).max())
+
+
+def fp16_steps(got, exact):
+    """max |got - exact| in units of the fp16 spacing at max(|exact|, rms(exact) / 16) (0.5 = correctly rounded wherever
+    the entry is not far below the result's typical magnitude)."""
+    got = np.asarray(got, dtype=np.float64)
+    exact = np.asarray(exact, dtype=np.float64)
+    floor = max(float(np.sqrt(np.mean(exact * exact))) / 16.0, 2.0 ** -14)
+    spacing = np.spacing(np.maximum(np.abs(exact), floor).astype(np.float16)).astype(np.float64)
+    return float((np.abs(got - exact) / spacing).max())
+
+
 def golden_cases():
     return sorted(glob.glob(os.path.join(GOLDEN_DIR, "vnm_*.npz")))
 

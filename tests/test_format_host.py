@@ -140,6 +140,50 @@ def test_random_pattern_known_answers():
         assert np.array_equal(columns, np.array(c["columns"], np.uint32)), (c["rows"], c["cols"])
 
 
+def _golden_json(name):
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name)) as f:
+        return json.load(f)
+
+
+def test_small_int_fill_known_answers():
+    """`rand() % 9 - 4` after srand(1): glibc's stream starts 1804289383, 846930886, 1681692777, 1714636915, 1957747793,
+    424238335, i.e. -3, 3, -4, 3, 1, 3 (reference fill: src/format/format_sr_nm.cpp:64-68, src/util/matrix_utils.h:88-97).
+    Literals, not a second evaluation of the formula."""
+    want = [-3.0, 3.0, -4.0, 3.0, 1.0, 3.0]
+    assert _golden_json("benchmark_draw_order_kat.json")["fill_head"] == want
+    oracle.srand(1)
+    assert oracle.fill_rand_ints(6).tolist() == want
+    oracle.srand(1)
+    got = F.fill_rand_small_ints(6)
+    assert got.dtype == np.float16 and got.astype(np.float32).tolist() == want
+    assert got.view(np.uint16).tolist() == [0xC200, 0x4200, 0xC400, 0x4200, 0x3C00, 0x4200]
+
+
+def test_benchmark_draw_order_known_answers():
+    """One benchmark run consumes rand() as B, then pattern, then values (src/dataset/dataset.cpp:70-90,
+    src/format/format_sr_nm.cpp:62-68).  The driver draws through spatha_benchmark_inputs_f16; its output is held against
+    a pure-Python walk of glibc's stream (tests/golden/make_random_mask_kat.py), two runs of one process in a row."""
+    kat = _golden_json("benchmark_draw_order_kat.json")
+    first = kat["runs"][0]
+    assert first["B"][:3] == [-3, 3, -4] and first["draws"] == 256 + 16 * 8 * 3 + 4 * 7 + 32 * 16
+    oracle.srand(1)
+    for c in kat["runs"]:
+        B, meta, columns, vals = F.benchmark_inputs(c["rows"], c["cols"], c["ncolsB"], 2, c["m"], c["v"])
+        assert B.astype(np.int64).reshape(-1).tolist() == c["B"]
+        assert meta.tolist() == c["metadata"] and columns.tolist() == c["columns"]
+        assert vals.astype(np.int64).tolist() == c["values"]
+    # the oracle's pieces called in that order agree as well
+    oracle.srand(1)
+    for c in kat["runs"]:
+        oB = oracle.fill_rand_ints(c["cols"] * c["ncolsB"])
+        ometa, ocols = oracle.random_mask(c["rows"], c["cols"], 2, c["m"], c["v"])
+        ovals = oracle.fill_rand_ints(len(c["values"]))
+        assert oB.tolist() == c["B"] and ometa.tolist() == c["metadata"] and ocols.tolist() == c["columns"]
+        assert ovals.tolist() == c["values"]
+
+
 def test_meta_blob_layout():
     meta = np.arange(1, 12, dtype=np.uint32)          # 11 words -> column-loc starts at word 16
     columns = np.arange(100, 105, dtype=np.uint32)

@@ -35,6 +35,7 @@ SIGNATURES = {
     "spatha_vnm_geometry_init": (c_int, [c_int, c_int, c_int, c_int, c_int, POINTER(Geometry)]),
     "spatha_vnm_random_pattern": (c_int, [c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "spatha_fill_rand_small_ints_f16": (c_int, [c_void_p, c_int64]),
+    "spatha_benchmark_inputs_f16": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "spatha_vnm_encode_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int]),
     "spatha_vnm_encode_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int]),
     "spatha_vnm_decode_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int]),

@@ -291,35 +291,59 @@ def main(argv=None):
                     help="with --fuse-ffn: GELU in the kernel's write-out too (default: torch's elementwise pass over the "
                          "feature-major buffer, which keeps the model's output bit-identical to the unfused layers)")
     args = ap.parse_args(argv)
-    torch.set_grad_enabled(False)
-    dev = torch.device("cuda:0")
-    dense_model = build_bert_large(args.layers).to(dev).half()
-    sparse_model = build_bert_large(args.layers)
-    sparse_model = linear_to_spmm(sparse_model.to(dev).half(), args.n, args.m, args.v, args.magnitude)
-    if args.fuse_ffn:
-        fuse_feed_forward(sparse_model, activation_in_kernel=args.kernel_gelu)
-    if args.merge_qkv:
-        merge_qkv(sparse_model)
-    if args.fuse_ln:
-        fuse_add_layernorm(dense_model)
-        fuse_add_layernorm(sparse_model)
-    ids = torch.randint(0, 30522, (args.batch, args.seq), device=dev)
-
-    def run(model):
-        out = model(ids).last_hidden_state
-        torch.cuda.synchronize()
-        return out
-
-    run(sparse_model)
-    timeit.repeat(lambda: run(dense_model), repeat=5, number=1)
-    t_dense = report_time("dense", timeit.repeat(lambda: run(dense_model), repeat=args.repeats, number=1), 1, args.n, args.m, args.v)
-    timeit.repeat(lambda: run(sparse_model), repeat=5, number=1)
-    t_sparse = report_time("n:m", timeit.repeat(lambda: run(sparse_model), repeat=args.repeats, number=1), 1, args.n, args.m, args.v)
-    print("# dense %.2f ms, %d:%d:%d%s %.2f ms, speed-up %.2fx" % (t_dense, args.v, args.n, args.m,
+    r = measure(args.n, args.m, args.v, layers=args.layers, batch=args.batch, seq=args.seq, repeats=args.repeats,
+                magnitude=args.magnitude, fuse_ffn=args.fuse_ffn, merge=args.merge_qkv, fuse_ln=args.fuse_ln,
+                kernel_gelu=args.kernel_gelu, report=True)
+    print("# dense %.2f ms, %d:%d:%d%s %.2f ms, speed-up %.2fx" % (r["dense_ms"], args.v, args.n, args.m,
                                                                     ((" (fused feed-forward%s)" % (", activation in the kernel" if args.kernel_gelu else "")) if args.fuse_ffn else "")
                                                                     + (" (merged q/k/v)" if args.merge_qkv else "")
-                                                                    + (" (fused add + LayerNorm in both)" if args.fuse_ln else ""), t_sparse,
-                                                                    t_dense / t_sparse))
+                                                                    + (" (fused add + LayerNorm in both)" if args.fuse_ln else ""), r["vnm_ms"],
+                                                                    r["speedup"]))
+
+
+def measure(n=2, m=8, v=64, layers=24, batch=32, seq=512, repeats=30, warmups=5, magnitude=False, fuse_ffn=False, merge=False,
+            fuse_ln=False, kernel_gelu=False, report=False):
+    """Times the dense fp16 encoder and the same encoder with its Linears in V:N:M on cuda:0 (the reference's procedure,
+    end2end/bert_pytorch.py:211-219: warm-ups, then `repeats` forward passes timed one by one, each ended by a device
+    synchronisation); returns mean and median milliseconds of both and their ratio."""
+    import copy
+
+    prev_grad = torch.is_grad_enabled()
+    torch.set_grad_enabled(False)
+    try:
+        dev = torch.device("cuda:0")
+        base = build_bert_large(layers)
+        dense_model = copy.deepcopy(base).to(dev).half()
+        sparse_model = linear_to_spmm(base.to(dev).half(), n, m, v, magnitude)
+        if fuse_ffn:
+            fuse_feed_forward(sparse_model, activation_in_kernel=kernel_gelu)
+        if merge:
+            merge_qkv(sparse_model)
+        if fuse_ln:
+            fuse_add_layernorm(dense_model)
+            fuse_add_layernorm(sparse_model)
+        ids = torch.randint(0, 30522, (batch, seq), device=dev)
+
+        def run(model):
+            out = model(ids).last_hidden_state
+            torch.cuda.synchronize()
+            return out
+
+        run(sparse_model)
+        timeit.repeat(lambda: run(dense_model), repeat=warmups, number=1)
+        d = [t * 1e3 for t in timeit.repeat(lambda: run(dense_model), repeat=repeats, number=1)]
+        timeit.repeat(lambda: run(sparse_model), repeat=warmups, number=1)
+        s = [t * 1e3 for t in timeit.repeat(lambda: run(sparse_model), repeat=repeats, number=1)]
+        if report:
+            report_time("dense", [t / 1e3 for t in d], 1, n, m, v)
+            report_time("n:m", [t / 1e3 for t in s], 1, n, m, v)
+        spatha.clear_plan_cache()
+        return {"dense_ms": round(statistics.mean(d), 3), "vnm_ms": round(statistics.mean(s), 3),
+                "dense_median_ms": round(statistics.median(d), 3), "vnm_median_ms": round(statistics.median(s), 3),
+                "speedup": round(statistics.mean(d) / statistics.mean(s), 3), "repeats": repeats,
+                "format": "%d:%d:%d" % (v, n, m), "layers": layers, "tokens": batch * seq}
+    finally:
+        torch.set_grad_enabled(prev_grad)
 
 
 if __name__ == "__main__":

@@ -166,9 +166,7 @@ int main(int argc, const char** argv) {
     // ---- inputs, in the reference's drawing order: B, pattern, values
     std::vector<uint16_t> hB((size_t)k * n), hVal((size_t)geo.n_values);
     std::vector<uint32_t> hMeta((size_t)geo.n_metadata, 0u), hCols((size_t)geo.n_columns, 0u);
-    SPATHA_OK_OR_DIE(spatha_fill_rand_small_ints_f16(hB.data(), (int64_t)hB.size()));
-    SPATHA_OK_OR_DIE(spatha_vnm_random_pattern(m, k, nn_row, mm_row, V, hMeta.data(), hCols.data()));
-    SPATHA_OK_OR_DIE(spatha_fill_rand_small_ints_f16(hVal.data(), (int64_t)hVal.size()));
+    SPATHA_OK_OR_DIE(spatha_benchmark_inputs_f16(m, k, n, nn_row, mm_row, V, hB.data(), hMeta.data(), hCols.data(), hVal.data()));
     // --path_to_dset (parsed and ignored by the reference, src/util/argparse.h:123-126): the encoded A is read
     // from that container when it exists (its shape must match the flags), and written there otherwise
     if (!path_to_dset.empty()) {

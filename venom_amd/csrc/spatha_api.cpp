@@ -32,7 +32,7 @@ bool variant_has_fused_writeout(int variant) {
         case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x256_S3: case SPMM_VARIANT_W64x256_S3:
         case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DSH256x128_S3_C8:
         case SPMM_VARIANT_UP512x128_S3: case SPMM_VARIANT_DU512x128_M16: case SPMM_VARIANT_WS128x128_S3:
-        case SPMM_VARIANT_WS64x256_S3:
+        case SPMM_VARIANT_WS64x256_S3: case SPMM_VARIANT_H64x256_S2: case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2:
             return true;
         default:
             return false;
@@ -356,6 +356,18 @@ int spatha_fill_rand_small_ints_f16(uint16_t* out, int64_t count) {
     return SPATHA_OK;
 }
 
+int spatha_benchmark_inputs_f16(int rows, int cols, int ncols_b, int n, int m, int v, uint16_t* b, uint32_t* metadata,
+                                uint32_t* columns, uint16_t* values) {
+    spatha_vnm_geometry geo;
+    int st = spatha::geometry_init(rows, cols, n, m, v, &geo);
+    if (st != SPATHA_OK) return st;
+    if (!b || !metadata || !columns || !values || ncols_b <= 0) return SPATHA_ERR_BAD_ARGUMENT;
+    st = spatha_fill_rand_small_ints_f16(b, (int64_t)cols * ncols_b);
+    if (st == SPATHA_OK) st = spatha::random_pattern(rows, cols, n, m, v, metadata, columns);
+    if (st == SPATHA_OK) st = spatha_fill_rand_small_ints_f16(values, geo.n_values);
+    return st;
+}
+
 int spatha_vnm_encode_f32(const float* dense, const int32_t* mask, const uint32_t* columns, int rows, int cols, int n,
                           int m, int v, float* values, uint32_t* metadata, int threads) {
     return spatha::encode_f32(dense, mask, columns, rows, cols, n, m, v, values, metadata, threads);
@@ -487,8 +499,9 @@ int spatha_spmm_plan_destroy(spatha_spmm_plan* plan) {
 
 }  // extern "C"
 
-int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, uint16_t* out_dev,
-                     int out_layout, int activation, bool fused_entry, int variant, void* stream) {
+int spatha::plan_run_check(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
+                           const uint16_t* out_dev, int out_layout, int activation, bool fused_entry, int variant,
+                           int* chosen) {
     if (!plan || !B_dev || !out_dev || N <= 0) return SPATHA_ERR_BAD_ARGUMENT;
     if (out_layout != SPATHA_OUT_ROW_MAJOR && out_layout != SPATHA_OUT_TRANSPOSED) return SPATHA_ERR_BAD_ARGUMENT;
     if (!fused_entry && out_layout == SPATHA_OUT_ROW_MAJOR && bias_dev) return SPATHA_ERR_BAD_ARGUMENT;
@@ -500,8 +513,18 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
     if (hipGetDevice(&dev) != hipSuccess || dev != plan->device) return SPATHA_ERR_BAD_ARGUMENT;   // plans live on one device
     // the bias of the transposed layout alone stays in the write-out itself
     const bool fuse = activation != SPATHA_ACT_NONE || (out_layout == SPATHA_OUT_ROW_MAJOR && bias_dev);
-    int var = pick_variant(plan, N, variant, fuse, out_layout);
+    const int var = pick_variant(plan, N, variant, fuse, out_layout);
     if (var < 0) return SPATHA_ERR_UNSUPPORTED;
+    if (chosen) *chosen = var;
+    return SPATHA_OK;
+}
+
+int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, uint16_t* out_dev,
+                     int out_layout, int activation, bool fused_entry, int variant, void* stream) {
+    int var = -1;
+    const int status = plan_run_check(plan, B_dev, N, bias_dev, out_dev, out_layout, activation, fused_entry, variant, &var);
+    if (status != SPATHA_OK) return status;
+    const bool fuse = activation != SPATHA_ACT_NONE || (out_layout == SPATHA_OUT_ROW_MAJOR && bias_dev);
     spatha::SpmmParams p;
     p.apack = plan->apack; p.rowtab = plan->rowtab;
     p.B = B_dev; p.bias = bias_dev; p.C = out_dev; p.zeros = plan->zeros; p.gtab = plan->gtab;
@@ -514,6 +537,7 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
     p.apack_bytes = (uint32_t)plan->apack_bytes;
     p.rowtab_bytes = (uint32_t)plan->rowtab_bytes;
     p.fuse = fuse ? 1 : 0; p.act = activation;
+    p.cus = plan->cus > 0 ? plan->cus : 256;
     p.debug = 0; p.skew = 0; p.prof = nullptr;
 #ifdef SPATHA_DEV_PROFILE
     // development builds only: switch parts of a kernel off for time accounting (results are then wrong on purpose)

@@ -34,6 +34,10 @@ void plan_layout(int rows, int m, int v, int ksp, PlanLayout* out);
 hipError_t plan_pack(const spatha_spmm_plan* plan, const uint16_t* values_dev, const uint32_t* metadata_dev,
                      const uint32_t* columns_dev, hipStream_t stream);
 
+// the argument checks and the kernel choice of plan_run alone: nothing is launched; *chosen (may be null) gets the kernel id
+int plan_run_check(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, const uint16_t* out_dev,
+                   int out_layout, int activation, bool fused_entry, int variant, int* chosen);
+
 // argument checks, kernel choice and launch shared by every run entry point; returns a spatha_status
 int plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, uint16_t* out_dev,
              int out_layout, int activation, bool fused_entry, int variant, void* stream);

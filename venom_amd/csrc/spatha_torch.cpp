@@ -6,7 +6,12 @@
 //
 // The reference packs nothing per call (its kernel reads the canonical arrays); here the derived operand copies live
 // in a plan, so the extension keeps a cache of plans keyed by the identity and version of the three weight tensors.
-// An entry holds the tensors, so an address cannot be recycled under a stale plan.
+// An entry holds the tensors, so an address cannot be recycled under a stale plan.  A plan is held through a shared_ptr whose
+// deleter destroys it: a launch keeps its own reference, so an eviction or clear_plan_cache() from another thread cannot
+// free the plan's device buffers under a launch that is being enqueued.  An in-place update of the weights bumps the tensors'
+// version: the miss that follows drops the entries of the same three addresses with an older version, so a loop that
+// re-sparsifies in place keeps one plan per matrix.  A write that torch does not see (through `.data` or a raw pointer)
+// leaves the version alone: call invalidate_plans(values) or clear_plan_cache() after one.
 
 #include <torch/extension.h>
 
@@ -14,6 +19,7 @@
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 
 #include <list>
+#include <memory>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -48,7 +54,7 @@ struct PlanKeyHash {
 };
 struct PlanEntry {
     PlanKey key;
-    spatha_spmm_plan* plan;
+    std::shared_ptr<spatha_spmm_plan> plan;
     torch::Tensor values, metadata, columns;      // kept alive for the plan's lifetime
 };
 
@@ -71,7 +77,24 @@ void check_weight(const torch::Tensor& t, c10::ScalarType a, c10::ScalarType b, 
 
 uint32_t version_of(const torch::Tensor& t) { return (uint32_t)t.unsafeGetTensorImpl()->version_counter().current_version(); }
 
-spatha_spmm_plan* plan_for(const torch::Tensor& values, const torch::Tensor& metadata, const torch::Tensor& columns, int rows,
+bool same_storage(const PlanKey& a, const PlanKey& b) {
+    return a.values == b.values && a.metadata == b.metadata && a.columns == b.columns && a.device == b.device;
+}
+
+// (g_lock held) drops every entry for which `stale` holds; launches that still hold a reference keep their plan alive
+template <class Pred>
+void drop_entries(Pred stale) {
+    for (auto it = g_lru.begin(); it != g_lru.end();) {
+        if (stale(*it)) {
+            g_index.erase(it->key);
+            it = g_lru.erase(it);
+        } else {
+            ++it;
+        }
+    }
+}
+
+std::shared_ptr<spatha_spmm_plan> plan_for(const torch::Tensor& values, const torch::Tensor& metadata, const torch::Tensor& columns, int rows,
                            int cols, int n, int m, int v, hipStream_t stream) {
     PlanKey key{values.data_ptr(), metadata.data_ptr(), columns.data_ptr(), version_of(values), version_of(metadata),
                 version_of(columns), rows, cols, n, m, v, (int)values.get_device()};
@@ -81,16 +104,17 @@ spatha_spmm_plan* plan_for(const torch::Tensor& values, const torch::Tensor& met
         g_lru.splice(g_lru.begin(), g_lru, hit->second);
         return hit->second->plan;
     }
-    spatha_spmm_plan* plan = nullptr;
+    spatha_spmm_plan* raw = nullptr;
     check(spatha_spmm_plan_create(rows, cols, n, m, v, (const uint16_t*)values.data_ptr(), (const uint32_t*)metadata.data_ptr(),
-                                  (const uint32_t*)columns.data_ptr(), stream, &plan),
+                                  (const uint32_t*)columns.data_ptr(), stream, &raw),
           "spatha_spmm_plan_create");
+    std::shared_ptr<spatha_spmm_plan> plan(raw, [](spatha_spmm_plan* p) { spatha_spmm_plan_destroy(p); });
+    // the same three tensors at another version: the weights were rewritten in place, those plans are stale
+    drop_entries([&key](const PlanEntry& e) { return same_storage(e.key, key); });
     g_lru.push_front(PlanEntry{key, plan, values, metadata, columns});
     g_index[key] = g_lru.begin();
     while (g_lru.size() > kMaxPlans) {
-        PlanEntry& old = g_lru.back();
-        spatha_spmm_plan_destroy(old.plan);
-        g_index.erase(old.key);
+        g_index.erase(g_lru.back().key);
         g_lru.pop_back();
     }
     return plan;
@@ -114,16 +138,17 @@ torch::Tensor run(const torch::Tensor& A_metadata, const torch::Tensor& A_indice
     const int tokens = (int)rhs_matrix.size(1);
     const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(A_values.device());
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(A_values.get_device()).stream();
-    spatha_spmm_plan* plan = plan_for(A_values.detach(), A_metadata, A_indices, rows, cols, n, m, v, stream);
+    // (this reference outlives the launch calls below, whatever another thread does to the cache meanwhile)
+    const std::shared_ptr<spatha_spmm_plan> plan = plan_for(A_values.detach(), A_metadata, A_indices, rows, cols, n, m, v, stream);
     torch::Tensor out = torch::empty(transposed_out ? std::vector<int64_t>{tokens, rows} : std::vector<int64_t>{rows, tokens},
                                      rhs_matrix.options());
     const int layout = transposed_out ? SPATHA_OUT_TRANSPOSED : SPATHA_OUT_ROW_MAJOR;
     if (fused)
-        check(spatha_spmm_run_fused(plan, (const uint16_t*)rhs_matrix.data_ptr(), tokens, bias_ptr, (uint16_t*)out.data_ptr(), layout,
+        check(spatha_spmm_run_fused(plan.get(), (const uint16_t*)rhs_matrix.data_ptr(), tokens, bias_ptr, (uint16_t*)out.data_ptr(), layout,
                                     activation, 0, stream),
               "spatha_spmm_run_fused");
     else
-        check(spatha_spmm_run(plan, (const uint16_t*)rhs_matrix.data_ptr(), tokens, bias_ptr, (uint16_t*)out.data_ptr(), layout, 0,
+        check(spatha_spmm_run(plan.get(), (const uint16_t*)rhs_matrix.data_ptr(), tokens, bias_ptr, (uint16_t*)out.data_ptr(), layout, 0,
                               stream),
               "spatha_spmm_run");
     return out;
@@ -154,9 +179,17 @@ torch::Tensor spmm_fused(torch::Tensor A_metadata, torch::Tensor A_indices, torc
 
 void clear_plan_cache() {
     std::lock_guard<std::mutex> guard(g_lock);
-    for (PlanEntry& e : g_lru) spatha_spmm_plan_destroy(e.plan);
     g_lru.clear();
     g_index.clear();
+}
+
+// Drops the plans built from this values tensor (any version): for weights changed behind torch's back.
+int64_t invalidate_plans(const torch::Tensor& A_values) {
+    std::lock_guard<std::mutex> guard(g_lock);
+    const size_t before = g_lru.size();
+    const void* ptr = A_values.data_ptr();
+    drop_entries([ptr](const PlanEntry& e) { return e.key.values == ptr; });
+    return (int64_t)(before - g_lru.size());
 }
 
 int64_t plan_cache_size() {
@@ -176,5 +209,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, mod) {
             py::arg("A_num_cols"), py::arg("vec_length"), py::arg("n"), py::arg("m"), py::arg("activation") = 0,
             py::arg("transposed_out") = false);
     mod.def("clear_plan_cache", &clear_plan_cache, "drop every cached plan");
+    mod.def("invalidate_plans", &invalidate_plans, "drop the cached plans built from this values tensor; returns how many",
+            py::arg("A_values"));
     mod.def("plan_cache_size", &plan_cache_size, "number of cached plans");
 }

@@ -645,7 +645,7 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     static_assert(!PINGPONG || NC == 8, "ping-pong needs eight consumer waves");
-    static int cus = 0;
+    const int cus = p.cus;        // compute units of the plan's device
     void (*kern)(SpmmParams);
     if constexpr (PINGPONG) kern = spmm_dspp_kernel<M, NS, NP, OUT_LAYOUT>;
     else kern = spmm_ds_kernel<M, NS, NP, NC, OUT_LAYOUT, HALF>;
@@ -653,9 +653,6 @@ static hipError_t launch_ds(const SpmmParams& p, hipStream_t stream) {
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
-        int dev = 0;
-        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
-        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
         attr_set = true;
     }
     const int tiles = p.tiles_m * p.tiles_n;

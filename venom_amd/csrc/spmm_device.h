@@ -347,6 +347,28 @@ struct WsCfg {
     static constexpr uint32_t RT_BASE = EPI_BASE + EPI_BYTES;
 };
 
+// LDS layout of the producer / consumer kernel with store waves (spmm_wsw_kernel, spmm_warpspec.hip): the stages of
+// WsCfg, a staging buffer that holds one whole finished tile, and the row-table slots.
+template <int WM_, int WN_, int NS, int NP_>
+struct WswCfg {
+    static_assert(WM_ * WN_ == 4, "four consumer waves, four store waves");
+    static constexpr int WM = WM_, WN = WN_, NP = NP_;
+    static constexpr int NC = 4, NSW = 4;
+    static constexpr int BM = WM * 64, BN = WN * 64;
+    static constexpr int ROW_BYTES = BN * 2;
+    static constexpr int B_BYTES = 64 * ROW_BYTES;
+    static constexpr int STAGE_BYTES = B_BYTES + WM * APACK_BLOCK;
+    static constexpr int PA = NS - 1;
+    static constexpr int STG_PITCH = BM * 2 + 16;                   // transposed output: a tile column (BM rows) + 16 B
+    // the staging buffer: row-major output 4 blocks x 8 slabs x 1 KB, transposed output BN tile columns
+    static constexpr int EPI_BYTES = BN * STG_PITCH > 4 * 8192 ? BN * STG_PITCH : 4 * 8192;
+    static constexpr int RT_BYTES = NP * (PA + 1) * 256;
+    static constexpr int LDS_BYTES = NS * STAGE_BYTES + EPI_BYTES + RT_BYTES;
+    static constexpr int THREADS = (NC + NP + NSW) * 64;
+    static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
+    static constexpr uint32_t RT_BASE = EPI_BASE + EPI_BYTES;
+};
+
 // Tile walk shared by both roles: XCD x (= workgroup id % 8) owns a contiguous range of tile
 // ids (id -> n-tile major, m-tile minor) and its workgroups take them round robin; the
 // coordinates advance by a fixed (dm, dn) with carry, so no division per tile.

@@ -31,9 +31,9 @@ const VariantInfo kVariants[] = {
     {SPMM_VARIANT_D64x256_S3, "smfmac16x16x64_warpspec_deferred_tile64x256_3stage", 64, 256, WsCfg<1, 4, 3, 2>::LDS_BYTES, 0,
      launch_warpspec},
     {SPMM_VARIANT_WS128x128_S3, "smfmac16x16x64_warpspec_storewaves_tile128x128_3stage", 128, 128,
-     3 * (64 * 256 + 2 * APACK_BLOCK) + 128 * 272 + 4 * 3 * 256, 0, launch_warpspec},
+     WswCfg<2, 2, 3, 4>::LDS_BYTES, 0, launch_warpspec},
     {SPMM_VARIANT_WS64x256_S3, "smfmac16x16x64_warpspec_storewaves_tile64x256_3stage", 64, 256,
-     3 * (64 * 512 + APACK_BLOCK) + 256 * 144 + 2 * 3 * 256, 0, launch_warpspec},
+     WswCfg<1, 4, 3, 2>::LDS_BYTES, 0, launch_warpspec},
     {SPMM_VARIANT_T128x256_S3, "smfmac16x16x64_warpspec_tall_tile128x256_3stage", 128, 256, WsCfg<2, 4, 3, 4>::LDS_BYTES, 0,
      launch_warpspec},
     {SPMM_VARIANT_DS256x128_S3_C8, "smfmac16x16x64_warpspec_densestage_tile256x128_3stage_8consumers", 256, 128,

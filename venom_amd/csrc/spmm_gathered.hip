@@ -395,6 +395,36 @@ static hipError_t launch_pipe(const SpmmParams& p, hipStream_t stream) {
 // The row tables of the tile's two halves sit in LDS as 16-bit row numbers (0xffff = zero row).
 // Tile 64 x (64*WN), one wave per 64 columns; everything else as in spmm_pipe_kernel.
 // ---------------------------------------------------------------------------
+// Fused epilogue (t = fp16(acc) + bias[row], then the activation in fp32) for the half-tile operand order: the lane's
+// values of instruction mb are tile rows 32*(mb/2) + 8*ib + 4*(mb%2) + r.  `hi_rows` is false for the padded second half
+// of a last tile (rows % 64 == 32), whose bias entries do not exist.
+template <int ACT>
+__device__ __forceinline__ void fused_bias_act_half_impl(float4_t (&acc)[4][4], const uint16_t* bias, int64_t m0, int ib,
+                                                         bool hi_rows) {
+#pragma unroll
+    for (int mb = 0; mb < 4; mb++) {
+        half4_t bv = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+        if (bias && (mb < 2 || hi_rows)) bv = *(const half4_t*)(bias + m0 + 32 * (mb >> 1) + 8 * ib + 4 * (mb & 1));
+#pragma unroll
+        for (int nb = 0; nb < 4; nb++) {
+            float4_t v = acc[mb][nb];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const float t = (float)((_Float16)v[r] + bv[r]);
+                v[r] = ACT == SPATHA_ACT_GELU ? act_gelu_erf(t) : ACT == SPATHA_ACT_GELU_TANH ? act_gelu_tanh(t) : t;
+            }
+            acc[mb][nb] = v;
+            if (ACT != SPATHA_ACT_NONE) __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+__device__ __forceinline__ void fused_bias_act_half(float4_t (&acc)[4][4], const uint16_t* bias, int64_t m0, int ib, bool hi_rows,
+                                                    int act) {
+    if (act == SPATHA_ACT_GELU) fused_bias_act_half_impl<SPATHA_ACT_GELU>(acc, bias, m0, ib, hi_rows);
+    else if (act == SPATHA_ACT_GELU_TANH) fused_bias_act_half_impl<SPATHA_ACT_GELU_TANH>(acc, bias, m0, ib, hi_rows);
+    else fused_bias_act_half_impl<SPATHA_ACT_NONE>(acc, bias, m0, ib, hi_rows);
+}
+
 template <int WN, int NS, int OUT_LAYOUT>
 __global__ __launch_bounds__(WN * 64) void spmm_half_kernel(SpmmParams p) {
     constexpr int BN = WN * 64;
@@ -534,14 +564,16 @@ __global__ __launch_bounds__(WN * 64) void spmm_half_kernel(SpmmParams p) {
 
     // ------------------------------------------------------------------ write-out
     const int j = lane & 15, ib = lane >> 4;
+    const bool hi_rows = m0 + 32 < p.rows;
+    if (p.fuse) fused_bias_act_half(acc, p.bias, m0, ib, hi_rows, p.act);
+    const uint16_t* bias = p.fuse ? nullptr : p.bias;         // the plain transposed write-out adds the bias itself
     if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
         // per output column the lane holds rows 8*ib .. +7 (instructions 0, 1) and 32 + 8*ib .. +7 (2, 3)
         const int64_t row_lo = (int64_t)m0 + ib * 8, row_hi = row_lo + 32;
-        const bool hi_rows = m0 + 32 < p.rows;
         half8_t bias_lo, bias_hi = {};
-        if (p.bias) {
-            bias_lo = *(const half8_t*)(p.bias + row_lo);
-            if (hi_rows) bias_hi = *(const half8_t*)(p.bias + row_hi);
+        if (bias) {
+            bias_lo = *(const half8_t*)(bias + row_lo);
+            if (hi_rows) bias_hi = *(const half8_t*)(bias + row_hi);
         }
 #pragma unroll
         for (int nb = 0; nb < 4; nb++) {
@@ -554,7 +586,7 @@ __global__ __launch_bounds__(WN * 64) void spmm_half_kernel(SpmmParams p) {
                     lo[mb * 4 + r] = (_Float16)acc[mb][nb][r];
                     hi[mb * 4 + r] = (_Float16)acc[mb + 2][nb][r];
                 }
-            if (p.bias) {
+            if (bias) {
                 lo = lo + bias_lo;
                 hi = hi + bias_hi;
             }
@@ -882,15 +914,12 @@ static hipError_t launch_persist(const SpmmParams& p, hipStream_t stream) {
     using Cfg = PersistCfg<WM, WN, NS>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static int cus = 0;
+    const int cus = p.cus;        // compute units of the plan's device
     auto kern = spmm_persist_kernel<WM, WN, NS, OUT_LAYOUT>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
-        int dev = 0;
-        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
-        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
         attr_set = true;
     }
     const int per_cu = (160 * 1024) / lds;

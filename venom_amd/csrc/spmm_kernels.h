@@ -23,6 +23,7 @@ struct SpmmParams {
     int m;                    // dense columns per group (dense-staged kernels)
     uint32_t b_bytes, apack_bytes, rowtab_bytes;   // sizes for buffer descriptors (persistent kernels)
     int tiles_m, tiles_n;
+    int cus;                  // compute units of the device the launch goes to (grid size of the persistent kernels)
     int skew;                 // start-up skew between workgroups, in units of 1024 clocks (0 = none)
     long long* prof;          // development cycle-accounting buffer (SPATHA_DEV_PROFILE builds), else null
     int fuse;                 // 1: bias and activation are applied ahead of the write-out (fused_bias_act)

@@ -323,7 +323,7 @@ template <int OUT_LAYOUT, bool FUSE, bool GROUPED>
 static hipError_t launch_up(const SpmmParams& p, hipStream_t stream) {
     constexpr int lds = UpCfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static int cus = 0;
+    const int cus = p.cus;        // compute units of the plan's device
     void (*kern)(SpmmParams) = spmm_up_kernel<OUT_LAYOUT, FUSE, GROUPED>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
@@ -335,9 +335,6 @@ static hipError_t launch_up(const SpmmParams& p, hipStream_t stream) {
         if (fa.localSizeBytes != 0) return hipErrorNotSupported;
         e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
-        int dev = 0;
-        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
-        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
         attr_set = true;
     }
     const int tiles = p.tiles_m * p.tiles_n;

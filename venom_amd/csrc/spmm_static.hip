@@ -87,6 +87,11 @@ extern "C" int spatha_spmm_run_noalloc(int rows, int cols, int n, int m, int v, 
     plan.apack_bytes = lay.apack_bytes; plan.rowtab_bytes = lay.rowtab_bytes;
     plan.gtab_bytes = lay.gtab_bytes;
 
+    // every argument check and the kernel choice come before the first launch: a call that is going to be refused must
+    // not have touched the array another (valid) call may be about to read
+    if ((st = spatha::plan_run_check(&plan, B_dev, N, bias_dev, out_dev, out_layout, SPATHA_ACT_NONE, false, 0, nullptr)) != SPATHA_OK)
+        return st;
+
     // The array keeps what the last call left: the block of zeros is cleared again, everything else is rewritten in
     // full by the pack kernels (every byte the SpMM kernels read for this shape).
     hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (uint32_t*)base, 256);

@@ -444,15 +444,12 @@ static hipError_t launch_wst(const SpmmParams& p, hipStream_t stream) {
     using Cfg = WsCfg<2, WN, NS, NP>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static int cus = 0;
+    const int cus = p.cus;        // compute units of the plan's device
     auto kern = spmm_wst_kernel<WN, NS, NP, OUT_LAYOUT>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
-        int dev = 0;
-        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
-        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
         attr_set = true;
     }
     const int per_cu = (160 * 1024) / lds;
@@ -501,15 +498,12 @@ static hipError_t launch_ws(const SpmmParams& p, hipStream_t stream) {
     using Cfg = WsCfg<WM, WN, NS, NP>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
-    static int cus = 0;
+    const int cus = p.cus;        // compute units of the plan's device
     auto kern = spmm_ws_kernel<WM, WN, NS, NP, OUT_LAYOUT, DEFER>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
-        int dev = 0;
-        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
-        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
         attr_set = true;
     }
     const int per_cu = (160 * 1024) / lds;
@@ -535,25 +529,7 @@ static hipError_t launch_ws(const SpmmParams& p, hipStream_t stream) {
 // The staging buffer is free again when the consumers dump the next tile: the store waves have read all of it before they
 // join the second step barrier, and a tile has two k-steps or more (the host refuses S = 1 for this kernel).
 // ---------------------------------------------------------------------------
-template <int WM_, int WN_, int NS, int NP_>
-struct WswCfg {
-    static_assert(WM_ * WN_ == 4, "four consumer waves, four store waves");
-    static constexpr int WM = WM_, WN = WN_, NP = NP_;
-    static constexpr int NC = 4, NSW = 4;
-    static constexpr int BM = WM * 64, BN = WN * 64;
-    static constexpr int ROW_BYTES = BN * 2;
-    static constexpr int B_BYTES = 64 * ROW_BYTES;
-    static constexpr int STAGE_BYTES = B_BYTES + WM * APACK_BLOCK;
-    static constexpr int PA = NS - 1;
-    static constexpr int STG_PITCH = BM * 2 + 16;                   // transposed output: a tile column (BM rows) + 16 B
-    // the staging buffer: row-major output 4 blocks x 8 slabs x 1 KB, transposed output BN tile columns
-    static constexpr int EPI_BYTES = BN * STG_PITCH > 4 * 8192 ? BN * STG_PITCH : 4 * 8192;
-    static constexpr int RT_BYTES = NP * (PA + 1) * 256;
-    static constexpr int LDS_BYTES = NS * STAGE_BYTES + EPI_BYTES + RT_BYTES;
-    static constexpr int THREADS = (NC + NP + NSW) * 64;
-    static constexpr uint32_t EPI_BASE = NS * STAGE_BYTES;
-    static constexpr uint32_t RT_BASE = EPI_BASE + EPI_BYTES;
-};
+// (WswCfg, the LDS layout of this kernel, lives in spmm_device.h beside WsCfg: the kernel registry sizes LDS from it)
 
 template <class Cfg, int OUT_LAYOUT>
 __device__ __forceinline__ void wsw_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
@@ -739,15 +715,12 @@ static hipError_t launch_wsw(const SpmmParams& p, hipStream_t stream) {
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     if (p.S < 2) return hipErrorInvalidValue;
-    static int cus = 0;
+    const int cus = p.cus;        // compute units of the plan's device
     auto kern = spmm_wsw_kernel<WM, WN, NS, NP, OUT_LAYOUT>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return e;
-        int dev = 0;
-        if ((e = hipGetDevice(&dev)) != hipSuccess) return e;
-        if ((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) != hipSuccess) return e;
         attr_set = true;
     }
     const int tiles = p.tiles_m * p.tiles_n;

@@ -98,6 +98,18 @@ def fill_rand_small_ints(count):
     return out
 
 
+def benchmark_inputs(rows, cols, ncols_b, n, m, v):
+    """(B, metadata, columns, values) of one reference benchmark run, drawn from rand() in its order."""
+    g = geometry(rows, cols, n, m, v)
+    B = np.empty((cols, ncols_b), np.float16)
+    meta = np.zeros(g.n_metadata, np.uint32)
+    columns = np.zeros(g.n_columns, np.uint32)
+    vals = np.empty(g.n_values, np.float16)
+    _lib.check(_lib.lib().spatha_benchmark_inputs_f16(rows, cols, ncols_b, n, m, v, _p(B), _p(meta), _p(columns), _p(vals)),
+               "spatha_benchmark_inputs_f16")
+    return B, meta, columns, vals
+
+
 def pack_meta_blob(metadata, columns):
     metadata = np.ascontiguousarray(metadata).view(np.uint32)
     columns = np.ascontiguousarray(columns, dtype=np.uint32).reshape(-1)

@@ -126,6 +126,13 @@ def clear_plan_cache():
     _extension().clear_plan_cache()
 
 
+def invalidate_plans(A_values):
+    """Drops the operator's cached plans built from this values tensor; returns how many.  Needed only after the weights were
+    changed in a way torch does not record (through `.data` or a raw pointer): in-place tensor operations bump the
+    tensor's version, and the operator rebuilds (and drops the stale plan) by itself."""
+    return int(_extension().invalidate_plans(A_values))
+
+
 def transpose(x):
     """x[rows, cols] fp16, contiguous -> a new contiguous [cols, rows] tensor (what `x.T.contiguous()` returns),
     through the library's tiled kernel on torch's current stream."""

@@ -41,6 +41,8 @@ MEASURED_TRAFFIC = {
         (323_090_000, "profiles/spmm_up_kernel_tile512x128_ffn_up_2-4.md"),
     ("smfmac16x16x64_warpspec_storewaves_tile128x128_3stage", 4096, 1024, 16384, 32, 128):
         (172_585_000, "profiles/spmm_wsw_kernel_tile128x128_ffn_up_128-2-32.md"),
+    ("smfmac16x16x64_warpspec_storewaves_tile128x128_3stage", 1024, 4096, 4096, 8, 128):
+        (61_530_000, "profiles/spmm_wsw_kernel_tile128x128_config1_128-2-8.md"),
     ("smfmac16x16x64_warpspec_tall_tile128x256_3stage", 49152, 12288, 2048, 16, 128):
         (2_202_100_000, "profiles/spmm_wst_kernel_tile128x256_gpt3_ffn_n2048.md"),
 }
@@ -128,6 +130,8 @@ def main():
     ap.add_argument("--m", type=int, default=8)
     ap.add_argument("--v", type=int, default=64)
     ap.add_argument("--variant", type=int, default=0)
+    ap.add_argument("--value-std", type=float, default=0.02, help="standard deviation of A's non-zeros (BASELINE config 1: 1.0)")
+    ap.add_argument("--b-uniform", action="store_true", help="B ~ U(-1, 1) instead of N(0, 1) (BASELINE config 1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extra", action="store_true", help="also time three shapes outside BASELINE.json (appended to 'extra')")
     ap.add_argument("--ablation", action="store_true",
@@ -230,7 +234,7 @@ def main():
         del src, dst
 
     rows, cols, N, m, v = args.rows, args.cols, args.n, args.m, args.v
-    w = prepare(rows, cols, N, m, v)
+    w = prepare(rows, cols, N, m, v, value_std=args.value_std, b_uniform=args.b_uniform)
     ms_wall, ms_kernel = timed(w, args.steps, args.warmup, args.variant)
     ksp = w["geo"].ksp
     flops_dense = 2.0 * rows * cols * N
@@ -254,7 +258,8 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16 (fp32 accumulate)",
-        "data": "synthetic (seed 0: A %d:2:%d random pattern, values ~N(0,0.02); B ~N(0,1))" % (v, m),
+        "data": "synthetic (seed 0: A %d:2:%d random pattern, values ~N(0,%g); B ~%s)" % (v, m, args.value_std,
+                                                                                            "U(-1,1)" if args.b_uniform else "N(0,1)"),
         "config": {"workload": "spmm A %dx%d %d:2:%d (Ksp %d) x B %dx%d, row-major C" % (rows, cols, v, m, ksp, cols, N),
                    "kernel": w["plan"].kernel_name(N, 0, args.variant)},
         "pct_smfmac_peak": round(100.0 * flops_smfmac / (ms_kernel * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2),
@@ -381,7 +386,8 @@ def main():
         for (r2, c2) in ((1024, 1024), (4096, 1024), (1024, 4096)):
             for v2 in (64, 128):
                 for m2 in (8, 16, 32):
-                    if (r2, c2, m2, v2) == (rows, cols, m, v) and N == 16384 and args.variant == 0:
+                    if (r2, c2, m2, v2) == (rows, cols, m, v) and N == 16384 and args.variant == 0 and args.value_std == 0.02 \
+                            and not args.b_uniform:
                         w2, k2 = w, ms_kernel               # the headline cell: measured above
                     else:
                         w2 = prepare(r2, c2, 16384, m2, v2)

@@ -30,7 +30,7 @@ bool variant_has_fused_writeout(int variant) {
     switch (variant) {
         case SPMM_VARIANT_P128x128_S3: case SPMM_VARIANT_P64x256_S2: case SPMM_VARIANT_R64x256_S3:
         case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x256_S3: case SPMM_VARIANT_W64x256_S3:
-        case SPMM_VARIANT_W128x128_S5: case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DSH256x128_S3_C8:
+        case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DSH256x128_S3_C8:
         case SPMM_VARIANT_UP512x128_S3: case SPMM_VARIANT_DU512x128_M16: case SPMM_VARIANT_WS128x128_S3:
         case SPMM_VARIANT_WS64x256_S3: case SPMM_VARIANT_H64x256_S2: case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2:
             return true;

@@ -25,8 +25,6 @@ const VariantInfo kVariants[] = {
      launch_gathered},
     {SPMM_VARIANT_W128x128_S3, "smfmac16x16x64_warpspec_tile128x128_3stage", 128, 128, WsCfg<2, 2, 3, 4>::LDS_BYTES, 0,
      launch_warpspec},
-    {SPMM_VARIANT_W128x128_S5, "smfmac16x16x64_warpspec_tile128x128_5stage", 128, 128, WsCfg<2, 2, 5, 4>::LDS_BYTES, 0,
-     launch_warpspec},
     {SPMM_VARIANT_W128x256_S3, "smfmac16x16x64_warpspec_tile128x256_3stage", 128, 256, WsCfg<2, 4, 3, 4>::LDS_BYTES, 0,
      launch_warpspec},
     {SPMM_VARIANT_W64x256_S3, "smfmac16x16x64_warpspec_tile64x256_3stage", 64, 256, WsCfg<1, 4, 3, 2>::LDS_BYTES, 0, launch_warpspec},

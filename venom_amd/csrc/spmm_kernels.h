@@ -58,8 +58,7 @@ enum {
     SPMM_VARIANT_DU512x128_M16 = 19,    // 8 < m <= 16: one phase group, 64 KB stages, two of them
     SPMM_VARIANT_WS128x128_S3 = 20,     // id 6 with store waves: finished tiles leave through an LDS staging buffer and a third role
     SPMM_VARIANT_WS64x256_S3 = 21,      // id 8 with store waves
-    SPMM_VARIANT_W128x128_S5 = 22,      // id 6 with five stages: four k-steps of loads in flight, for tiles whose B rows come from HBM
-    SPMM_VARIANT_COUNT = 23
+    SPMM_VARIANT_COUNT = 22
 };
 
 const char* spmm_variant_name(int variant);

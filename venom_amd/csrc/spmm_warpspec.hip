@@ -737,8 +737,6 @@ hipError_t launch_warpspec(int variant, int out_layout, const SpmmParams& p, hip
     switch (variant) {
         case SPMM_VARIANT_W128x128_S3:
             return t ? launch_ws<2, 2, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_ws<2, 2, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
-        case SPMM_VARIANT_W128x128_S5:
-            return t ? launch_ws<2, 2, 5, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_ws<2, 2, 5, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
         case SPMM_VARIANT_W128x256_S3:
             return t ? launch_ws<2, 4, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_ws<2, 4, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
         case SPMM_VARIANT_W64x256_S3:

@@ -426,6 +426,13 @@ def main():
         t_e2e = time.perf_counter()
         out["e2e"] = dict(bert.measure(n=2, m=8, v=64, repeats=10, warmups=3),
                           config="5: BERT-large encoder, 24 layers, batch 32 x seq 512, random-init weights, 64:2:8 drop-in layers")
+        # ... and with the library's own additions to that path: feed-forward blocks without the transposed copy of the
+        # [tokens, 4*hidden] activation (bias + GELU in the SpMM's write-out), the three attention projections as one SpMM,
+        # residual + LayerNorm as one kernel (that one in the DENSE model as well: it does not depend on the weight format)
+        torch.cuda.empty_cache()
+        out["e2e"]["with_fused_blocks"] = dict(
+            bert.measure(n=2, m=8, v=64, repeats=10, warmups=3, fuse_ffn=True, merge=True, fuse_ln=True, kernel_gelu=True),
+            what="fused feed-forward (bias + GELU in the write-out), merged q/k/v projections, residual + LayerNorm kernel in both models")
         out["e2e"]["wall_s_incl_model_build"] = round(time.perf_counter() - t_e2e, 1)
 
     if args.ablation:

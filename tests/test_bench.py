@@ -47,7 +47,7 @@ def test_no_power_sampling_under_a_profiler(monkeypatch):
 @pytest.mark.gpu
 def test_short_run_prints_one_line_with_roofline_power_and_calibration():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "5", "--warmup", "2", "--settle-ms", "0",
-                        "--no-extra", "--no-cpu-baseline", "--power-seconds", "0.6", "--calibrate"],
+                        "--no-extra", "--no-e2e", "--no-cpu-baseline", "--power-seconds", "0.6", "--calibrate"],
                        capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [x for x in r.stdout.splitlines() if x.strip()]
@@ -67,3 +67,28 @@ def test_short_run_prints_one_line_with_roofline_power_and_calibration():
     assert 1.0 < cal["store_c_alone"]["tb_per_s"] < 20.0
     # zeros are the cheapest operands: never slower than Gaussian ones, and never above the nominal peak
     assert cal["smfmac_alone_gaussian"]["pct_smfmac_peak"] <= cal["smfmac_alone_zeros"]["pct_smfmac_peak"] * 1.05 <= 105.0
+
+
+@pytest.mark.gpu
+def test_default_run_carries_every_baseline_workload():
+    """What the driver runs: one line with the headline figure, the other BASELINE workloads under `extra` (config 1, the 2:4
+    baseline, 18 sweep cells, the GPT-3 matrix at three token counts), the encoder under `e2e`, the CPU baseline."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "20", "--warmup", "5", "--power-seconds", "0.6"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [x for x in r.stdout.splitlines() if x.strip()]
+    assert len(lines) == 1
+    out = json.loads(lines[0])
+    extra = out["extra"]
+    assert [e["config"][0] for e in extra] == ["1", "2"] + ["3"] * 18 + ["4"] * 3
+    for e in extra:
+        assert e["us"] > 0 and 0.02 < e["hbm_frac"] < 1.0 and e["bound"] in ("hbm", "mfma") and 0.05 < e["frac_of_bound"] < 1.0
+        assert e["kernel"].startswith("smfmac16x16x64_")
+    assert extra[0]["shape"] == "1024x4096x4096 128:2:8" and extra[0]["traffic"] is not None
+    assert {e["shape"].split(" ")[1] for e in extra[2:20]} == {"%d:2:%d" % (v, m) for v in (64, 128) for m in (8, 16, 32)}
+    assert [e["shape"].split("x")[2].split(" ")[0] for e in extra[20:]] == ["16", "256", "2048"]
+    e2e = out["e2e"]
+    assert e2e["format"] == "64:2:8" and e2e["layers"] == 24 and e2e["tokens"] == 16384
+    assert e2e["dense_ms"] > e2e["vnm_ms"] > 0 and e2e["with_fused_blocks"]["vnm_ms"] < e2e["vnm_ms"]
+    cpu = out["cpu_baseline"]
+    assert cpu["kind"] == "port" and cpu["cores"] >= 1 and cpu["value"] > 0 and "bit-identical" in cpu["sample"]

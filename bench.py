@@ -146,10 +146,13 @@ def main():
     ap.add_argument("--no-power", action="store_true",
                     help="skip the sustained run with `amd-smi` power / clock sampling that follows the timed region ('power')")
     ap.add_argument("--power-seconds", type=float, default=2.0, help="length of that sustained run")
+    ap.add_argument("--no-calibrate", action="store_true",
+                    help="skip the machine calibration kernels and the power floor derived from them ('calibration', 'power_floor'); "
+                         "they run by default wherever power sampling works")
     ap.add_argument("--calibrate", action="store_true",
-                    help="also run the machine calibration kernels (venom_amd/csrc/calibrate.hip) under the same sampling: a "
-                         "write of C alone, and sparse matrix instructions alone on Gaussian / small-integer / zero operands "
-                         "('calibration')")
+                    help="run the machine calibration kernels (venom_amd/csrc/calibrate.hip: a write of C alone, and sparse matrix "
+                         "instructions alone on Gaussian / small-integer / zero operands; 'calibration') even where power sampling "
+                         "does not work")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the SpMM path has no multi-GPU part); run with --gpus 1",
@@ -163,7 +166,7 @@ def main():
         alt = os.path.join(ROOT, "venom_amd", "lib", "libspatha_out32b.so")
         if os.path.exists(alt):
             import subprocess
-            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu-baseline", "--no-extra", "--no-e2e", "--steps", str(args.steps),
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--no-cpu-baseline", "--no-extra", "--no-e2e", "--no-calibrate", "--steps", str(args.steps),
                                 "--warmup", str(args.warmup), "--variant", str(args.variant)],
                                env=dict(os.environ, SPATHA_LIBRARY=alt), stdout=subprocess.PIPE, text=True)
             if r.returncode == 0 and r.stdout.strip():
@@ -287,7 +290,7 @@ def main():
     else:
         out["power"] = None
 
-    if args.calibrate:
+    if args.calibrate or (idle is not None and not args.no_calibrate):
         cal = ctypes.CDLL(os.path.join(ROOT, "venom_amd", "lib", "libspatha_calibrate.so"))
         cal.spatha_calibrate_store.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
         cal.spatha_calibrate_smfmac.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
@@ -340,6 +343,23 @@ def main():
                         60.0, lambda us_c: {"wave_instructions": n_inst, "dense_equiv_tflops": round(flops / us_c * 1e-6, 1),
                                             "pct_smfmac_peak": round(100 * flops / us_c * 1e-6 / SMFMAC_PEAK_TFLOPS, 1)})
         out["calibration"] = calib
+        # The floor the socket's power limit puts under this workload, from the parts measured alone just now: the energy above
+        # idle of its matrix instructions (on Gaussian operands) and of writing C once, spent at (limit - idle) watts, the limit
+        # being the highest sustained socket power seen in this run.  Operand movement (L2 -> CU, LDS) is NOT in it.
+        g, st = calib.get("smfmac_alone_gaussian"), calib.get("store_c_alone")
+        if g and st and g["socket_w"] and st["socket_w"] and out.get("power") and out["power"]["socket_w"]:
+            idle_w = float(idle[0])
+            limit_w = max([out["power"]["socket_w"]] + [c["socket_w"] for c in calib.values() if c["socket_w"]])
+            n_inst = (rows // 16) * (N // 16) * (ksp // 32)
+            e_mfma = (g["socket_w"] - idle_w) * g["us"] * n_inst / g["wave_instructions"]          # microjoules
+            e_store = (st["socket_w"] - idle_w) * st["us"] * (2.0 * rows * N) / st["bytes"]
+            floor_us = (e_mfma + e_store) / (limit_w - idle_w)
+            out["power_floor"] = {"us": round(floor_us, 2), "frac": round(floor_us / (ms_kernel * 1e3), 3),
+                                  "matrix_mj": round(e_mfma * 1e-3, 2), "store_mj": round(e_store * 1e-3, 2),
+                                  "idle_w": idle_w, "limit_w": round(limit_w, 1),
+                                  "what": "(energy above idle of this workload's sparse matrix instructions on Gaussian operands + of "
+                                          "writing C once, each measured alone) / (highest sustained socket power of this run - idle); "
+                                          "operand movement not included; frac = that floor / the kernel's time"}
 
     def side_figures(r2, c2, n2, m2, v2, w2, k2, config):
         by = algorithmic_bytes(r2, c2, n2, m2, v2, w2["geo"].ksp)

@@ -67,6 +67,9 @@ def test_short_run_prints_one_line_with_roofline_power_and_calibration():
     assert 1.0 < cal["store_c_alone"]["tb_per_s"] < 20.0
     # zeros are the cheapest operands: never slower than Gaussian ones, and never above the nominal peak
     assert cal["smfmac_alone_gaussian"]["pct_smfmac_peak"] <= cal["smfmac_alone_zeros"]["pct_smfmac_peak"] * 1.05 <= 105.0
+    if out["power"] is not None and out["power"]["socket_w"]:
+        pf = out["power_floor"]             # matrix instructions + C alone at the power limit: a floor, so below the kernel's time
+        assert 0.2 < pf["frac"] < 1.05 and pf["matrix_mj"] > 0 and pf["store_mj"] > 0 and pf["limit_w"] > pf["idle_w"]
 
 
 @pytest.mark.gpu

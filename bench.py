@@ -438,6 +438,34 @@ def main():
             del w2
         out["extra"] = extra
 
+    if not args.no_extra:
+        # the k-split (spatha_spmm_run_ws): few tiles with long k-loops, here 128 tiles of 128 k-steps on the chip's CUs
+        r2, c2, n2, m2, v2 = 1024, 16384, 1024, 8, 128
+        w2 = prepare(r2, c2, n2, m2, v2)
+        _, k_plain = timed(w2, 50, 10, settle_ms=50.0)
+        need = w2["plan"].workspace_bytes(n2)
+        ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=dev)
+        sp2 = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+        def run_split():
+            _lib.check(L.spatha_spmm_run_ws(w2["plan"]._handle, w2["B"].data_ptr(), n2, None, w2["C"].data_ptr(), 0, 0, ws.data_ptr(),
+                                            need, sp2), "run_ws")
+
+        for _ in range(20):
+            run_split()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(50):
+            run_split()
+        e1.record()
+        torch.cuda.synchronize()
+        out["ksplit"] = {"shape": "%dx%dx%d %d:2:%d" % (r2, c2, n2, v2, m2), "kernel": w2["plan"].kernel_name(n2, 0, 0),
+                         "unsplit_us": round(k_plain * 1e3, 2), "split_us": round(e0.elapsed_time(e1) / 50 * 1e3, 2),
+                         "workspace_bytes": need,
+                         "what": "k-loops of the 128 tiles in parts over the CUs that tiles alone leave idle (spatha_spmm_run_ws)"}
+        del w2, ws
+
     if not args.no_e2e:
         # config 5: the BERT-large encoder, batch 32 x 512 tokens, every encoder Linear in 64:2:8 through the operator
         # (drop-in layers), against the same model on dense fp16 weights (hipBLASLt through torch)

@@ -192,6 +192,24 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
 int spatha_spmm_run_fused(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
                           uint16_t* out_dev, int out_layout, int activation, int variant, void* stream);
 
+/* spatha_spmm_run_fused (automatic kernel choice) for callers that bring scratch memory: with a workspace the library may
+ * split k-loops over several workgroups where tiles alone leave compute units idle: few tiles with long k-loops (small
+ * rows x N and large K, the "split-K for small M*N" case: e.g. 1024 x 16384 x 1024 at 128:2:8 runs 128 tiles of 128
+ * k-steps on 256 CUs, 50 us unsplit and 35 us in two parts).  The parts of a tile hand fp32 partial sums over through the
+ * workspace and the part that finishes last adds them in a fixed order, so results do not depend on timing; with
+ * integer-valued operands they equal spatha_spmm_run's bit for bit, otherwise they may differ from it by the rounding of
+ * another summation order.  spatha_spmm_workspace_bytes names the size a call needs for N columns (0: this shape is
+ * never split; the call then equals spatha_spmm_run_fused); a smaller or NULL workspace is not an error, the call just
+ * does not split.  The workspace (256-byte aligned device memory) is cleared ONCE with spatha_spmm_workspace_init after it
+ * has been allocated; every completed call leaves it ready for the next one, of any plan and shape (clear it again after a
+ * call that failed).  It belongs to a call until the call's work on `stream` has completed: calls that overlap in time
+ * need a workspace each.  Neither call allocates or synchronises.  No counterpart in the reference, whose kernels cover
+ * such shapes by a search over 179 tile tuples (src/spmm/spatha_spmm.hpp:49-585). */
+size_t spatha_spmm_workspace_bytes(const spatha_spmm_plan* plan, int N, int out_layout, int fused);
+int spatha_spmm_workspace_init(void* workspace_dev, size_t workspace_bytes, void* stream);
+int spatha_spmm_run_ws(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, uint16_t* out_dev,
+                       int out_layout, int activation, void* workspace_dev, size_t workspace_bytes, void* stream);
+
 /* One SpMM straight from the canonical arrays, for callers that cannot allocate (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same result as
  * spatha_spmm_plan_create + spatha_spmm_run (automatic kernel choice) + spatha_spmm_plan_destroy on the same arguments,

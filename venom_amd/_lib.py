@@ -49,6 +49,9 @@ SIGNATURES = {
     "spatha_spmm_run_fused": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "spatha_spmm_run_noalloc": (c_int, [c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                         c_void_p, c_int, c_void_p]),
+    "spatha_spmm_workspace_bytes": (ctypes.c_size_t, [c_void_p, c_int, c_int, c_int]),
+    "spatha_spmm_workspace_init": (c_int, [c_void_p, ctypes.c_size_t, c_void_p]),
+    "spatha_spmm_run_ws": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, ctypes.c_size_t, c_void_p]),
     "spatha_spmm_num_variants": (c_int, []),
     "spatha_spmm_kernel_name": (c_char_p, [c_void_p, c_int, c_int, c_int]),
     "spatha_spmm_time": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, POINTER(c_float)]),

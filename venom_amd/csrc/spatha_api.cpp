@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -286,6 +287,61 @@ int uneven_rest_rows(const spatha_spmm_plan* plan, int N, int requested, int cho
     if ((plan->geo.rows - rest_rows) % plan->geo.v != 0) return 0;
     return variant_ok(plan, N, spatha::SPMM_VARIANT_W128x128_S3, fused) ? rest_rows : 0;
 }
+
+// ---- k-split (runs that bring a workspace) ----------------------------------------------------------------------
+// Few tiles with long k-loops (small rows x N, large K: the chosen kernel's tiles fill at most half of the CUs): every tile's
+// k-loop is cut into `parts` parts, one workgroup each.  Parts hand their fp32 partial blocks over through the workspace; the
+// part that finishes last adds them in part order and writes the block (ksplit_exchange in spmm_warpspec.hip): deterministic,
+// no workgroup waits for another.
+// The hand-over costs 6-9 us (three dependent trips to the memory side: partial stores, ticket, partial loads; 64 or 128 KB
+// of fp32 per tile and part) and a k-step 0.3-0.6 us, so a split must save about 48 k-steps per tile and leave parts of 32:
+//   1024 x 16384 x 1024 at 128:2:8   (128 tiles of 128 k-steps, 2 parts)  34.7 against 50.2 us
+//   12288 x 49152 x 128 at 128:2:16  ( 96 tiles of 192 k-steps, 2 parts)  48.3 against 73.2 us
+//   768 x 12288 x 2048 at 128:2:8    ( 96 tiles of  96 k-steps, 2 parts)  30.5 against 38.9 us
+//   1024 x 24576 x 2048 at 128:2:16  (128 tiles of  96 k-steps, 2 parts)  31.9 against 39.3 us
+//   tiles of 64 k-steps in four parts of 16: between 15 % ahead and 7 % behind (256 x 8192 x 256, 4096 x 16384 x 256): not split.
+// The rest of an uneven last round as a split second launch of the same kernel (instead of smaller tiles, uneven_rest_rows)
+// was measured as well and does not pay: GPT-3 FFN matrix at 256 tokens (24 saved steps) 75 against 65 us, its FFN-down matrix
+// at 1024 tokens (96 saved steps) 228 against 232 us; 128 x 256 tiles hand over twice the bytes.
+#ifndef SPATHA_KSPLIT_MIN_SAVED_STEPS
+#define SPATHA_KSPLIT_MIN_SAVED_STEPS 48
+#endif
+#ifndef SPATHA_KSPLIT_MIN_PART_STEPS
+#define SPATHA_KSPLIT_MIN_PART_STEPS 32
+#endif
+
+struct SplitChoice {
+    int variant = 0;        // kernel of the split launch (6 or 10)
+    int parts = 1;
+    size_t tickets_bytes = 0, partial_bytes = 0;
+    size_t bytes() const { return tickets_bytes + partial_bytes; }
+};
+
+bool split_choice(const spatha_spmm_plan* plan, int N, int requested, int chosen, bool fused, SplitChoice* out) {
+    using namespace spatha;
+    if (requested != SPMM_VARIANT_AUTO || plan->cus < 8 || plan->half_tiles) return false;
+    int var = chosen;
+    if (var == SPMM_VARIANT_WS128x128_S3) var = SPMM_VARIANT_W128x128_S3;      // the store waves have no hand-over
+    // (the 128 x 256 tiles with 64 x 64 consumer blocks are chosen for short k-loops only, where a split never pays)
+    if (var != SPMM_VARIANT_W128x128_S3 && var != SPMM_VARIANT_T128x256_S3) return false;
+    if (!variant_ok(plan, N, var, fused)) return false;
+    const int bm = spmm_variant_bm(var), bn = spmm_variant_bn(var), S = plan->S;
+    const int grid = (plan->cus / 8) * 8;
+    const int64_t tiles = (int64_t)(plan->geo.rows / bm) * ((N + bn - 1) / bn);
+    if (tiles * 2 > grid) return false;
+    // as many parts as fit one round of the CUs, at most four, S a multiple of them
+    int k = (int)std::min<int64_t>(grid / tiles, 4);
+    while (k > 1 && (S % k != 0 || S / k < SPATHA_KSPLIT_MIN_PART_STEPS || S - S / k < SPATHA_KSPLIT_MIN_SAVED_STEPS)) --k;
+    if (k < 2) return false;
+    SplitChoice c;
+    c.variant = var;
+    c.parts = k;
+    const int blocks_per_tile = (bm / 64) * (bn / 64);
+    c.tickets_bytes = (((size_t)tiles * blocks_per_tile * 4) + 255) & ~(size_t)255;
+    c.partial_bytes = (size_t)tiles * c.parts * bm * bn * 4;
+    *out = c;
+    return true;
+}
 }  // namespace
 
 namespace spatha {
@@ -520,7 +576,8 @@ int spatha::plan_run_check(const spatha_spmm_plan* plan, const uint16_t* B_dev, 
 }
 
 int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, uint16_t* out_dev,
-                     int out_layout, int activation, bool fused_entry, int variant, void* stream) {
+                     int out_layout, int activation, bool fused_entry, int variant, void* stream, void* workspace,
+                     size_t workspace_bytes) {
     int var = -1;
     const int status = plan_run_check(plan, B_dev, N, bias_dev, out_dev, out_layout, activation, fused_entry, variant, &var);
     if (status != SPATHA_OK) return status;
@@ -538,6 +595,7 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
     p.rowtab_bytes = (uint32_t)plan->rowtab_bytes;
     p.fuse = fuse ? 1 : 0; p.act = activation;
     p.cus = plan->cus > 0 ? plan->cus : 256;
+    p.ksplit = 1; p.partial = nullptr; p.partial_bytes = 0; p.tickets = nullptr;
     p.debug = 0; p.skew = 0; p.prof = nullptr;
 #ifdef SPATHA_DEV_PROFILE
     // development builds only: switch parts of a kernel off for time accounting (results are then wrong on purpose)
@@ -545,6 +603,20 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
     { const char* d = std::getenv("SPATHA_SKEW"); p.skew = d ? std::atoi(d) : 0; }
     { const char* d = std::getenv("SPATHA_PROF_PTR"); if (d) p.prof = (long long*)std::strtoull(d, nullptr, 0); }
 #endif
+    SplitChoice sc;
+    if (workspace && split_choice(plan, N, variant, var, fuse, &sc) && workspace_bytes >= sc.bytes() &&
+        ((uintptr_t)workspace & 255) == 0) {
+        // every tile's k-loop in parts: the walk's m-tiles are (row tile, part) pairs
+        spatha::SpmmParams q = p;
+        q.tiles_m = (plan->geo.rows / spatha::spmm_variant_bm(sc.variant)) * sc.parts;
+        q.tiles_n = (N + spatha::spmm_variant_bn(sc.variant) - 1) / spatha::spmm_variant_bn(sc.variant);
+        q.ksplit = sc.parts;
+        q.tickets = (uint32_t*)workspace;       // zero: cleared once by spatha_spmm_workspace_init, put back by every completed run
+        q.partial = (float*)((char*)workspace + sc.tickets_bytes);
+        q.partial_bytes = (uint32_t)sc.partial_bytes;
+        const hipError_t e2 = spatha::launch_spmm(sc.variant, out_layout, q, (hipStream_t)stream);
+        return e2 == hipSuccess ? SPATHA_OK : hip_fail(e2);
+    }
     if (const int rest_rows = uneven_rest_rows(plan, N, variant, var, fuse)) {
         const int main_rows = plan->geo.rows - rest_rows;
         spatha::SpmmParams head = p, tail = p;
@@ -578,6 +650,27 @@ int spatha_spmm_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, 
 int spatha_spmm_run_fused(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
                           uint16_t* out_dev, int out_layout, int activation, int variant, void* stream) {
     return spatha::plan_run(plan, B_dev, N, bias_dev, out_dev, out_layout, activation, true, variant, stream);
+}
+
+size_t spatha_spmm_workspace_bytes(const spatha_spmm_plan* plan, int N, int out_layout, int fused) {
+    if (!plan || N <= 0 || N % 8 != 0) return 0;
+    const int var = pick_variant(plan, N, spatha::SPMM_VARIANT_AUTO, fused != 0, out_layout);
+    SplitChoice sc;
+    if (var < 0 || !split_choice(plan, N, spatha::SPMM_VARIANT_AUTO, var, fused != 0, &sc)) return 0;
+    return sc.bytes();
+}
+
+int spatha_spmm_workspace_init(void* workspace_dev, size_t workspace_bytes, void* stream) {
+    if (!workspace_dev || ((uintptr_t)workspace_dev & 255) || workspace_bytes % 4 != 0) return SPATHA_ERR_BAD_ARGUMENT;
+    if (workspace_bytes / 4 > 0x7fffffffull) return SPATHA_ERR_TOO_LARGE;
+    const hipError_t e = spatha::launch_clear_words((uint32_t*)workspace_dev, (int)(workspace_bytes / 4), (hipStream_t)stream);
+    return e == hipSuccess ? SPATHA_OK : hip_fail(e);
+}
+
+int spatha_spmm_run_ws(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, uint16_t* out_dev,
+                       int out_layout, int activation, void* workspace_dev, size_t workspace_bytes, void* stream) {
+    return spatha::plan_run(plan, B_dev, N, bias_dev, out_dev, out_layout, activation, true, spatha::SPMM_VARIANT_AUTO, stream,
+                            workspace_dev, workspace_bytes);
 }
 
 int spatha_spmm_num_variants(void) { return spatha::SPMM_VARIANT_COUNT; }

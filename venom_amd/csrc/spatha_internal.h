@@ -38,9 +38,11 @@ hipError_t plan_pack(const spatha_spmm_plan* plan, const uint16_t* values_dev, c
 int plan_run_check(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, const uint16_t* out_dev,
                    int out_layout, int activation, bool fused_entry, int variant, int* chosen);
 
-// argument checks, kernel choice and launch shared by every run entry point; returns a spatha_status
+// argument checks, kernel choice and launch shared by every run entry point; returns a spatha_status.  With a workspace
+// (device memory of at least the size split_workspace_bytes names) the automatic choice may split k-loops over workgroups.
 int plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev, uint16_t* out_dev,
-             int out_layout, int activation, bool fused_entry, int variant, void* stream);
+             int out_layout, int activation, bool fused_entry, int variant, void* stream, void* workspace = nullptr,
+             size_t workspace_bytes = 0);
 
 // records a HIP error for spatha_last_hip_error and returns SPATHA_ERR_HIP
 int note_hip_error(hipError_t e);

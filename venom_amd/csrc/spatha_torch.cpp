@@ -19,6 +19,7 @@
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 
 #include <list>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <stdexcept>
@@ -67,6 +68,17 @@ void check(int status, const char* what) {
     if (status != SPATHA_OK)
         throw std::runtime_error(std::string(what) + ": " + spatha_status_string(status) +
                                  (status == SPATHA_ERR_HIP ? " (HIP error " + std::to_string(spatha_last_hip_error()) + ")" : ""));
+}
+
+// Scratch memory of split runs (spatha_spmm_run_ws): one zero-initialised buffer per (device, stream), grown on demand.
+// Calls on one stream are ordered, so they can share it; the library leaves it clean after every completed call.
+std::map<std::pair<int, hipStream_t>, torch::Tensor> g_workspaces;
+
+torch::Tensor workspace_for(int device, hipStream_t stream, size_t bytes, const torch::TensorOptions& like) {
+    std::lock_guard<std::mutex> guard(g_lock);
+    torch::Tensor& ws = g_workspaces[{device, stream}];
+    if (!ws.defined() || (size_t)ws.numel() < bytes) ws = torch::zeros({(int64_t)bytes}, like.dtype(torch::kUInt8));
+    return ws;
 }
 
 void check_weight(const torch::Tensor& t, c10::ScalarType a, c10::ScalarType b, const char* name) {
@@ -143,6 +155,15 @@ torch::Tensor run(const torch::Tensor& A_metadata, const torch::Tensor& A_indice
     torch::Tensor out = torch::empty(transposed_out ? std::vector<int64_t>{tokens, rows} : std::vector<int64_t>{rows, tokens},
                                      rhs_matrix.options());
     const int layout = transposed_out ? SPATHA_OUT_TRANSPOSED : SPATHA_OUT_ROW_MAJOR;
+    // few tokens against a long k-loop: the library splits the k-loops over workgroups if it is given scratch memory
+    const bool fuses = fused && (activation != SPATHA_ACT_NONE || (!transposed_out && bias_ptr));
+    if (const size_t need = spatha_spmm_workspace_bytes(plan.get(), tokens, layout, fuses ? 1 : 0)) {
+        torch::Tensor ws = workspace_for((int)A_values.get_device(), stream, need, rhs_matrix.options());
+        check(spatha_spmm_run_ws(plan.get(), (const uint16_t*)rhs_matrix.data_ptr(), tokens, bias_ptr, (uint16_t*)out.data_ptr(), layout,
+                                 fused ? activation : SPATHA_ACT_NONE, ws.data_ptr(), (size_t)ws.numel(), stream),
+              "spatha_spmm_run_ws");
+        return out;
+    }
     if (fused)
         check(spatha_spmm_run_fused(plan.get(), (const uint16_t*)rhs_matrix.data_ptr(), tokens, bias_ptr, (uint16_t*)out.data_ptr(), layout,
                                     activation, 0, stream),
@@ -181,6 +202,7 @@ void clear_plan_cache() {
     std::lock_guard<std::mutex> guard(g_lock);
     g_lru.clear();
     g_index.clear();
+    g_workspaces.clear();
 }
 
 // Drops the plans built from this values tensor (any version): for weights changed behind torch's back.

@@ -24,6 +24,12 @@ struct SpmmParams {
     uint32_t b_bytes, apack_bytes, rowtab_bytes;   // sizes for buffer descriptors (persistent kernels)
     int tiles_m, tiles_n;
     int cus;                  // compute units of the device the launch goes to (grid size of the persistent kernels)
+    // k-split (producer/consumer kernels 6 and 10 only; 1 everywhere else): tiles_m then counts (row tile, part) pairs and
+    // every part runs S / ksplit k-steps; fp32 partial blocks and one ticket per 64 x 64 block live in the caller's workspace
+    int ksplit;
+    float* partial;
+    uint32_t partial_bytes;
+    uint32_t* tickets;
     int skew;                 // start-up skew between workgroups, in units of 1024 clocks (0 = none)
     long long* prof;          // development cycle-accounting buffer (SPATHA_DEV_PROFILE builds), else null
     int fuse;                 // 1: bias and activation are applied ahead of the write-out (fused_bias_act)
@@ -88,6 +94,9 @@ struct SelectWinner {
 };
 hipError_t launch_select_winners(const float* dense_abs_dev, int rows, int cols, int m, int v, SelectWinner* out_dev,
                                  hipStream_t stream);
+
+// words of 32 bits set to zero by a kernel (tickets of a k-split launch; a kernel, so that the launch can be recorded into a graph)
+hipError_t launch_clear_words(uint32_t* words, int count, hipStream_t stream);
 
 hipError_t launch_pack_gtab(const uint32_t* columns, int rows, int m, int v, int ksp, int S, int block_rows, uint16_t* gtab,
                             hipStream_t stream);

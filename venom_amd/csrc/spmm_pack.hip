@@ -122,5 +122,15 @@ hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const u
     return hipGetLastError();
 }
 
-}  // namespace spatha
+__global__ void clear_words_kernel(uint32_t* words, int count) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) words[i] = 0u;
+}
 
+hipError_t launch_clear_words(uint32_t* words, int count, hipStream_t stream) {
+    if (count <= 0) return hipSuccess;
+    hipLaunchKernelGGL(clear_words_kernel, dim3((count + 255) / 256), dim3(256), 0, stream, words, count);
+    return hipGetLastError();
+}
+
+}  // namespace spatha

@@ -39,12 +39,6 @@ hipError_t scratch_address(int device, unsigned char** out) {
     return hipSuccess;
 }
 
-// (a kernel, not hipMemsetAsync: the call may be recorded into a graph by its caller)
-__global__ void clear_words_kernel(uint32_t* p, int words) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < words) p[i] = 0u;
-}
-
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 }  // namespace
@@ -94,8 +88,8 @@ extern "C" int spatha_spmm_run_noalloc(int rows, int cols, int n, int m, int v, 
 
     // The array keeps what the last call left: the block of zeros is cleared again, everything else is rewritten in
     // full by the pack kernels (every byte the SpMM kernels read for this shape).
-    hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (uint32_t*)base, 256);
-    if ((e = hipGetLastError()) != hipSuccess) return spatha::note_hip_error(e);
+    // (a kernel, not hipMemsetAsync: the call may be recorded into a graph by its caller)
+    if ((e = spatha::launch_clear_words((uint32_t*)base, 256, (hipStream_t)stream)) != hipSuccess) return spatha::note_hip_error(e);
     if ((e = spatha::plan_pack(&plan, values_dev, metadata_dev, columns_dev, (hipStream_t)stream)) != hipSuccess)
         return spatha::note_hip_error(e);
     return spatha::plan_run(&plan, B_dev, N, bias_dev, out_dev, out_layout, SPATHA_ACT_NONE, false, 0, stream);

@@ -35,9 +35,13 @@ __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk&
     static_assert(64 % (RPI * NP) == 0 && A_INSTR % NP == 0, "DMA work must split evenly over the producers");
     static_assert((PA - 1) * LOADS < 64, "vmcnt range");
 
-    const int S = p.S, N = p.N;
-    const int Q = walk.my_tiles * S;
+    // k-split: the walk's m-tiles are (row tile, part) pairs, vm = row tile * KS + part, and a part is SC = S / KS k-steps
+    // starting at step part * SC (KS = 1: the whole k-loop, vm = row tile)
+    const int S = p.S, N = p.N, KS = p.ksplit, SC = S / KS;
+    const int Q = walk.my_tiles * SC;
     const int tiles_per_vblock = p.v / BM;
+    auto rt_offset = [&](int vm) { return (uint32_t)(((vm / KS) / tiles_per_vblock) * S + (vm % KS) * SC) * 256u; };
+    auto a_offset = [&](int vm) { return (uint32_t)(((vm / KS) * WM) * S + (vm % KS) * SC) * (uint32_t)APACK_BLOCK; };
     const i32x4 rsrc_b = make_buffer(p.B, p.b_bytes);
     const i32x4 rsrc_a = make_buffer(p.apack, p.apack_bytes);
     const i32x4 rsrc_rt = make_buffer(p.rowtab, p.rowtab_bytes);
@@ -57,8 +61,8 @@ __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk&
     uint32_t is_stage = 0;
     uint32_t rt_read = 0;
     int rt_tm = walk.tm0, rt_tn = walk.tn0, rt_step = 0, rt_left = Q - 1;
-    uint32_t rt_soff = (uint32_t)((rt_tm / tiles_per_vblock) * S) * 256u;
-    uint32_t a_soff = (uint32_t)((is_tm * WM) * S) * (uint32_t)APACK_BLOCK;    // wave-tile row 0 of the tile
+    uint32_t rt_soff = rt_offset(rt_tm);
+    uint32_t a_soff = a_offset(is_tm);    // wave-tile row 0 of the tile, first step of the part
     uint32_t coloff[NB_LOADS];
     auto set_coloff = [&]() {
 #pragma unroll
@@ -72,10 +76,10 @@ __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk&
         if (rt_left > 0) {
             --rt_left;
             rt_soff += 256u;
-            if (++rt_step == S) {
+            if (++rt_step == SC) {
                 rt_step = 0;
                 walk.next(rt_tm, rt_tn);
-                rt_soff = (uint32_t)((rt_tm / tiles_per_vblock) * S) * 256u;
+                rt_soff = rt_offset(rt_tm);
             }
         }
     };
@@ -105,10 +109,10 @@ __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk&
         is_stage = (is_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : is_stage + STAGE_BYTES;
         rt_read = (rt_read == (uint32_t)PA * 256u) ? 0u : rt_read + 256u;
         a_soff += (uint32_t)APACK_BLOCK;
-        if (++is_step == S) {
+        if (++is_step == SC) {
             is_step = 0;
             walk.next(is_tm, is_tn);
-            a_soff = (uint32_t)((is_tm * WM) * S) * (uint32_t)APACK_BLOCK;
+            a_soff = a_offset(is_tm);
             set_coloff();
         }
     };
@@ -118,11 +122,11 @@ __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk&
         int st_tm = walk.tm0, st_tn = walk.tn0, st_step = 0;
 #pragma unroll
         for (int t = 0; t < PA; t++) {
-            const int64_t base = ((int64_t)(st_tm / tiles_per_vblock) * S + st_step) * 64;
+            const int64_t base = ((int64_t)((st_tm / KS) / tiles_per_vblock) * S + (st_tm % KS) * SC + st_step) * 64;
 #pragma unroll
             for (int j = 0; j < NB_LOADS; j++)
                 rows0[t][j] = (t < Q) ? p.rowtab[base + (PR * NB_LOADS + j) * RPI + slot_row] : 0xffffffffu;
-            if (++st_step == S) { st_step = 0; walk.next(st_tm, st_tn); }
+            if (++st_step == SC) { st_step = 0; walk.next(st_tm, st_tn); }
         }
 #pragma unroll
         for (int t = 0; t < PA; t++) rt_advance();
@@ -152,12 +156,54 @@ __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk&
     if (FINAL_BARRIER) __syncthreads();     // (kernels with store waves: the last tile's hand-over)
 }
 
+// k-split hand-over of one wave's 64 x 64 block (KS parts of a tile's k-loop, each computed by another workgroup): the wave
+// stores its fp32 partial block and takes a ticket; the wave that draws the last ticket adds the parts up IN PART ORDER (its
+// own from registers, the others from memory), so the sum does not depend on which part arrives last, and returns true: it
+// owns the block's write-out.  No wave ever waits for another.
+// The parts of a tile may run on different XCDs, whose L2s do not see each other's lines: partial blocks are written and
+// read with the device-scope cache policy (sc1: through the L2 to the memory side), the stores are complete (vmcnt) before
+// the ticket is drawn with a device-scope atomic, and the loads are issued behind it.  A device-scope FENCE would do as well
+// and costs far more: it writes back and invalidates the XCD's whole L2 (1024 x 4096 x 2048 at 128:2:8: 39.7 us with
+// fences, 16.4 us unsplit).
+// `slot` = index of the (tile, block) among the launch's blocks; partial: [slot][part][16][64] float4; tickets: [slot], zero
+// at launch; the wave that draws the last ticket puts the zero back, so a workspace that was cleared once stays usable.
+__device__ __forceinline__ bool ksplit_exchange(float4_t (&acc)[4][4], const SpmmParams& p, int64_t slot, int part, int lane) {
+    const int KS = p.ksplit;
+    constexpr int SC1 = 16;         // cache policy bit of the buffer instructions: device scope
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)p.partial, 0, (int)p.partial_bytes, 0x00020000);
+    const uint32_t block0 = (uint32_t)(slot * KS) * 16384u + (uint32_t)lane * 16u;     // part 0 of this block, this lane
+    const uint32_t mine = block0 + (uint32_t)part * 16384u;
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i >> 2][i & 3]), rsrc, (int)(mine + i * 1024), 0, SC1);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");          // the stores have completed (a wait, no cache operation)
+    uint32_t ticket = 0;
+    if (lane == 0) ticket = __hip_atomic_fetch_add(p.tickets + slot, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ticket = (uint32_t)__builtin_amdgcn_readfirstlane((int)ticket);
+    if (ticket != (uint32_t)(KS - 1)) return false;
+    if (lane == 0) __hip_atomic_store(p.tickets + slot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");          // (keeps the loads below behind the ticket)
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        float4_t t = acc[i >> 2][i & 3];
+        if (part != 0) t = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(block0 + i * 1024), 0, SC1));
+        for (int q = 1; q < KS; q++) {
+            float4_t v = acc[i >> 2][i & 3];
+            if (q != part)
+                v = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(block0 + q * 16384 + i * 1024), 0, SC1));
+            t += v;
+        }
+        acc[i >> 2][i & 3] = t;
+    }
+    return true;
+}
+
 template <class Cfg, int WN, int OUT_LAYOUT>
 __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
     constexpr int EPI_PITCH = Cfg::EPI_PITCH;
-    const int S = p.S, N = p.N;
+    const int S = p.S, N = p.N, KS = p.ksplit, SC = S / KS;
     const int wm = wave / WN, wn = wave - wm * WN;
     float4_t acc[4][4];
     const int li = lane & 15, kb = lane >> 4;
@@ -174,17 +220,22 @@ __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk&
     const int j16 = lane & 15, ib = lane >> 4;
     int c_tm = walk.tm0, c_tn = walk.tn0;
     uint32_t c_stage = 0;
-    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++) {
+    for (int c_tile = 0; c_tile < walk.my_tiles; c_tile++, walk.next(c_tm, c_tn)) {
 #pragma unroll
         for (int a = 0; a < 4; a++)
 #pragma unroll
             for (int b = 0; b < 4; b++) acc[a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
-        for (int c_step = 0; c_step < S; c_step++) {
+        for (int c_step = 0; c_step < SC; c_step++) {
             __syncthreads();
             if (!SPATHA_KNOB(16)) mma_stage<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc, [&]() {});
             c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
         }
-        const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+        const int r_tm = c_tm / KS;          // row tile (the walk's m index counts (row tile, part) pairs)
+        if (KS > 1) {
+            const int64_t slot = ((int64_t)c_tn * (walk.tiles_m / KS) + r_tm) * Cfg::NC + wave;
+            if (!ksplit_exchange(acc, p, slot, c_tm - r_tm * KS, lane)) continue;      // another part's wave writes the block
+        }
+        const int cm0 = r_tm * BM, cn0 = c_tn * BN;
         if (p.fuse) fused_bias_act(acc, p.bias, (int64_t)cm0 + wm * 64 + ib * 16, p.act);
         const uint16_t* bias = p.fuse ? nullptr : p.bias;
         if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
@@ -212,7 +263,6 @@ __device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk&
                 __builtin_amdgcn_wave_barrier();
             }
         }
-        walk.next(c_tm, c_tn);
     }
 }
 
@@ -350,7 +400,7 @@ __device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const Tile
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
     constexpr int EPI_PITCH = Cfg::EPI_PITCH;
     static_assert(BM == 128, "two stacked 64-row halves");
-    const int S = p.S, N = p.N;
+    const int S = p.S, N = p.N, KS = p.ksplit, SC = S / KS;
     const int wn = wave;
     float4_t acc[2][4][4];
     const int li = lane & 15, kb = lane >> 4;
@@ -374,14 +424,19 @@ __device__ __forceinline__ void ws_consumer_tall(const SpmmParams& p, const Tile
             for (int a = 0; a < 4; a++)
 #pragma unroll
                 for (int b = 0; b < 4; b++) acc[h][a][b] = (float4_t){0.f, 0.f, 0.f, 0.f};
-        for (int c_step = 0; c_step < S; c_step++) {
+        for (int c_step = 0; c_step < SC; c_step++) {
             __syncthreads();
             if (!SPATHA_KNOB(16)) mma_stage_tall<ROW_BYTES>(smem + c_stage, a_off, i_off, tr_off, acc);
             c_stage = (c_stage + STAGE_BYTES == NS * STAGE_BYTES) ? 0u : c_stage + STAGE_BYTES;
         }
-        const int cm0 = c_tm * BM, cn0 = c_tn * BN;
+        const int r_tm = c_tm / KS;          // row tile (the walk's m index counts (row tile, part) pairs)
+        const int cm0 = r_tm * BM, cn0 = c_tn * BN;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
+            if (KS > 1) {       // the wave's two 64 x 64 blocks are handed over separately: 2 * WN blocks per tile
+                const int64_t slot = ((int64_t)c_tn * (walk.tiles_m / KS) + r_tm) * (2 * WN) + wave * 2 + h;
+                if (!ksplit_exchange(acc[h], p, slot, c_tm - r_tm * KS, lane)) continue;
+            }
             if (p.fuse) fused_bias_act(acc[h], p.bias, (int64_t)cm0 + h * 64 + ib * 16, p.act);
             if (OUT_LAYOUT == SPATHA_OUT_TRANSPOSED) {
                 if (!SPATHA_KNOB(4))

@@ -56,16 +56,25 @@ class SpmmPlan:
                                                  columns.data_ptr(), _stream_ptr(self.device), ctypes.byref(handle)),
                        "spatha_spmm_plan_create")
         self._handle = handle
+        self._workspaces = {}          # stream -> zero-initialised scratch tensor of split runs
         self._finalizer = weakref.finalize(self, L.spatha_spmm_plan_destroy, handle)
 
     def kernel_name(self, N, out_layout=OUT_ROW_MAJOR, variant=0):
         name = _lib.lib().spatha_spmm_kernel_name(self._handle, N, out_layout, variant)
         return None if name is None else name.decode()
 
-    def run(self, B, bias=None, transposed_out=False, variant=0, out=None, activation=None):
+    def workspace_bytes(self, N, transposed_out=False, fused=False):
+        """Bytes of scratch memory with which `run(..., split=True)` would split k-loops for N columns (0: never for this shape)."""
+        return int(_lib.lib().spatha_spmm_workspace_bytes(self._handle, N, OUT_TRANSPOSED if transposed_out else OUT_ROW_MAJOR,
+                                                          1 if fused else 0))
+
+    def run(self, B, bias=None, transposed_out=False, variant=0, out=None, activation=None, split=False, workspace=None):
         """C = A B (or its transpose), fp16.  Without `activation`, a bias needs the transposed layout (the
         reference operator's contract).  With `activation` given ("none", "gelu", "gelu_tanh") the call goes through
-        the fused entry point: out = act(fp16(A B) + bias) in either layout."""
+        the fused entry point: out = act(fp16(A B) + bias) in either layout.
+        split=True (automatic kernel choice only) lets the library split k-loops over workgroups where tiles alone leave CUs
+        idle; the scratch memory it needs is `workspace` (a uint8 tensor on the GPU that was zero-filled once, e.g. by
+        torch.zeros) or, if None, a buffer the plan keeps per stream."""
         _check_dev(B, torch.float16, "rhs")
         if B.dim() != 2 or B.shape[0] != self.cols:
             raise ValueError("rhs must be [%d, N], got %s" % (self.cols, tuple(B.shape)))
@@ -82,6 +91,29 @@ class SpmmPlan:
             if tuple(out.shape) != shape:
                 raise ValueError("out must be %s" % (shape,))
         layout = OUT_TRANSPOSED if transposed_out else OUT_ROW_MAJOR
+        if split:
+            if variant != 0:
+                raise ValueError("split=True goes with the automatic kernel choice (variant=0)")
+            if activation is None and bias is not None and not transposed_out:
+                raise RuntimeError("spatha_spmm_run: a bias needs the transposed layout (or an activation argument)")
+            act = "none" if activation is None else activation
+            if act not in _ACTIVATIONS:
+                raise ValueError("unknown activation %r" % (activation,))
+            fused = _ACTIVATIONS[act] != ACT_NONE or (bias is not None and not transposed_out)
+            need = self.workspace_bytes(N, transposed_out, fused)
+            if workspace is None and need:
+                key = torch.cuda.current_stream(self.device).cuda_stream
+                workspace = self._workspaces.get(key)
+                if workspace is None or workspace.numel() < need:
+                    workspace = self._workspaces[key] = torch.zeros(need, dtype=torch.uint8, device=B.device)
+            ws_ptr = None if workspace is None else workspace.data_ptr()
+            ws_len = 0 if workspace is None else workspace.numel() * workspace.element_size()
+            with torch.cuda.device(self.device):
+                _lib.check(_lib.lib().spatha_spmm_run_ws(self._handle, B.data_ptr(), N, None if bias is None else bias.data_ptr(),
+                                                         out.data_ptr(), layout, _ACTIVATIONS[act], ws_ptr, ws_len,
+                                                         _stream_ptr(self.device)), "spatha_spmm_run_ws")
+            torch.autograd.graph.increment_version(out)
+            return out
         with torch.cuda.device(self.device):
             if activation is None:
                 _lib.check(_lib.lib().spatha_spmm_run(self._handle, B.data_ptr(), N,

@@ -164,7 +164,8 @@ __device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk&
 // read with the device-scope cache policy (sc1: through the L2 to the memory side), the stores are complete (vmcnt) before
 // the ticket is drawn with a device-scope atomic, and the loads are issued behind it.  A device-scope FENCE would do as well
 // and costs far more: it writes back and invalidates the XCD's whole L2 (1024 x 4096 x 2048 at 128:2:8: 39.7 us with
-// fences, 16.4 us unsplit).
+// fences, 21.2 us this way, 16.4 us unsplit).  Weaker cache policies (L2-local loads, write-back stores) measure the same
+// as these on every shape tried: the hand-over's 4-8 us are its three dependent round trips, not its cache traffic.
 // `slot` = index of the (tile, block) among the launch's blocks; partial: [slot][part][16][64] float4; tickets: [slot], zero
 // at launch; the wave that draws the last ticket puts the zero back, so a workspace that was cleared once stays usable.
 __device__ __forceinline__ bool ksplit_exchange(float4_t (&acc)[4][4], const SpmmParams& p, int64_t slot, int part, int lane) {

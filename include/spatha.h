@@ -265,6 +265,14 @@ int spatha_transpose_f16(const uint16_t* in_dev, int rows, int cols, uint16_t* o
 int spatha_add_layernorm_f16(const uint16_t* x_dev, const uint16_t* residual_dev, const uint16_t* gamma_dev,
                              const uint16_t* beta_dev, float eps, int tokens, int hidden, uint16_t* out_dev, void* stream);
 
+/* spatha_add_layernorm_f16 that writes its result twice: out[tokens][hidden] as above and out_t[hidden][tokens], the
+ * feature-major copy a following spatha_spmm_run takes as its B operand - the copy the reference's layer makes with
+ * `x.T.contiguous()` in front of every SpMM (end2end/bert_pytorch.py:87, :130-134), here written by the kernel that
+ * already holds the values.  tokens % 8 == 0 as well. */
+int spatha_add_layernorm_f16_t(const uint16_t* x_dev, const uint16_t* residual_dev, const uint16_t* gamma_dev,
+                               const uint16_t* beta_dev, float eps, int tokens, int hidden, uint16_t* out_dev, uint16_t* out_t_dev,
+                               void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -319,6 +319,73 @@ def test_add_layernorm_matches_torch_addition_and_layer_norm(gpu, tokens, hidden
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tokens,hidden,with_residual", [(16384, 1024, True), (304, 1024, False), (64, 1280, True), (40, 4096, True),
+                                                          (8, 8, True), (72, 72, False), (1000, 512, True)])
+def test_add_layernorm_feature_major_copy(gpu, tokens, hidden, with_residual):
+    """The variant that writes its result twice: the row-major output equals the plain kernel's bit for bit, the second output is
+    its transpose, and nothing is written outside either (guard bands)."""
+    from venom_amd import _lib, spatha
+    import ctypes
+
+    print("layer norm, feature-major copy", tokens, hidden, with_residual, flush=True)
+    g = torch.Generator(device=gpu)
+    g.manual_seed(tokens * 31 + hidden)
+    x = (torch.randn((tokens, hidden), generator=g, device=gpu) * 1.5 + 0.3).half()
+    r = torch.randn((tokens, hidden), generator=g, device=gpu).half() if with_residual else None
+    w = (1.0 + 0.1 * torch.randn(hidden, generator=g, device=gpu)).half()
+    b = (0.1 * torch.randn(hidden, generator=g, device=gpu)).half()
+    want = spatha.add_layernorm(x, r, w, b, 1e-12)
+    out, out_t = spatha.add_layernorm(x, r, w, b, 1e-12, feature_major=True)
+    assert tuple(out_t.shape) == (hidden, tokens) and out_t.is_contiguous()
+    assert torch.equal(out, want) and torch.equal(out_t, want.t())
+    # through the C ABI into buffers with guard bands
+    guard = 2048
+    n = tokens * hidden
+    buf = torch.full((2 * n + 3 * guard,), 7.0, dtype=torch.float16, device=gpu)
+    o1, o2 = buf[guard:guard + n], buf[2 * guard + n:2 * guard + 2 * n]
+    stream = ctypes.c_void_p(torch.cuda.current_stream(gpu).cuda_stream)
+    _lib.check(_lib.lib().spatha_add_layernorm_f16_t(x.data_ptr(), None if r is None else r.data_ptr(), w.data_ptr(), b.data_ptr(), 1e-12,
+                                                     tokens, hidden, o1.data_ptr(), o2.data_ptr(), stream), "ln_t")
+    torch.cuda.synchronize()
+    assert torch.equal(o1.view(tokens, hidden), want) and torch.equal(o2.view(hidden, tokens), want.t())
+    assert bool((buf[:guard] == 7.0).all()) and bool((buf[guard + n:2 * guard + n] == 7.0).all()) and bool((buf[2 * guard + 2 * n:] == 7.0).all())
+    if tokens == 8:
+        with pytest.raises(_lib.SpathaError):           # tokens % 8
+            spatha.add_layernorm(x[:5].contiguous(), None, w, b, 1e-12, feature_major=True)
+
+
+@pytest.mark.gpu
+def test_feature_major_layer_norm_feeds_the_next_projection(gpu):
+    """The encoder with the residual + LayerNorm kernel handing its feature-major copy to the next SrnmSpmm: same output as with the
+    plain fused kernel (the projections read the same numbers, only who transposes them changes), and the library's transpose kernel
+    runs once per layer instead of three times."""
+    from venom_amd import spatha
+    from venom_amd.bert import build_bert_large, fuse_add_layernorm, linear_to_spmm
+
+    torch.set_grad_enabled(False)
+    torch.manual_seed(3)
+    plain = fuse_add_layernorm(linear_to_spmm(build_bert_large(layers=2).to(gpu).half(), 2, 8, 64))
+    torch.manual_seed(3)
+    handed = fuse_add_layernorm(linear_to_spmm(build_bert_large(layers=2).to(gpu).half(), 2, 8, 64), feature_major=True)
+    ids = torch.randint(0, 30522, (2, 64), device=gpu)
+    calls = []
+    real = spatha.transpose
+    try:
+        spatha.transpose = lambda t: (calls.append(tuple(t.shape)), real(t))[1]
+        a = plain(ids).last_hidden_state
+        n_plain = len(calls)
+        calls.clear()
+        b = handed(ids).last_hidden_state
+        n_handed = len(calls)
+    finally:
+        spatha.transpose = real
+    assert torch.equal(a, b)
+    # per layer: q/k/v input, attention context, FFN-up input, FFN-down input -> the first layer keeps all but one (its q/k/v input
+    # comes from the embeddings), every later layer keeps the context and the FFN-down input only
+    assert n_plain == 8 and n_handed == 5, (n_plain, n_handed)
+
+
+@pytest.mark.gpu
 def test_add_layernorm_rejects_what_the_kernel_does_not_take(gpu):
     from venom_amd import _lib, spatha
 

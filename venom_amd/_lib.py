@@ -61,6 +61,7 @@ SIGNATURES = {
     "spatha_vnm_file_read": (c_int, [c_char_p, c_void_p, c_void_p, c_void_p]),
     "spatha_transpose_f16": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "spatha_add_layernorm_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_void_p, c_void_p]),
+    "spatha_add_layernorm_f16_t": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p]),
 }
 
 _lib = None

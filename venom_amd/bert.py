@@ -86,6 +86,14 @@ class SrnmSpmm(torch.nn.Module):
         cls._last_rhs = (key, flat, rhs)
         return rhs
 
+    @classmethod
+    def offer_transposed(cls, x, x_t):
+        """A producer that has x[..., features] feature-major already (x_t[features, tokens]) leaves it for the layer that reads
+        x next, in place of the transposed copy that layer would make."""
+        flat = torch.flatten(x, start_dim=0, end_dim=-2)
+        key = (flat.data_ptr(), tuple(flat.shape), tuple(flat.stride()), flat._version, flat.device)
+        cls._last_rhs = (key, flat, x_t)
+
     _group = None          # set by merge_qkv: the projections this layer is computed together with
     _group_index = 0
 
@@ -217,9 +225,11 @@ class FusedProjectionNorm(torch.nn.Module):
     projection may be an nn.Linear or an SrnmSpmm.  In training, or for tensors the kernel does not take, the stock
     sequence runs."""
 
-    def __init__(self, mod):
+    def __init__(self, mod, feature_major=False):
         super().__init__()
         self.dense, self.LayerNorm, self.dropout = mod.dense, mod.LayerNorm, mod.dropout
+        # also write the result feature-major and hand that copy to the next SrnmSpmm (which would otherwise transpose it)
+        self.feature_major = feature_major
         self.train(mod.training)
 
     def forward(self, hidden_states, input_tensor):
@@ -228,17 +238,23 @@ class FusedProjectionNorm(torch.nn.Module):
         if self.training or not h.is_cuda or h.dtype != torch.float16 or h.shape[-1] % 8 or h.shape[-1] > 4096 \
                 or ln.weight is None or ln.bias is None:
             return ln(self.dropout(h) + input_tensor)
-        return spatha.add_layernorm(h.contiguous(), input_tensor.contiguous(), ln.weight, ln.bias, ln.eps)
+        h = h.contiguous()
+        if self.feature_major and (h.numel() // h.shape[-1]) % 8 == 0:
+            out, out_t = spatha.add_layernorm(h, input_tensor.contiguous(), ln.weight, ln.bias, ln.eps, feature_major=True)
+            SrnmSpmm.offer_transposed(out, out_t)
+            return out
+        return spatha.add_layernorm(h, input_tensor.contiguous(), ln.weight, ln.bias, ln.eps)
 
 
-def fuse_add_layernorm(model):
-    """Replaces, in place, every BertSelfOutput / BertOutput by FusedProjectionNorm (same parameters)."""
+def fuse_add_layernorm(model, feature_major=False):
+    """Replaces, in place, every BertSelfOutput / BertOutput by FusedProjectionNorm (same parameters).  feature_major: for a
+    model whose projections are SrnmSpmm layers - the kernel also writes the feature-major copy the next projection reads."""
     from transformers.models.bert.modeling_bert import BertOutput, BertSelfOutput
 
     for mod in model.modules():
         for name, child in list(mod.named_children()):
             if isinstance(child, (BertSelfOutput, BertOutput)):
-                setattr(mod, name, FusedProjectionNorm(child))
+                setattr(mod, name, FusedProjectionNorm(child, feature_major))
     return model
 
 
@@ -287,22 +303,25 @@ def main(argv=None):
     ap.add_argument("--fuse-ln", action="store_true",
                     help="residual addition + LayerNorm after the attention-output and FFN-down projections as one kernel, "
                          "in BOTH models (the fusion does not depend on the weight format)")
+    ap.add_argument("--ln-feature-major", action="store_true",
+                    help="with --fuse-ln: the V:N:M model's residual + LayerNorm kernel also writes its result feature-major, the "
+                         "layout the next projection reads (two of the three transposed copies per layer disappear)")
     ap.add_argument("--kernel-gelu", action="store_true",
                     help="with --fuse-ffn: GELU in the kernel's write-out too (default: torch's elementwise pass over the "
                          "feature-major buffer, which keeps the model's output bit-identical to the unfused layers)")
     args = ap.parse_args(argv)
     r = measure(args.n, args.m, args.v, layers=args.layers, batch=args.batch, seq=args.seq, repeats=args.repeats,
                 magnitude=args.magnitude, fuse_ffn=args.fuse_ffn, merge=args.merge_qkv, fuse_ln=args.fuse_ln,
-                kernel_gelu=args.kernel_gelu, report=True)
+                kernel_gelu=args.kernel_gelu, report=True, ln_feature_major=args.ln_feature_major)
     print("# dense %.2f ms, %d:%d:%d%s %.2f ms, speed-up %.2fx" % (r["dense_ms"], args.v, args.n, args.m,
                                                                     ((" (fused feed-forward%s)" % (", activation in the kernel" if args.kernel_gelu else "")) if args.fuse_ffn else "")
                                                                     + (" (merged q/k/v)" if args.merge_qkv else "")
-                                                                    + (" (fused add + LayerNorm in both)" if args.fuse_ln else ""), r["vnm_ms"],
+                                                                    + (" (fused add + LayerNorm in both%s)" % (", feature-major copy for the next projection" if args.ln_feature_major else "") if args.fuse_ln else ""), r["vnm_ms"],
                                                                     r["speedup"]))
 
 
 def measure(n=2, m=8, v=64, layers=24, batch=32, seq=512, repeats=30, warmups=5, magnitude=False, fuse_ffn=False, merge=False,
-            fuse_ln=False, kernel_gelu=False, report=False):
+            fuse_ln=False, kernel_gelu=False, report=False, ln_feature_major=False):
     """Times the dense fp16 encoder and the same encoder with its Linears in V:N:M on cuda:0 (the reference's procedure,
     end2end/bert_pytorch.py:211-219: warm-ups, then `repeats` forward passes timed one by one, each ended by a device
     synchronisation); returns mean and median milliseconds of both and their ratio."""
@@ -321,7 +340,7 @@ def measure(n=2, m=8, v=64, layers=24, batch=32, seq=512, repeats=30, warmups=5,
             merge_qkv(sparse_model)
         if fuse_ln:
             fuse_add_layernorm(dense_model)
-            fuse_add_layernorm(sparse_model)
+            fuse_add_layernorm(sparse_model, feature_major=ln_feature_major)
         ids = torch.randint(0, 30522, (batch, seq), device=dev)
 
         def run(model):

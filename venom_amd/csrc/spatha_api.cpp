@@ -742,4 +742,18 @@ int spatha_add_layernorm_f16(const uint16_t* x_dev, const uint16_t* residual_dev
     return e == hipSuccess ? SPATHA_OK : hip_fail(e);
 }
 
+int spatha_add_layernorm_f16_t(const uint16_t* x_dev, const uint16_t* residual_dev, const uint16_t* gamma_dev,
+                               const uint16_t* beta_dev, float eps, int tokens, int hidden, uint16_t* out_dev, uint16_t* out_t_dev,
+                               void* stream) {
+    if (!x_dev || !gamma_dev || !beta_dev || !out_dev || !out_t_dev || tokens <= 0 || hidden <= 0) return SPATHA_ERR_BAD_ARGUMENT;
+    if (hidden % 8 != 0 || tokens % 8 != 0) return SPATHA_ERR_BAD_SHAPE;       // 16-byte pieces of both layouts
+    if (hidden > 4096) return SPATHA_ERR_UNSUPPORTED;
+    if (((uintptr_t)x_dev | (uintptr_t)residual_dev | (uintptr_t)gamma_dev | (uintptr_t)beta_dev | (uintptr_t)out_dev |
+         (uintptr_t)out_t_dev) & 15u)
+        return SPATHA_ERR_BAD_ARGUMENT;
+    hipError_t e = spatha::launch_add_layernorm_f16_t(x_dev, residual_dev, gamma_dev, beta_dev, eps, tokens, hidden, out_dev, out_t_dev,
+                                                      (hipStream_t)stream);
+    return e == hipSuccess ? SPATHA_OK : hip_fail(e);
+}
+
 }  // extern "C"

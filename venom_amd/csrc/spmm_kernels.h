@@ -105,6 +105,9 @@ hipError_t launch_transpose_f16(const uint16_t* in, int rows, int cols, uint16_t
 hipError_t launch_add_layernorm_f16(const uint16_t* x, const uint16_t* residual, const uint16_t* gamma, const uint16_t* beta,
                                     float eps, int tokens, int hidden, uint16_t* out, hipStream_t stream);
 
+hipError_t launch_add_layernorm_f16_t(const uint16_t* x, const uint16_t* residual, const uint16_t* gamma, const uint16_t* beta,
+                                      float eps, int tokens, int hidden, uint16_t* out, uint16_t* out_t, hipStream_t stream);
+
 hipError_t launch_dense_gemm(const uint16_t* A, const uint16_t* B, int rows, int cols, int N, uint16_t* C,
                              hipStream_t stream);
 

@@ -179,10 +179,12 @@ def transpose(x):
     return out
 
 
-def add_layernorm(x, residual, weight, bias, eps):
+def add_layernorm(x, residual, weight, bias, eps, feature_major=False):
     """LayerNorm(x + residual) over the last dimension in one kernel (residual may be None): fp16 tensors on the GPU,
     x and residual contiguous and of the same shape, weight and bias of length x.shape[-1] (a multiple of 8, at most
-    4096).  Same arithmetic as torch's addition followed by torch.nn.functional.layer_norm on fp16 tensors."""
+    4096).  Same arithmetic as torch's addition followed by torch.nn.functional.layer_norm on fp16 tensors.
+    feature_major=True returns (out, out_t): the kernel also writes the result as [hidden, tokens] (tokens a multiple
+    of 8), which the next V:N:M projection takes as its right-hand side without a transposed copy."""
     _check_dev(x, torch.float16, "x")
     hidden = x.shape[-1]
     if residual is not None:
@@ -194,6 +196,15 @@ def add_layernorm(x, residual, weight, bias, eps):
     if weight.numel() != hidden or bias.numel() != hidden:
         raise ValueError("weight and bias must have x.shape[-1] elements")
     out = torch.empty_like(x)
+    if feature_major:
+        tokens = x.numel() // hidden
+        out_t = torch.empty((hidden, tokens), dtype=torch.float16, device=x.device)
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.lib().spatha_add_layernorm_f16_t(x.data_ptr(), residual.data_ptr() if residual is not None else None,
+                                                             weight.data_ptr(), bias.data_ptr(), float(eps), tokens, hidden,
+                                                             out.data_ptr(), out_t.data_ptr(), _stream_ptr(x.device)),
+                       "spatha_add_layernorm_f16_t")
+        return out, out_t
     if x.numel():
         with torch.cuda.device(x.device):
             _lib.check(_lib.lib().spatha_add_layernorm_f16(x.data_ptr(), residual.data_ptr() if residual is not None else None,

@@ -132,6 +132,9 @@ def main():
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--value-std", type=float, default=0.02, help="standard deviation of A's non-zeros (BASELINE config 1: 1.0)")
     ap.add_argument("--b-uniform", action="store_true", help="B ~ U(-1, 1) instead of N(0, 1) (BASELINE config 1)")
+    ap.add_argument("--split", action="store_true",
+                    help="time the measured workload through spatha_spmm_run_ws (with a workspace: the library may split k-loops "
+                         "over workgroups) instead of spatha_spmm_run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--extra", action="store_true", help="also time three shapes outside BASELINE.json (appended to 'extra')")
     ap.add_argument("--ablation", action="store_true",
@@ -209,20 +212,29 @@ def main():
         stream = torch.cuda.current_stream(dev)
         sp = ctypes.c_void_p(stream.cuda_stream)
         settle_ms = args.settle_ms if settle_ms is None else settle_ms
+        if w.get("workspace") is not None:
+            ws = w["workspace"]
+
+            def launch():
+                _lib.check(L.spatha_spmm_run_ws(plan._handle, B.data_ptr(), B.shape[1], None, C.data_ptr(), 0, 0, ws.data_ptr(),
+                                                ws.numel(), sp), "run_ws")
+        else:
+            def launch():
+                _lib.check(L.spatha_spmm_run(plan._handle, B.data_ptr(), B.shape[1], None, C.data_ptr(), 0, variant, sp), "run")
         t_settle = time.perf_counter()
         while (time.perf_counter() - t_settle) * 1e3 < settle_ms:       # time based: the clock settles on work done, not on a count
             for _ in range(20):
-                _lib.check(L.spatha_spmm_run(plan._handle, B.data_ptr(), B.shape[1], None, C.data_ptr(), 0, variant, sp), "run")
+                launch()
             torch.cuda.synchronize()
         for _ in range(warmup):
-            _lib.check(L.spatha_spmm_run(plan._handle, B.data_ptr(), B.shape[1], None, C.data_ptr(), 0, variant, sp), "run")
+            launch()
         torch.cuda.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
         e0.record(stream)
         for _ in range(steps):
-            _lib.check(L.spatha_spmm_run(plan._handle, B.data_ptr(), B.shape[1], None, C.data_ptr(), 0, variant, sp), "run")
+            launch()
         e1.record(stream)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
@@ -238,6 +250,9 @@ def main():
 
     rows, cols, N, m, v = args.rows, args.cols, args.n, args.m, args.v
     w = prepare(rows, cols, N, m, v, value_std=args.value_std, b_uniform=args.b_uniform)
+    split_bytes = w["plan"].workspace_bytes(N) if args.split else 0
+    if split_bytes:
+        w["workspace"] = torch.zeros(split_bytes, dtype=torch.uint8, device=dev)
     ms_wall, ms_kernel = timed(w, args.steps, args.warmup, args.variant)
     ksp = w["geo"].ksp
     flops_dense = 2.0 * rows * cols * N
@@ -264,7 +279,8 @@ def main():
         "data": "synthetic (seed 0: A %d:2:%d random pattern, values ~N(0,%g); B ~%s)" % (v, m, args.value_std,
                                                                                             "U(-1,1)" if args.b_uniform else "N(0,1)"),
         "config": {"workload": "spmm A %dx%d %d:2:%d (Ksp %d) x B %dx%d, row-major C" % (rows, cols, v, m, ksp, cols, N),
-                   "kernel": w["plan"].kernel_name(N, 0, args.variant)},
+                   "kernel": w["plan"].kernel_name(N, 0, args.variant),
+                   "k_split_workspace_bytes": split_bytes},
         "pct_smfmac_peak": round(100.0 * flops_smfmac / (ms_kernel * 1e-3) / 1e12 / SMFMAC_PEAK_TFLOPS, 2),
         "roofline": {"bound": "hbm", "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved_gbs / HBM_PEAK_GBS, 4),

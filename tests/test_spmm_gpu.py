@@ -693,10 +693,9 @@ def test_run_time_errors(gpu):
     rows, cols, m, v = 128, 128, 8, 64
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=1, integer_values=True)
     plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
-    B = torch.zeros((cols, 20), dtype=torch.float16, device=gpu)     # N % 8 != 0
-    with pytest.raises(_lib.SpathaError) as e:
-        plan.run(B)
-    assert e.value.status == 2
+    B = torch.zeros((cols, 20), dtype=torch.float16, device=gpu)     # N % 8 != 0: the C entry point refuses it
+    out = torch.zeros((rows, 20), dtype=torch.float16, device=gpu)
+    assert _lib.lib().spatha_spmm_run(plan._handle, B.data_ptr(), 20, None, out.data_ptr(), 0, 0, None) == 2
     B = torch.zeros((cols, 16), dtype=torch.float16, device=gpu)
     with pytest.raises(_lib.SpathaError) as e:
         plan.run(B, variant=1)                                        # 128-row tile needs V % 128 == 0
@@ -704,3 +703,35 @@ def test_run_time_errors(gpu):
     with pytest.raises(_lib.SpathaError) as e:
         plan.run(B, bias=torch.zeros(rows, dtype=torch.float16, device=gpu))   # bias only with transposed output
     assert e.value.status == 1
+
+
+@pytest.mark.parametrize("N", [1, 20, 37, 263])
+def test_token_counts_that_are_no_multiple_of_8(gpu, N):
+    """The C entry points want N % 8 == 0; `SpmmPlan.run` and the operator run such a product on a zero-padded copy of the
+    right-hand side and cut the result back: same numbers as the oracle, both layouts, bias, fused bias."""
+    print("ragged token count", N, flush=True)
+    rows, cols, m, v = 256, 300, 10, 64
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=N, integer_values=True)
+    rng = np.random.default_rng(N)
+    B = rng.integers(-4, 5, size=(cols, N), dtype=np.int8).astype(np.float16)
+    bias = rng.integers(-8, 9, size=rows).astype(np.float16)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    dB, dbias = torch.from_numpy(B).to(gpu), torch.from_numpy(bias).to(gpu)
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B)
+    want_t = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias, transposed_out=True)
+    got = plan.run(dB)
+    assert got.shape == (rows, N) and got.is_contiguous()
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    got = plan.run(dB, bias=dbias, transposed_out=True)
+    assert got.shape == (N, rows) and got.is_contiguous()
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), want_t.view(np.uint16))
+    out = torch.full((rows, N), float("nan"), dtype=torch.float16, device=gpu)
+    assert plan.run(dB, bias=dbias, activation="none", out=out) is out
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), np.ascontiguousarray(want_t.T).view(np.uint16))
+    dv, dm, dc = _dev(vals, gpu), _dev(meta, gpu), _dev(columns, gpu)
+    got = spatha.spmm(dm, dc, dv, dB, dbias, rows, cols, N, v, 2, m)
+    assert got.shape == (N, rows) and got.is_contiguous()
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), want_t.view(np.uint16))
+    got = spatha.spmm_fused(dm, dc, dv, dB, dbias, rows, cols, v, 2, m)
+    assert got.shape == (rows, N) and got.is_contiguous()
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), np.ascontiguousarray(want_t.T).view(np.uint16))

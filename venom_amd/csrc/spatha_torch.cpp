@@ -149,6 +149,15 @@ torch::Tensor run(const torch::Tensor& A_metadata, const torch::Tensor& A_indice
     }
     const int tokens = (int)rhs_matrix.size(1);
     const c10::hip::HIPGuardMasqueradingAsCUDA device_guard(A_values.device());
+    if (tokens % 8 != 0 && tokens > 0) {
+        // The library moves rows of B and C in 16-byte pieces: a token count that is no multiple of 8 runs on a copy of
+        // rhs_matrix with zero columns appended, and the result is cut back (the appended columns give bias-only rows /
+        // columns, which are dropped).
+        const int pad = 8 - tokens % 8;
+        torch::Tensor padded = torch::constant_pad_nd(rhs_matrix, {0, pad}, 0);
+        torch::Tensor full = run(A_metadata, A_indices, A_values, padded, bias, rows, cols, v, n, m, transposed_out, activation, fused);
+        return transposed_out ? full.narrow(0, 0, tokens) : full.narrow(1, 0, tokens).contiguous();
+    }
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(A_values.get_device()).stream();
     // (this reference outlives the launch calls below, whatever another thread does to the cache meanwhile)
     const std::shared_ptr<spatha_spmm_plan> plan = plan_for(A_values.detach(), A_metadata, A_indices, rows, cols, n, m, v, stream);

@@ -83,6 +83,18 @@ class SpmmPlan:
             _check_dev(bias, torch.float16, "bias")
             if bias.numel() != self.rows:
                 raise ValueError("bias must have %d entries" % self.rows)
+        if N % 8 != 0 and N > 0:
+            # the library moves rows of B and C in 16-byte pieces: run on a copy with zero columns appended, cut the result back
+            full = self.run(torch.nn.functional.pad(B, (0, 8 - N % 8)), bias, transposed_out, variant, None, activation, split,
+                            workspace)
+            cut = full[:N] if transposed_out else full[:, :N]
+            if out is None:
+                return cut.contiguous()
+            _check_dev(out, torch.float16, "out")
+            if tuple(out.shape) != tuple(cut.shape):
+                raise ValueError("out must be %s" % (tuple(cut.shape),))
+            out.copy_(cut)
+            return out
         shape = (N, self.rows) if transposed_out else (self.rows, N)
         if out is None:
             out = torch.empty(shape, dtype=torch.float16, device=B.device)

@@ -4,8 +4,9 @@ Counterpart of the reference harness end2end/bert_pytorch.py (`NMVectorSparsifie
 `SrnmSpmm` :109-136, `linear_to_spmm` :155-167, timing :169-219).  Differences, on purpose:
 the model is built from a local `BertConfig` with random weights (no hub download), only
 `encoder.layer.*` Linears are swapped (the reference also swaps `pooler.dense`, whose 32-token
-input is narrower than its kernel's tile), and the STEN wrapper is replaced by a two-method
-stand-in because only `wrapped_from_dense(...)` / `.wrapped_tensor` are used.
+input is narrower than its kernel's tile), and where the STEN package is not installed its wrapper
+is replaced by a two-method stand-in (only `wrapped_from_dense(...)` / `.wrapped_tensor` are used;
+venom_amd/sten_registration.py holds it and the registration hooks for when STEN is there).
 
     python -m venom_amd.bert -m 8 -n 2 -v 64 [--layers 24] [--magnitude] [--repeats 30]
 prints `algo,n,m,v,mean_ms,median_ms,std_ms,len` rows for the dense and the V:N:M model."""
@@ -17,19 +18,7 @@ import torch
 
 from . import spatha
 from .grouped_nmv_tensor import SrNMTensor, nm_vector_mask_sparsify
-
-
-class SparseTensorWrapper:
-    """The part of sten.SparseTensorWrapper the harness uses."""
-
-    def __init__(self, wrapped_tensor, dense, grad_fmt=None):
-        self.wrapped_tensor = wrapped_tensor
-        self.dense_shape = tuple(dense.shape)
-        self.grad_fmt = grad_fmt
-
-    @staticmethod
-    def wrapped_from_dense(wrapped_tensor, dense, grad_fmt=None):
-        return SparseTensorWrapper(wrapped_tensor, dense, grad_fmt)
+from .sten_registration import SparseTensorWrapper, wrapper_class  # noqa: F401  (the stand-in keeps its old import path)
 
 
 class NMVectorSparsifier:
@@ -50,7 +39,7 @@ class NMVectorSparsifier:
             pat[0] = 1
             pat[2] = 1
             mask = pat.repeat(nrows, ncols // self.m)
-        return SparseTensorWrapper.wrapped_from_dense(
+        return wrapper_class().wrapped_from_dense(
             SrNMTensor(self.n, self.m, self.tileM, tensor, mask, columns, tensor.device), tensor, grad_fmt)
 
 

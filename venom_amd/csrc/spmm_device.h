@@ -372,10 +372,18 @@ struct WswCfg {
 // Tile walk shared by both roles: XCD x (= workgroup id % 8) owns a contiguous range of tile
 // ids (id -> n-tile major, m-tile minor) and its workgroups take them round robin; the
 // coordinates advance by a fixed (dm, dn) with carry, so no division per tile.
-struct TileWalk {
-    int my_tiles, tm0, tn0, step_dm, step_dn, tiles_m;
+// ROWS_FIRST: the XCD's tiles are consecutive in the order that runs through a tile row's column tiles first (tile index
+// tm * tiles_n + tn) instead of through a tile column's row tiles (tn * tiles_m + tm): the workgroups of an XCD then work on
+// few tile rows at a time, all their column tiles together - the packed A operands of a tile row enter that XCD's L2 once
+// instead of once per XCD that holds one of its column tiles.  Pays where a tile row of A is larger than a tile column of B
+// and there are few column tiles.
+template <bool ROWS_FIRST>
+struct TileWalkT {
+    int my_tiles, tm0, tn0, step_dm, step_dn, tiles_m, tiles_n;
     __device__ __forceinline__ void init(int tiles_m_, int tiles_n_) {
         tiles_m = tiles_m_;
+        tiles_n = tiles_n_;
+        const int fast = ROWS_FIRST ? tiles_n_ : tiles_m_;
         const int tiles = tiles_m_ * tiles_n_;
         const int chunk = (tiles + 7) >> 3;
         const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
@@ -383,17 +391,24 @@ struct TileWalk {
         const int last = (first + chunk) < tiles ? (first + chunk) : tiles;
         my_tiles = 0;
         if (first + slot < last) my_tiles = (last - first - slot + slots - 1) / slots;
-        step_dn = slots / tiles_m;
-        step_dm = slots - step_dn * tiles_m;
-        tn0 = (first + slot) / tiles_m;
-        tm0 = (first + slot) - tn0 * tiles_m;
+        const int step_slow = slots / fast, step_fast = slots - step_slow * fast;
+        const int slow0 = (first + slot) / fast, fast0 = (first + slot) - slow0 * fast;
+        step_dm = ROWS_FIRST ? step_slow : step_fast;
+        step_dn = ROWS_FIRST ? step_fast : step_slow;
+        tm0 = ROWS_FIRST ? slow0 : fast0;
+        tn0 = ROWS_FIRST ? fast0 : slow0;
     }
     __device__ __forceinline__ void next(int& tm, int& tn) const {
         tm += step_dm;
         tn += step_dn;
-        if (tm >= tiles_m) { tm -= tiles_m; tn += 1; }
+        if (ROWS_FIRST) {
+            if (tn >= tiles_n) { tn -= tiles_n; tm += 1; }
+        } else {
+            if (tm >= tiles_m) { tm -= tiles_m; tn += 1; }
+        }
     }
 };
+using TileWalk = TileWalkT<false>;
 
 // ---- deferred write-out -------------------------------------------------------------------
 // A finished 64 x 64 wave tile is rounded to fp16 pairs (32 registers) and written one quarter

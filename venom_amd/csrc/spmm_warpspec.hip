@@ -20,8 +20,8 @@ namespace spatha {
 // it comes to which DMA instructions of a stage it issues.
 // ---------------------------------------------------------------------------
 
-template <class Cfg, int NP, int PR, bool FINAL_BARRIER = false>
-__device__ __forceinline__ void ws_producer(const SpmmParams& p, const TileWalk& walk, char* smem, uint32_t smem_base,
+template <class Cfg, int NP, int PR, bool FINAL_BARRIER = false, class Walk = TileWalk>
+__device__ __forceinline__ void ws_producer(const SpmmParams& p, const Walk& walk, char* smem, uint32_t smem_base,
                                             int lane) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1, PA = Cfg::PA;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
@@ -199,8 +199,8 @@ __device__ __forceinline__ bool ksplit_exchange(float4_t (&acc)[4][4], const Spm
     return true;
 }
 
-template <class Cfg, int WN, int OUT_LAYOUT>
-__device__ __forceinline__ void ws_consumer(const SpmmParams& p, const TileWalk& walk, char* smem, int wave, int lane) {
+template <class Cfg, int WN, int OUT_LAYOUT, class Walk = TileWalk>
+__device__ __forceinline__ void ws_consumer(const SpmmParams& p, const Walk& walk, char* smem, int wave, int lane) {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, NS = Cfg::PA + 1;
     constexpr int ROW_BYTES = Cfg::ROW_BYTES, B_BYTES = Cfg::B_BYTES, STAGE_BYTES = Cfg::STAGE_BYTES;
     constexpr int EPI_PITCH = Cfg::EPI_PITCH;
@@ -518,15 +518,16 @@ static hipError_t launch_wst(const SpmmParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false>
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false, bool ROWS_FIRST = false>
 __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams p) {
     using Cfg = WsCfg<WM, WN, NS, NP>;
     static_assert(NP == 2 || NP == 4, "producer count");
+    static_assert(!(DEFER && ROWS_FIRST), "the deferred write-out walks column-first only");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    TileWalk walk;
+    TileWalkT<ROWS_FIRST> walk;
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
     // Workgroups of one XCD start up to 7 * skew apart, so that tiles do not all finish (and
@@ -536,7 +537,7 @@ __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams
         for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);      // 16 * 64 clocks
     }
     if (wave < Cfg::NC) {
-        if (DEFER) ws_consumer_deferred<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
+        if constexpr (DEFER) ws_consumer_deferred<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
         else ws_consumer<Cfg, WN, OUT_LAYOUT>(p, walk, smem, wave, lane);
     } else {
         // the producer index is a template argument: which DMA instructions a producer issues
@@ -549,13 +550,13 @@ __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams
     }
 }
 
-template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false>
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false, bool ROWS_FIRST = false>
 static hipError_t launch_ws(const SpmmParams& p, hipStream_t stream) {
     using Cfg = WsCfg<WM, WN, NS, NP>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     const int cus = p.cus;        // compute units of the plan's device
-    auto kern = spmm_ws_kernel<WM, WN, NS, NP, OUT_LAYOUT, DEFER>;
+    auto kern = spmm_ws_kernel<WM, WN, NS, NP, OUT_LAYOUT, DEFER, ROWS_FIRST>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -792,6 +793,9 @@ hipError_t launch_warpspec(int variant, int out_layout, const SpmmParams& p, hip
     const bool t = out_layout == SPATHA_OUT_TRANSPOSED;
     switch (variant) {
         case SPMM_VARIANT_W128x128_S3:
+            if (p.rows_first)
+                return t ? launch_ws<2, 2, 3, 4, SPATHA_OUT_TRANSPOSED, false, true>(p, stream)
+                         : launch_ws<2, 2, 3, 4, SPATHA_OUT_ROW_MAJOR, false, true>(p, stream);
             return t ? launch_ws<2, 2, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_ws<2, 2, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
         case SPMM_VARIANT_W128x256_S3:
             return t ? launch_ws<2, 4, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_ws<2, 4, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);

@@ -595,7 +595,7 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
     p.rowtab_bytes = (uint32_t)plan->rowtab_bytes;
     p.fuse = fuse ? 1 : 0; p.act = activation;
     p.cus = plan->cus > 0 ? plan->cus : 256;
-    p.rows_first = 0;
+    p.walk_group = 1;
     p.ksplit = 1; p.partial = nullptr; p.partial_bytes = 0; p.tickets = nullptr;
     p.debug = 0; p.skew = 0; p.prof = nullptr;
 #ifdef SPATHA_DEV_PROFILE
@@ -635,7 +635,7 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
         tail.tiles_n = (N + 127) / 128;
         // the two column tiles of a tile row on one XCD at the same time: its A operands (0.44 MB per tile row of the GPT-3
         // FFN matrix) enter one L2 instead of two
-        tail.rows_first = 1;
+        tail.walk_group = 0;
         hipError_t e2 = spatha::launch_spmm(var, out_layout, head, (hipStream_t)stream);
         if (e2 == hipSuccess) e2 = spatha::launch_spmm(spatha::SPMM_VARIANT_W128x128_S3, out_layout, tail, (hipStream_t)stream);
         return e2 == hipSuccess ? SPATHA_OK : hip_fail(e2);

@@ -372,18 +372,28 @@ struct WswCfg {
 // Tile walk shared by both roles: XCD x (= workgroup id % 8) owns a contiguous range of tile
 // ids (id -> n-tile major, m-tile minor) and its workgroups take them round robin; the
 // coordinates advance by a fixed (dm, dn) with carry, so no division per tile.
-// ROWS_FIRST: the XCD's tiles are consecutive in the order that runs through a tile row's column tiles first (tile index
-// tm * tiles_n + tn) instead of through a tile column's row tiles (tn * tiles_m + tm): the workgroups of an XCD then work on
-// few tile rows at a time, all their column tiles together - the packed A operands of a tile row enter that XCD's L2 once
-// instead of once per XCD that holds one of its column tiles.  Pays where a tile row of A is larger than a tile column of B
-// and there are few column tiles.
-template <bool ROWS_FIRST>
+// The tiles of a launch in walk order, eight consecutive chunks of them for the eight XCDs (workgroup id % 8), within a chunk
+// workgroup j of an XCD takes tiles j, j + workgroups, ...  The order decides what the workgroups of an XCD share in its L2.
+// GROUP == 1: through a tile column's row tiles, column after column (index tn * tiles_m + tm): the XCD works on one column
+// tile of B at a time and streams A past it.  GROUP == 0: through a tile row's column tiles first (index tm * tiles_n + tn),
+// GROUP == g > 1: the same within groups of g tile columns (tiles_n a multiple of g): the workgroups of an XCD then work on
+// fewer tile rows at a time, g column tiles of each - the packed A operands of a tile row enter that XCD's L2 once instead of
+// once per XCD that holds one of its column tiles.  Pays where tile rows of A are large against tile columns of B.
+template <int GROUP>
 struct TileWalkT {
-    int my_tiles, tm0, tn0, step_dm, step_dn, tiles_m, tiles_n;
+    int my_tiles, tm0, tn0, step_dm, step_dn, tiles_m, tiles_n, stride;
+    __device__ __forceinline__ int group() const { return GROUP == 0 ? tiles_n : GROUP; }
+    // tile number `t` of the walk -> tile coordinates (wave-uniform, kept in scalar registers: they end up in scalar operands)
+    __device__ __forceinline__ void locate(int t, int& tm, int& tn) const {
+        const int g = group(), per_group = tiles_m * g;
+        const int grp = t / per_group, rem = t - grp * per_group;
+        const int row = rem / g;
+        tm = __builtin_amdgcn_readfirstlane(row);
+        tn = __builtin_amdgcn_readfirstlane(grp * g + (rem - row * g));
+    }
     __device__ __forceinline__ void init(int tiles_m_, int tiles_n_) {
         tiles_m = tiles_m_;
         tiles_n = tiles_n_;
-        const int fast = ROWS_FIRST ? tiles_n_ : tiles_m_;
         const int tiles = tiles_m_ * tiles_n_;
         const int chunk = (tiles + 7) >> 3;
         const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
@@ -391,24 +401,29 @@ struct TileWalkT {
         const int last = (first + chunk) < tiles ? (first + chunk) : tiles;
         my_tiles = 0;
         if (first + slot < last) my_tiles = (last - first - slot + slots - 1) / slots;
-        const int step_slow = slots / fast, step_fast = slots - step_slow * fast;
-        const int slow0 = (first + slot) / fast, fast0 = (first + slot) - slow0 * fast;
-        step_dm = ROWS_FIRST ? step_slow : step_fast;
-        step_dn = ROWS_FIRST ? step_fast : step_slow;
-        tm0 = ROWS_FIRST ? slow0 : fast0;
-        tn0 = ROWS_FIRST ? fast0 : slow0;
+        stride = slots;
+        if constexpr (GROUP == 1) {
+            step_dn = slots / tiles_m;
+            step_dm = slots - step_dn * tiles_m;
+            tn0 = (first + slot) / tiles_m;
+            tm0 = (first + slot) - tn0 * tiles_m;
+        } else {
+            step_dm = step_dn = 0;
+            locate(first + slot, tm0, tn0);
+        }
     }
     __device__ __forceinline__ void next(int& tm, int& tn) const {
-        tm += step_dm;
-        tn += step_dn;
-        if (ROWS_FIRST) {
-            if (tn >= tiles_n) { tn -= tiles_n; tm += 1; }
-        } else {
+        if constexpr (GROUP == 1) {
+            tm += step_dm;
+            tn += step_dn;
             if (tm >= tiles_m) { tm -= tiles_m; tn += 1; }
+        } else {
+            const int g = group(), grp = tn / g;
+            locate(grp * tiles_m * g + tm * g + (tn - grp * g) + stride, tm, tn);
         }
     }
 };
-using TileWalk = TileWalkT<false>;
+using TileWalk = TileWalkT<1>;
 
 // ---- deferred write-out -------------------------------------------------------------------
 // A finished 64 x 64 wave tile is rounded to fp16 pairs (32 registers) and written one quarter

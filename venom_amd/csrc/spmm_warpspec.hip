@@ -518,16 +518,16 @@ static hipError_t launch_wst(const SpmmParams& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false, bool ROWS_FIRST = false>
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false, int WALK_GROUP = 1>
 __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams p) {
     using Cfg = WsCfg<WM, WN, NS, NP>;
     static_assert(NP == 2 || NP == 4, "producer count");
-    static_assert(!(DEFER && ROWS_FIRST), "the deferred write-out walks column-first only");
+    static_assert(!(DEFER && WALK_GROUP != 1), "the deferred write-out walks column-first only");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    TileWalkT<ROWS_FIRST> walk;
+    TileWalkT<WALK_GROUP> walk;
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
     // Workgroups of one XCD start up to 7 * skew apart, so that tiles do not all finish (and
@@ -550,13 +550,13 @@ __global__ __launch_bounds__((WM * WN + NP) * 64) void spmm_ws_kernel(SpmmParams
     }
 }
 
-template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false, bool ROWS_FIRST = false>
+template <int WM, int WN, int NS, int NP, int OUT_LAYOUT, bool DEFER = false, int WALK_GROUP = 1>
 static hipError_t launch_ws(const SpmmParams& p, hipStream_t stream) {
     using Cfg = WsCfg<WM, WN, NS, NP>;
     constexpr int lds = Cfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     const int cus = p.cus;        // compute units of the plan's device
-    auto kern = spmm_ws_kernel<WM, WN, NS, NP, OUT_LAYOUT, DEFER, ROWS_FIRST>;
+    auto kern = spmm_ws_kernel<WM, WN, NS, NP, OUT_LAYOUT, DEFER, WALK_GROUP>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
@@ -793,9 +793,9 @@ hipError_t launch_warpspec(int variant, int out_layout, const SpmmParams& p, hip
     const bool t = out_layout == SPATHA_OUT_TRANSPOSED;
     switch (variant) {
         case SPMM_VARIANT_W128x128_S3:
-            if (p.rows_first)
-                return t ? launch_ws<2, 2, 3, 4, SPATHA_OUT_TRANSPOSED, false, true>(p, stream)
-                         : launch_ws<2, 2, 3, 4, SPATHA_OUT_ROW_MAJOR, false, true>(p, stream);
+            if (p.walk_group == 0)
+                return t ? launch_ws<2, 2, 3, 4, SPATHA_OUT_TRANSPOSED, false, 0>(p, stream)
+                         : launch_ws<2, 2, 3, 4, SPATHA_OUT_ROW_MAJOR, false, 0>(p, stream);
             return t ? launch_ws<2, 2, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_ws<2, 2, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);
         case SPMM_VARIANT_W128x256_S3:
             return t ? launch_ws<2, 4, 3, 4, SPATHA_OUT_TRANSPOSED>(p, stream) : launch_ws<2, 4, 3, 4, SPATHA_OUT_ROW_MAJOR>(p, stream);

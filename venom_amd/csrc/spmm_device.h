@@ -375,21 +375,42 @@ struct WswCfg {
 // The tiles of a launch in walk order, eight consecutive chunks of them for the eight XCDs (workgroup id % 8), within a chunk
 // workgroup j of an XCD takes tiles j, j + workgroups, ...  The order decides what the workgroups of an XCD share in its L2.
 // GROUP == 1: through a tile column's row tiles, column after column (index tn * tiles_m + tm): the XCD works on one column
-// tile of B at a time and streams A past it.  GROUP == 0: through a tile row's column tiles first (index tm * tiles_n + tn),
-// GROUP == g > 1: the same within groups of g tile columns (tiles_n a multiple of g): the workgroups of an XCD then work on
-// fewer tile rows at a time, g column tiles of each - the packed A operands of a tile row enter that XCD's L2 once instead of
-// once per XCD that holds one of its column tiles.  Pays where tile rows of A are large against tile columns of B.
+// tile of B at a time and streams A past it.
+// GROUP == 0: through a tile row's column tiles first (index tm * tiles_n + tn); GROUP == g > 1: the same within groups of g
+// tile columns (tiles_n a multiple of g): the workgroups of an XCD then work on fewer tile rows at a time, g column tiles of
+// each - the packed A operands of a tile row enter that XCD's L2 once instead of once per XCD that holds one of its column
+// tiles.  Pays where tile rows of A are large against tile columns of B.
+// GROUP == -h < 0: tile rows in groups of h (tiles_m a multiple of h), within a group column after column: an XCD only ever
+// sees h tile rows of A (they stay in its L2 for the whole launch when they fit) and reads more tile columns of B instead.
 template <int GROUP>
 struct TileWalkT {
     int my_tiles, tm0, tn0, step_dm, step_dn, tiles_m, tiles_n, stride;
-    __device__ __forceinline__ int group() const { return GROUP == 0 ? tiles_n : GROUP; }
     // tile number `t` of the walk -> tile coordinates (wave-uniform, kept in scalar registers: they end up in scalar operands)
     __device__ __forceinline__ void locate(int t, int& tm, int& tn) const {
-        const int g = group(), per_group = tiles_m * g;
-        const int grp = t / per_group, rem = t - grp * per_group;
-        const int row = rem / g;
-        tm = __builtin_amdgcn_readfirstlane(row);
-        tn = __builtin_amdgcn_readfirstlane(grp * g + (rem - row * g));
+        if constexpr (GROUP >= 0) {
+            const int g = GROUP == 0 ? tiles_n : GROUP, per_group = tiles_m * g;
+            const int grp = t / per_group, rem = t - grp * per_group;
+            const int row = rem / g;
+            tm = __builtin_amdgcn_readfirstlane(row);
+            tn = __builtin_amdgcn_readfirstlane(grp * g + (rem - row * g));
+        } else {
+            constexpr int h = -GROUP;
+            const int per_group = tiles_n * h;
+            const int grp = t / per_group, rem = t - grp * per_group;
+            const int col = rem / h;
+            tn = __builtin_amdgcn_readfirstlane(col);
+            tm = __builtin_amdgcn_readfirstlane(grp * h + (rem - col * h));
+        }
+    }
+    __device__ __forceinline__ int number(int tm, int tn) const {
+        if constexpr (GROUP >= 0) {
+            const int g = GROUP == 0 ? tiles_n : GROUP, grp = tn / g;
+            return grp * tiles_m * g + tm * g + (tn - grp * g);
+        } else {
+            constexpr int h = -GROUP;
+            const int grp = tm / h;
+            return grp * tiles_n * h + tn * h + (tm - grp * h);
+        }
     }
     __device__ __forceinline__ void init(int tiles_m_, int tiles_n_) {
         tiles_m = tiles_m_;
@@ -418,8 +439,7 @@ struct TileWalkT {
             tn += step_dn;
             if (tm >= tiles_m) { tm -= tiles_m; tn += 1; }
         } else {
-            const int g = group(), grp = tn / g;
-            locate(grp * tiles_m * g + tm * g + (tn - grp * g) + stride, tm, tn);
+            locate(number(tm, tn) + stride, tm, tn);
         }
     }
 };

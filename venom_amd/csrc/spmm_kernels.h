@@ -25,7 +25,7 @@ struct SpmmParams {
     int tiles_m, tiles_n;
     int cus;                  // compute units of the device the launch goes to (grid size of the persistent kernels)
     int walk_group;           // order of the tile walk (TileWalkT): 1 column tiles one after the other (default); 0 a tile row's
-                              // column tiles first (kernel 6 only)
+                              // column tiles first (kernel 6 only); -4 tile rows in groups of four (kernel 18 only)
     // k-split (producer/consumer kernels 6 and 10 only; 1 everywhere else): tiles_m then counts (row tile, part) pairs and
     // every part runs S / ksplit k-steps; fp32 partial blocks and one ticket per 64 x 64 block live in the caller's workspace
     int ksplit;

@@ -58,6 +58,8 @@ namespace spatha {
 
 namespace {
 constexpr int UP_KNOBS = SPATHA_UP_KNOBS;
+// tile walks of this kernel: column after column, or tile rows in groups of four (SpmmParams::walk_group)
+constexpr int UP_WALK_ROWS = -4;
 __device__ __forceinline__ void pload_b128(u32x4& r, uint32_t voff, i32x4 rsrc, uint32_t soff) {
     asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=&v"(r) : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
@@ -72,8 +74,8 @@ __device__ __forceinline__ void pload_b64(u32x2& r, uint32_t voff, i32x4 rsrc, u
 // The whole life of one wave.  LATE is the wave's phase group (false: X, true: Y), a template argument so that each group
 // runs straight-line code of its own: an operand set that is in flight must never meet, at a join of two paths, a
 // version of itself that is not (the register copy the compiler may place there would copy a value that has not arrived).
-template <int OUT_LAYOUT, bool FUSE, bool GROUPED, bool LATE>
-__device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& walk, char* smem, uint32_t smem_base, int wave,
+template <int OUT_LAYOUT, bool FUSE, bool GROUPED, bool LATE, class Walk>
+__device__ __forceinline__ void up_wave(const SpmmParams& p, const Walk& walk, char* smem, uint32_t smem_base, int wave,
                                         int lane) {
     using Cfg = UpCfg;
     constexpr int NB = Cfg::NB;
@@ -306,25 +308,25 @@ __device__ __forceinline__ void up_wave(const SpmmParams& p, const TileWalk& wal
 #undef SPATHA_UP_WAIT_ALL
 }
 
-template <int OUT_LAYOUT, bool FUSE, bool GROUPED>
+template <int OUT_LAYOUT, bool FUSE, bool GROUPED, int WALK>
 __global__ __launch_bounds__(512) void spmm_up_kernel(SpmmParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const uint32_t smem_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    TileWalk walk;
+    TileWalkT<WALK> walk;
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
     if (wave >= 4) up_wave<OUT_LAYOUT, FUSE, GROUPED, true>(p, walk, smem, smem_base, wave, lane);
     else up_wave<OUT_LAYOUT, FUSE, GROUPED, false>(p, walk, smem, smem_base, wave, lane);
 }
 
-template <int OUT_LAYOUT, bool FUSE, bool GROUPED>
-static hipError_t launch_up(const SpmmParams& p, hipStream_t stream) {
+template <int OUT_LAYOUT, bool FUSE, bool GROUPED, int WALK>
+static hipError_t launch_up_walk(const SpmmParams& p, hipStream_t stream) {
     constexpr int lds = UpCfg::LDS_BYTES;
     static_assert(lds <= 160 * 1024, "LDS budget");
     const int cus = p.cus;        // compute units of the plan's device
-    void (*kern)(SpmmParams) = spmm_up_kernel<OUT_LAYOUT, FUSE, GROUPED>;
+    void (*kern)(SpmmParams) = spmm_up_kernel<OUT_LAYOUT, FUSE, GROUPED, WALK>;
     bool& attr_set = lds_attr_flag((const void*)kern);
     if (!attr_set) {
         // the kernel's register loads complete asynchronously into named variables: an instantiation that keeps
@@ -344,6 +346,12 @@ static hipError_t launch_up(const SpmmParams& p, hipStream_t stream) {
     if (grid < 8) grid = 8;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(UpCfg::THREADS), lds, stream, p);
     return hipGetLastError();
+}
+
+template <int OUT_LAYOUT, bool FUSE, bool GROUPED>
+static hipError_t launch_up(const SpmmParams& p, hipStream_t stream) {
+    if (p.walk_group == UP_WALK_ROWS && p.tiles_m % 4 == 0) return launch_up_walk<OUT_LAYOUT, FUSE, GROUPED, UP_WALK_ROWS>(p, stream);
+    return launch_up_walk<OUT_LAYOUT, FUSE, GROUPED, 1>(p, stream);
 }
 
 // largest m that runs the grouped form of the matrix phase

@@ -467,6 +467,24 @@ def test_uneven_last_round_runs_as_two_launches(gpu, transposed):
     assert np.array_equal(fused.cpu().numpy().view(np.uint16), want_b.view(np.uint16))
 
 
+@pytest.mark.parametrize("transposed", [False, True])
+def test_tile_rows_walked_in_groups_equal_the_oracle(gpu, transposed):
+    """Packed A larger than an XCD's L2 (plain 2:4, 4096 rows: 4.7 MB) with eight tile rows of the 512 x 128 kernel and 32 or
+    more tile columns: the launch walks the tile rows in groups of four.  Every tile still lands where it belongs: all of C
+    equals the oracle bit for bit (integer operands), both layouts."""
+    rows, cols, N, m, v = 4096, 1024, 4096 + 136, 4, 128
+    print("tile rows in groups", rows, cols, N, transposed, flush=True)
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=9, integer_values=True)
+    rng = np.random.default_rng(12)
+    B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+    bias = rng.integers(-3, 4, size=rows).astype(np.float16)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    assert plan.kernel_name(N, 1 if transposed else 0, 18) == "smfmac16x16x64_unified_pingpong_densestage_aregs_tile512x128_3stage"
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias if transposed else None, transposed_out=transposed)
+    got = plan.run(_dev(B, gpu), bias=_dev(bias, gpu) if transposed else None, transposed_out=transposed, variant=18)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
 @pytest.mark.parametrize("rows,cols,N,m,v", [(1024, 512, 256, 8, 64),        # unified 512 x 128 kernel
                                             (512, 2048, 520, 16, 128),       # producer/consumer kernel, ragged N
                                             (256, 1024, 16, 16, 128)])       # skinny kernel

@@ -597,12 +597,12 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
     p.cus = plan->cus > 0 ? plan->cus : 256;
     p.walk_group = 1;
     if (var == spatha::SPMM_VARIANT_UP512x128_S3) {
-        // Packed A too large to stay in an XCD's L2 beside the stream of B (plain 2:4 on a 4096-row matrix: 4.7 MB against
-        // 4 MB; it is then fetched again in every round, 160 MB per launch): tile rows in groups of four, so that an XCD only
+        // Packed A larger than an XCD's L2 (plain 2:4 on a 4096-row matrix: 4.7 MB against 4 MB; it is then fetched again in
+        // every round, 160 MB per launch): tile rows in groups of four, so that an XCD only
         // ever sees four of them (2.4 MB, resident) and reads twice as many tile columns of B instead.  2:4 FFN-up: 85-86
         // against 87-89 us.  Where A fits anyway (64:2:8: 2.4 MB) the default walk reads less.
         const size_t a_bytes = plan->apack_bytes + plan->gtab_bytes, four_rows = a_bytes / p.tiles_m * 4;
-        if (p.tiles_m % 4 == 0 && p.tiles_m >= 8 && p.tiles_n >= 32 && a_bytes > (7u << 19) && four_rows <= (3u << 20)) p.walk_group = -4;
+        if (p.tiles_m % 4 == 0 && p.tiles_m >= 8 && p.tiles_n >= 32 && a_bytes > (4u << 20) && four_rows <= (3u << 20)) p.walk_group = -4;
     }
     p.ksplit = 1; p.partial = nullptr; p.partial_bytes = 0; p.tickets = nullptr;
     p.debug = 0; p.skew = 0; p.prof = nullptr;

@@ -317,6 +317,12 @@ __global__ __launch_bounds__(512) void spmm_up_kernel(SpmmParams p) {
     TileWalkT<WALK> walk;
     walk.init(p.tiles_m, p.tiles_n);
     if (walk.my_tiles == 0) return;
+    // (development builds: the workgroups of an XCD start in four groups, skew * 1024 clocks apart, so that their write-outs
+    // no longer fall together)
+    if (SPATHA_SKEW_ON(p)) {
+        const int units = ((blockIdx.x >> 3) & 3) * p.skew;
+        for (int i = 0; i < units; i++) __builtin_amdgcn_s_sleep(16);
+    }
     if (wave >= 4) up_wave<OUT_LAYOUT, FUSE, GROUPED, true>(p, walk, smem, smem_base, wave, lane);
     else up_wave<OUT_LAYOUT, FUSE, GROUPED, false>(p, walk, smem, smem_base, wave, lane);
 }

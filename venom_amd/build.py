@@ -117,8 +117,9 @@ def build_variant(tag, defines, verbose=False, only=None):
     spmm_pingpong.hip, SPATHA_UP_KNOBS=<bits>) -> venom_amd/lib/libspatha_<tag>.so; `SPATHA_LIBRARY=<that file>` makes the
     Python binding and bench.py load it.  Needs the objects of a normal build.  Such builds compute wrong results on
     purpose (a knob removes part of the kernel's work) and are for timing and power measurements only.  `only` names the
-    kernel sources that see the switches (default: all of them)."""
-    sources = [src for src in KERNEL_SOURCES if not only or src in only]
+    sources that see the switches (default: all kernel sources; spatha_api.cpp, which reads the environment knobs of
+    -DSPATHA_DEV_PROFILE builds, has to be named)."""
+    sources = [src for src in HIP_SOURCES if src in only] if only else list(KERNEL_SOURCES)
     jobs = [[HIPCC] + HIP_FLAGS + ["-D" + d for d in defines] +
             ["-x", "hip", "-c", os.path.join(CSRC, src), "-o", os.path.join(OBJDIR, "%s.%s.o" % (src, tag))] for src in sources]
     _compile_all(jobs, verbose)

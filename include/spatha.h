@@ -243,6 +243,17 @@ int spatha_spmm_time(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
                      uint16_t* out_dev, int out_layout, int variant, int warmup, int iters, void* stream,
                      float* ms_per_launch);
 
+/* Times the automatic choice and every kernel id that accepts this plan, N and layout (spatha_spmm_time each), and
+ * reports the fastest: *best_variant (0 when nothing beats the automatic choice, which may be a form no single id gives,
+ * see spatha_spmm_kernel_name), *best_ms, and *auto_ms, the automatic choice's time.  ms_per_variant, when not NULL,
+ * holds spatha_spmm_num_variants() floats: [0] the automatic choice, [id] that kernel, negative where it does not apply.
+ * The result of every timed kernel lands in out_dev.  For callers that would rather measure their shape than trust the
+ * rule table; replaces the search over the reference's tile tuples (src/spmm/spatha_spmm.hpp:49-585, swept per shape by
+ * benchmark/run_spmm_spatha.sh). */
+int spatha_spmm_tune(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
+                     uint16_t* out_dev, int out_layout, int warmup, int iters, void* stream, int* best_variant,
+                     float* best_ms, float* auto_ms, float* ms_per_variant);
+
 /* Dense fp16 GEMM C[rows x N] = A[rows x cols] * B[cols x N] (fp32 accumulate)
  * on the GPU: the dense baseline and --check product of the benchmark.
  * Replaces Cublas_gemm<half,half,float>::sgemm (src/gemm/cublas_gemm.cpp:54-96). */

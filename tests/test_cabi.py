@@ -40,6 +40,9 @@ def test_spmm_entry_points_reject_bad_arguments_without_a_gpu():
     assert L.spatha_spmm_run(None, None, 8, None, None, 0, 0, None) == 1
     assert L.spatha_spmm_plan_destroy(None) == 0
     assert L.spatha_dense_gemm_f16(None, None, 8, 8, 8, None, None) == 1
+    best, ms = ctypes.c_int(), ctypes.c_float()
+    assert L.spatha_spmm_tune(None, None, 8, None, None, 0, 1, 1, None, None, None, None, None) == 1
+    assert L.spatha_spmm_tune(None, None, 8, None, None, 0, 1, 1, None, ctypes.byref(best), ctypes.byref(ms), None, None) == 1
 
 
 def test_unified_kernels_use_no_scratch_memory(tmp_path):

@@ -91,6 +91,21 @@ def test_config1_invocation_passes_its_own_check(gpu):
 
 
 @pytest.mark.gpu
+def test_tune_times_every_kernel_and_runs_the_fastest(gpu):
+    """--tune: the times of the automatic choice and of every kernel id that takes the shape go to stderr, the fastest id
+    runs the benchmark, and --check still holds."""
+    r = _run(_replace(_replace(CONFIG1, "--n", 2048), "--m", 512) + ["--tune"])
+    assert r.returncode == 0, r.stderr
+    lines = [l for l in r.stderr.splitlines() if l.startswith("tune:")]
+    assert len(lines) >= 3 and lines[0].startswith("tune: id  0 ")
+    assert sum("<- fastest" in l for l in lines) == 1
+    row = _row(r.stdout)
+    assert row["error"] == "0"
+    fastest = [l for l in lines if "<- fastest" in l][0]
+    assert row["kernel"] in fastest
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("m,k,n,mm_row,bm", [
     (256, 1000, 264, 10, 64),      # K % m == 0 but Ksp padded; ragged N
     (512, 330, 136, 7, 128),       # two-column tail group

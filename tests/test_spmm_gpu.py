@@ -753,3 +753,23 @@ def test_token_counts_that_are_no_multiple_of_8(gpu, N):
     got = spatha.spmm_fused(dm, dc, dv, dB, dbias, rows, cols, v, 2, m)
     assert got.shape == (rows, N) and got.is_contiguous()
     assert np.array_equal(got.cpu().numpy().view(np.uint16), np.ascontiguousarray(want_t.T).view(np.uint16))
+
+
+def test_tune_reports_the_fastest_kernel(gpu):
+    """`spatha_spmm_tune`: times for the automatic choice (id 0) and for every id that takes the shape; the reported id is the
+    minimum of them, never slower than the automatic choice, and computes the product."""
+    rows, cols, N, m, v = 1024, 2048, 1024, 8, 128
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=3, integer_values=True)
+    B = np.random.default_rng(3).integers(-4, 5, size=(cols, N)).astype(np.float16)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    dB = _dev(B, gpu)
+    out = torch.empty((rows, N), dtype=torch.float16, device=gpu)
+    best, best_ms, auto_ms, per = plan.tune(dB, out)
+    print("tune:", best, best_ms, auto_ms, per, flush=True)
+    assert 0 in per and abs(per[0] - auto_ms) < 1e-9 and len(per) >= 4
+    assert best in per and best_ms == min(per.values()) and best_ms <= auto_ms
+    assert all(1 <= i < _lib.lib().spatha_spmm_num_variants() for i in per if i)
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B)
+    got = plan.run(dB, variant=best)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))       # the last kernel timed wrote it too

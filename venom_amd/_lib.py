@@ -55,6 +55,8 @@ SIGNATURES = {
     "spatha_spmm_num_variants": (c_int, []),
     "spatha_spmm_kernel_name": (c_char_p, [c_void_p, c_int, c_int, c_int]),
     "spatha_spmm_time": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, POINTER(c_float)]),
+    "spatha_spmm_tune": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, POINTER(c_int),
+                                 POINTER(c_float), POINTER(c_float), POINTER(c_float)]),
     "spatha_dense_gemm_f16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "spatha_vnm_file_write": (c_int, [c_char_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "spatha_vnm_file_info": (c_int, [c_char_p, c_void_p, POINTER(c_int)]),

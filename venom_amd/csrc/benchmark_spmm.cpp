@@ -49,7 +49,7 @@ const char* kUsage =
     "\tOptional cmdline args:\n"
     "\t--block-size [4] --meta-block-size [32] --nn_row [2] --mm_row [m] --acc_t [fp32]\n"
     "\t--bm [V] --bn --bk --wm --wn --wk --mm --mn --mk --nstage   (tile flags: only --bm is used)\n"
-    "\t--variant [kernel id, 0 = automatic] --random --check --path_to_dset [file]\n";
+    "\t--variant [kernel id, 0 = automatic] --tune --random --check --path_to_dset [file]\n";
 
 [[noreturn]] void die(const std::string& msg) {
     std::fprintf(stderr, "%s%s\n", kUsage, msg.c_str());
@@ -96,6 +96,7 @@ int main(int argc, const char** argv) {
     int m = 0, n = 0, k = 0, block_sz = 1, meta_block_sz = 0, spmm_code = -1, gemm_code = -1, acc_code = 0;
     int pattern_code = -1, precision_code = -1, bm = 0, bn = 0, bk = 0, wm = 0, wn = 0, wk = 0, mm = 0, mn = 0, mk = 0;
     int nstage = 0, nn_row = 0, mm_row = 0, variant = 0;
+    bool tune = false;
     float density = 0.f;
     unsigned seed = 2022;
     bool check = false;
@@ -124,6 +125,7 @@ int main(int argc, const char** argv) {
         else if (a == "--mk" && has_val) mk = next_int(i);
         else if (a == "--nstage" && has_val) nstage = next_int(i);
         else if (a == "--variant" && has_val) variant = next_int(i);
+        else if (a == "--tune") tune = true;
         else if (a == "--path_to_dset" && has_val) path_to_dset = argv[++i];
         else if (a == "--random") seed = (unsigned)std::chrono::system_clock::now().time_since_epoch().count();
         else if (a == "--check") check = true;
@@ -227,6 +229,17 @@ int main(int argc, const char** argv) {
     if (st != SPATHA_OK) {
         std::fprintf(stderr, "no kernel for this configuration: %s\n", spatha_status_string(st));
         return EXIT_FAILURE;
+    }
+    if (tune) {
+        // --tune: every kernel id that takes the shape is timed, the fastest one runs the benchmark (times to stderr)
+        std::vector<float> per((size_t)spatha_spmm_num_variants(), -1.f);
+        float best_ms = 0.f, auto_ms = 0.f;
+        SPATHA_OK_OR_DIE(spatha_spmm_tune(plan, dB, n, nullptr, dC, SPATHA_OUT_ROW_MAJOR, 5, 30, nullptr, &variant, &best_ms, &auto_ms,
+                                          per.data()));
+        for (size_t id = 0; id < per.size(); id++)
+            if (per[id] >= 0.f)
+                std::fprintf(stderr, "tune: id %2zu %-72s %9.2f us%s\n", id, spatha_spmm_kernel_name(plan, n, SPATHA_OUT_ROW_MAJOR, (int)id),
+                             per[id] * 1e3f, (int)id == variant ? "  <- fastest" : "");
     }
     const char* kname = spatha_spmm_kernel_name(plan, n, SPATHA_OUT_ROW_MAJOR, variant);
     if (!kname) {

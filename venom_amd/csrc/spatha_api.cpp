@@ -726,6 +726,32 @@ int spatha_spmm_time(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
     return SPATHA_OK;
 }
 
+int spatha_spmm_tune(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N, const uint16_t* bias_dev,
+                     uint16_t* out_dev, int out_layout, int warmup, int iters, void* stream, int* best_variant,
+                     float* best_ms, float* auto_ms, float* ms_per_variant) {
+    if (!best_variant || !best_ms) return SPATHA_ERR_BAD_ARGUMENT;
+    float t_auto = 0.f;
+    int st = spatha_spmm_time(plan, B_dev, N, bias_dev, out_dev, out_layout, spatha::SPMM_VARIANT_AUTO, warmup, iters, stream, &t_auto);
+    if (st) return st;
+    if (auto_ms) *auto_ms = t_auto;
+    if (ms_per_variant) ms_per_variant[0] = t_auto;
+    int best = spatha::SPMM_VARIANT_AUTO;
+    float t_best = t_auto;
+    for (int id = 1; id < spatha::SPMM_VARIANT_COUNT; id++) {
+        if (ms_per_variant) ms_per_variant[id] = -1.f;
+        if (!variant_ok(plan, N, id, false)) continue;
+        float t = 0.f;
+        st = spatha_spmm_time(plan, B_dev, N, bias_dev, out_dev, out_layout, id, warmup, iters, stream, &t);
+        if (st == SPATHA_ERR_UNSUPPORTED) continue;     // (accepted by the shape checks, refused by the kernel's launcher)
+        if (st) return st;
+        if (ms_per_variant) ms_per_variant[id] = t;
+        if (t < t_best) { t_best = t; best = id; }
+    }
+    *best_variant = best;
+    *best_ms = t_best;
+    return SPATHA_OK;
+}
+
 int spatha_dense_gemm_f16(const uint16_t* A_dev, const uint16_t* B_dev, int rows, int cols, int N, uint16_t* C_dev,
                           void* stream) {
     if (!A_dev || !B_dev || !C_dev || rows <= 0 || cols <= 0 || N <= 0) return SPATHA_ERR_BAD_ARGUMENT;

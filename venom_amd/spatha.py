@@ -153,6 +153,21 @@ class SpmmPlan:
                        "spatha_spmm_time")
         return ms.value
 
+    def tune(self, B, out, bias=None, transposed_out=False, warmup=5, iters=30):
+        """Times the automatic choice and every kernel id that accepts this shape; returns (best id, its ms, the automatic
+        choice's ms, {id: ms}) with id 0 = the automatic choice (the best id is 0 when nothing beats it)."""
+        L = _lib.lib()
+        n = L.spatha_spmm_num_variants()
+        best, best_ms, auto_ms = ctypes.c_int(), ctypes.c_float(), ctypes.c_float()
+        per = (ctypes.c_float * n)()
+        with torch.cuda.device(self.device):
+            _lib.check(L.spatha_spmm_tune(self._handle, B.data_ptr(), B.shape[1], None if bias is None else bias.data_ptr(),
+                                          out.data_ptr(), OUT_TRANSPOSED if transposed_out else OUT_ROW_MAJOR, warmup, iters,
+                                          _stream_ptr(self.device), ctypes.byref(best), ctypes.byref(best_ms),
+                                          ctypes.byref(auto_ms), per), "spatha_spmm_tune")
+        torch.autograd.graph.increment_version(out)
+        return best.value, best_ms.value, auto_ms.value, {i: per[i] for i in range(n) if per[i] >= 0}
+
 
 def _extension():
     """The PyTorch C++ extension that holds the operator (csrc/spatha_torch.cpp, built in place by `python -m

@@ -440,13 +440,13 @@ def test_gpt3_ffn_shape_blocks_within_tolerance(gpu, N):
 
 @pytest.mark.parametrize("transposed", [False, True])
 def test_uneven_last_round_runs_as_two_launches(gpu, transposed):
-    """More 128 x 256 tiles than compute units with a rest of at most half a round: the automatic choice runs the rest's row
-    tiles as a second launch on 128 x 128 tiles.  Both launches together equal the oracle bit for bit (integer operands),
+    """More 128 x 256 tiles than compute units with a rest of at most half a round, long k-loops: the automatic choice runs the
+    rest's row tiles as a second launch on 128 x 128 tiles.  Both launches together equal the oracle bit for bit (integer operands),
     also with the bias of the transposed layout and with the fused bias of the row-major one, and equal the one-launch result
     of the same kernel asked for by id."""
     cus = torch.cuda.get_device_properties(gpu).multi_processor_count
     grid = cus // 8 * 8
-    N, m, v, cols = 2048, 16, 128, 3072
+    N, m, v, cols = 2048, 16, 128, 8192               # 32 k-steps per tile: with shorter k-loops a second launch does not pay
     rows = (grid // 8 + grid // 16) * 128            # 1.5 rounds of 128 x 256 tiles (8 column tiles)
     print("uneven last round", rows, cols, N, transposed, flush=True)
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=5, integer_values=True)

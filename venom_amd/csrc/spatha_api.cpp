@@ -103,16 +103,32 @@ struct Shape {
         const int64_t rounds = (t + cus - 1) / cus;
         return rounds == 1 ? t * 4 >= cus * 3 : t * 10 >= rounds * cus * 9;
     }
+    // unified 512 x 128 tiles against dense-staged 256 x 128 ones by rounds of tiles over the CUs, a 512-row tile counted as
+    // two and 10 % off for what it saves per tile (5120 x 1280 x 2048 at 2:8 and 2:4: 160 tiles on 256 CUs in one round, 17 and
+    // 24 us, against 1.25 rounds of 320 dense-staged tiles, 20 and 32 us)
+    bool unified_rounds_ahead() const {
+        const int64_t r_up = (tiles(512, 128) + cus - 1) / cus, r_ds = (tiles(256, 128) + cus - 1) / cus;
+        return r_up * 18 <= r_ds * 10;
+    }
     // 128 x 256 tiles ahead of 128 x 128 ones: from 1024 tiles on, from 768 with two or more k-steps, from 512 with eight or
-    // more, from 192 with a dozen or more (every kernel on the BERT layer shapes x N = 2048 .. 8192 x 2:10 .. 2:100;
+    // more; with fewer, from 192 tiles of 32 or more k-steps, and with 10 .. 31 k-steps where the rounds say so (1280 x 5120 at
+    // 128:2:16 / 20 / 32: 4096 tokens, 160 tiles in one round, 18.7 / 16.5 / 13.0 against 22.0 / 18.8 / 14.1 us; 8192 tokens, 320
+    // tiles in two rounds against 640 in three, 28.1 / 22.0 against 25.9 / 19.3 us at 2:20 / 2:32) (every kernel on the BERT layer shapes x N = 2048 .. 8192 x 2:10 .. 2:100;
     // 1024 x 1024 x 16384 at 128:2:16, 512 wide tiles of 4 k-steps, runs 19 % faster on 128 x 128 tiles)
     // (never for a single, half-empty column tile: GPT-3 FFN matrix at 128 tokens, 46.5 us on 128 x 128 against 61.5 us)
     bool wide() const {
         const int64_t t = tiles(128, 256);
-        return N > 128 && (t >= 1024 || (t >= 768 && S >= 2) || (t >= 512 && S >= 8) || (t >= 192 && S >= 12));
+        if (N <= 128) return false;
+        if (t >= 1024 || (t >= 768 && S >= 2) || (t >= 512 && S >= 8)) return true;
+        if (S >= 32) return t >= 192;
+        // few tiles of 10 .. 31 k-steps: by rounds of tiles over the CUs, a 128 x 256 tile counted as 1.6 tiles of 128 x 128
+        const int64_t r_wide = (t + cus - 1) / cus, r_narrow = (tiles(128, 128) + cus - 1) / cus;
+        return S >= 10 && t >= 160 && r_wide * 16 <= r_narrow * 10;
     }
-    // 64 x 256 tiles with long k-loops and either many rounds or at most one
-    bool long_k() const { const int64_t t = tiles(64, 256); return S >= 32 && (t >= 2048 || t <= 256); }
+    // 64 x 256 tiles with long k-loops: the persistent three-stage pipeline leads the per-tile one with two stages at any tile
+    // count (1280 x 5120 at 64:2:10, 4096 .. 16384 tokens, 320 .. 1280 tiles: 45 / 66 / 108 against 56 / 84 / 139 us;
+    // 12288 x 12288 x 512 at 64:2:16 and 64:2:10: 66 / 100 against 86 / 132 us)
+    bool long_k() const { return S >= 32; }
     // 64 x 256 tiles: many tiles of few k-steps, m >= 32, row-major
     bool short_k_many() const { return m >= 32 && !transposed && tiles(64, 256) >= 2048 && S <= 8; }
 };
@@ -152,7 +168,7 @@ const Rule kRules[] = {
     {V_128 | V_64, spatha::SPMM_VARIANT_UP512x128_S3,
      [](const Shape& s) {
          const int64_t t = s.tiles(512, 128);
-         return s.m <= 8 && s.whole_rounds(t) && (!s.transposed || t >= 2 * s.cus || s.S >= 16);
+         return s.m <= 8 && (s.whole_rounds(t) || s.unified_rounds_ahead()) && (!s.transposed || t >= 2 * s.cus || s.S >= 16);
      }},
     // 8 < m <= 16, one phase group with two 64 KB stages: 7-26 % ahead of the gathered 64 x 256 tiles on the BERT-large
     // layer shapes at N = 16384 (64:2:16 and 64:2:10, both layouts); on long k-loops ahead at 1.5 rounds too (12288 x 12288
@@ -168,7 +184,9 @@ const Rule kRules[] = {
     // transposed output, m <= 8: the kernels that write through the 8-column slab lead by 10-25 % (BERT-large layer shapes,
     // N = 16384, with bias); not on long k-loops, where the gathered 128 x 256 tile moves fewer bytes per output element
     // (GPT-3 block at 128:2:8, 96 k-steps: 6.95 ms against 8.26 ms; GPT-2-large FFN-down, 40 k-steps: dense staging 20 % ahead)
-    {V_128, spatha::SPMM_VARIANT_DS256x128_S3_C8, [](const Shape& s) { return s.transposed && s.m <= 8 && s.S <= 40; }},
+    // (m <= 5: every dense row is a gathered row or nearly so, dense staging leads at any k: 1280 x 5120 x 4096 at 2:4, 80
+    // k-steps, 45 against 65 us on 128 x 128 tiles; 12288 x 12288 x 512 at 2:4 115 against 127 us on 128 x 256 tiles)
+    {V_128, spatha::SPMM_VARIANT_DS256x128_S3_C8, [](const Shape& s) { return s.transposed && s.m <= 8 && (s.S <= 40 || s.m <= 5); }},
     // row-major, m <= 8: dense staging leads the gathered tiles by 5-35 % as soon as its 256 x 128 tiles fill three quarters
     // of the CUs (BERT layer shapes, N = 2048 .. 16384; from 160 tiles on the GPT-2-large ones).  Up to 768 tiles the form in
     // two phase groups leads the eight-consumer form by 2-5 %; it has no fused write-out, and falls behind on long k-loops
@@ -179,7 +197,9 @@ const Rule kRules[] = {
          return !s.transposed && !s.fused && s.m <= 8 && s.rows % 256 == 0 && t >= 160 && t <= 768 && s.S <= 32;
      }},
     {V_128, spatha::SPMM_VARIANT_DS256x128_S3_C8,
-     [](const Shape& s) { return !s.transposed && s.m <= 8 && s.rows % 256 == 0 && s.tiles(256, 128) >= 160 && s.S <= 64; }},
+     [](const Shape& s) {
+         return !s.transposed && s.m <= 8 && s.rows % 256 == 0 && s.tiles(256, 128) >= 160 && (s.S <= 64 || s.m <= 5);
+     }},
     // transposed output, m > 8, more than one 128-column tile: 128 x 256 tiles at any tile count (5-15 % ahead of 128 x 128 on the BERT-large and
     // GPT-2-large layer shapes, N = 4096 and 16384); 64 x 64 consumer blocks up to 16 k-steps, else the tall consumers
     {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m >= 16 && s.S <= 16; }},
@@ -282,6 +302,9 @@ int uneven_rest_rows(const spatha_spmm_plan* plan, int N, int requested, int cho
     const int tiles_n = (N + 255) / 256;
     const int64_t tiles = (int64_t)(plan->geo.rows / 128) * tiles_n, rest = tiles % grid;
     if (tiles <= grid || rest == 0 || rest % tiles_n != 0) return 0;
+    // (short k-loops: a second launch costs more than the half-empty round; 1280 x 5120 x 16384 at 128:2:16 / 20 / 32, 20 / 16 /
+    // 10 k-steps: 52 / 46 / 36 us in one launch against 56 / 50 / 40 in two)
+    if (plan->S < 32) return 0;
     const int rest_rows = (int)(rest / tiles_n) * 128;
     if ((int64_t)(rest_rows / 128) * ((N + 127) / 128) > grid) return 0;        // more than half a round: one launch
     if ((plan->geo.rows - rest_rows) % plan->geo.v != 0) return 0;
@@ -641,9 +664,19 @@ int spatha::plan_run(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
         tail.C = out_layout == SPATHA_OUT_TRANSPOSED ? out_dev + main_rows : out_dev + (size_t)main_rows * N;
         tail.tiles_m = rest_rows / 128;
         tail.tiles_n = (N + 127) / 128;
-        // the two column tiles of a tile row on one XCD at the same time: its A operands (0.44 MB per tile row of the GPT-3
-        // FFN matrix) enter one L2 instead of two
-        tail.walk_group = 0;
+        // Which way the tail's tiles are walked decides what an XCD's workgroups (grid / 8 tiles at a time) pull into its L2
+        // per round: column-first, the A operands of up to grid / 8 tile rows + few tile columns of B; row-first, all tile
+        // columns of few tile rows.  GPT-3 FFN matrix at 256 tokens (0.44 MB of A per tile row, two tile columns of 3.1 MB):
+        // 13.4 against 17.3 MB row-first, the second launch fetches 108 instead of 142 MB; with few tile rows and many tile
+        // columns (1280 x 5120 at 8192 tokens: 2 x 128 tiles) column-first moves half as much.
+        {
+            const int64_t at_a_time = std::max(1, p.cus / 8);
+            const double a_row = (double)plan->apack_bytes / (plan->geo.rows / 128.0), b_col = (double)plan->geo.cols * 128 * 2;
+            const int64_t tm = tail.tiles_m, tn = tail.tiles_n;
+            const double col_first = (double)std::min(at_a_time, tm) * a_row + (double)((at_a_time + tm - 1) / tm) * b_col;
+            const double row_first = (double)((at_a_time + tn - 1) / tn) * a_row + (double)std::min(at_a_time, tn) * b_col;
+            tail.walk_group = row_first < col_first ? 0 : 1;
+        }
         hipError_t e2 = spatha::launch_spmm(var, out_layout, head, (hipStream_t)stream);
         if (e2 == hipSuccess) e2 = spatha::launch_spmm(spatha::SPMM_VARIANT_W128x128_S3, out_layout, tail, (hipStream_t)stream);
         return e2 == hipSuccess ? SPATHA_OK : hip_fail(e2);
@@ -730,13 +763,12 @@ int spatha_spmm_tune(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
                      uint16_t* out_dev, int out_layout, int warmup, int iters, void* stream, int* best_variant,
                      float* best_ms, float* auto_ms, float* ms_per_variant) {
     if (!best_variant || !best_ms) return SPATHA_ERR_BAD_ARGUMENT;
+    // (a first, untimed pass of the automatic choice: argument checks, and the clocks are up when the first id is timed)
     float t_auto = 0.f;
     int st = spatha_spmm_time(plan, B_dev, N, bias_dev, out_dev, out_layout, spatha::SPMM_VARIANT_AUTO, warmup, iters, stream, &t_auto);
     if (st) return st;
-    if (auto_ms) *auto_ms = t_auto;
-    if (ms_per_variant) ms_per_variant[0] = t_auto;
     int best = spatha::SPMM_VARIANT_AUTO;
-    float t_best = t_auto;
+    float t_best = 0.f;
     for (int id = 1; id < spatha::SPMM_VARIANT_COUNT; id++) {
         if (ms_per_variant) ms_per_variant[id] = -1.f;
         if (!variant_ok(plan, N, id, false)) continue;
@@ -745,8 +777,14 @@ int spatha_spmm_tune(const spatha_spmm_plan* plan, const uint16_t* B_dev, int N,
         if (st == SPATHA_ERR_UNSUPPORTED) continue;     // (accepted by the shape checks, refused by the kernel's launcher)
         if (st) return st;
         if (ms_per_variant) ms_per_variant[id] = t;
-        if (t < t_best) { t_best = t; best = id; }
+        if (best == spatha::SPMM_VARIANT_AUTO || t < t_best) { t_best = t; best = id; }
     }
+    // the automatic choice last, in the same warm state as the ids: it wins ties (it may be one of them)
+    st = spatha_spmm_time(plan, B_dev, N, bias_dev, out_dev, out_layout, spatha::SPMM_VARIANT_AUTO, warmup, iters, stream, &t_auto);
+    if (st) return st;
+    if (auto_ms) *auto_ms = t_auto;
+    if (ms_per_variant) ms_per_variant[0] = t_auto;
+    if (best == spatha::SPMM_VARIANT_AUTO || t_auto <= t_best) { t_best = t_auto; best = spatha::SPMM_VARIANT_AUTO; }
     *best_variant = best;
     *best_ms = t_best;
     return SPATHA_OK;

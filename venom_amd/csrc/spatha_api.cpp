@@ -108,7 +108,9 @@ struct Shape {
     // 24 us, against 1.25 rounds of 320 dense-staged tiles, 20 and 32 us)
     bool unified_rounds_ahead() const {
         const int64_t r_up = (tiles(512, 128) + cus - 1) / cus, r_ds = (tiles(256, 128) + cus - 1) / cus;
-        return r_up * 18 <= r_ds * 10;
+        // (long k-loops, where a tile's write-out weighs less: 25 % off - 12288 x 12288 x 2048 at 64:2:8 and 2:4, 384 tiles in two
+        // rounds against 768 in three, 212 / 396 against 236 / 429 us)
+        return r_up * (S >= 64 ? 15 : 18) <= r_ds * 10;
     }
     // 128 x 256 tiles ahead of 128 x 128 ones: from 1024 tiles on, from 768 with two or more k-steps, from 512 with eight or
     // more; with fewer, from 192 tiles of 32 or more k-steps, and with 10 .. 31 k-steps where the rounds say so (1280 x 5120 at
@@ -124,6 +126,13 @@ struct Shape {
         // few tiles of 10 .. 31 k-steps: by rounds of tiles over the CUs, a 128 x 256 tile counted as 1.6 tiles of 128 x 128
         const int64_t r_wide = (t + cus - 1) / cus, r_narrow = (tiles(128, 128) + cus - 1) / cus;
         return S >= 10 && t >= 160 && r_wide * 16 <= r_narrow * 10;
+    }
+    // transposed output: 128 x 256 tiles from 512 tiles on, with fewer by rounds (a 128 x 256 tile counted as 1.6 of 128 x 128)
+    bool wide_transposed() const {
+        const int64_t t = tiles(128, 256);
+        if (t >= 512) return true;
+        const int64_t r_wide = (t + cus - 1) / cus, r_narrow = (tiles(128, 128) + cus - 1) / cus;
+        return r_wide * 16 <= r_narrow * 10;
     }
     // 64 x 256 tiles with long k-loops: the persistent three-stage pipeline leads the per-tile one with two stages at any tile
     // count (1280 x 5120 at 64:2:10, 4096 .. 16384 tokens, 320 .. 1280 tiles: 45 / 66 / 108 against 56 / 84 / 139 us;
@@ -168,7 +177,10 @@ const Rule kRules[] = {
     {V_128 | V_64, spatha::SPMM_VARIANT_UP512x128_S3,
      [](const Shape& s) {
          const int64_t t = s.tiles(512, 128);
-         return s.m <= 8 && (s.whole_rounds(t) || s.unified_rounds_ahead()) && (!s.transposed || t >= 2 * s.cus || s.S >= 16);
+         // (transposed output with one or two full rounds of 8 k-steps is level with the dense-staged 256 x 128 tiles or 2-3 %
+         // behind; with less than a round - 3072 x 1024 x 4096, 5120 x 1280 x 2048: 192 and 160 tiles - 11-13 % ahead)
+         return s.m <= 8 && (s.whole_rounds(t) || s.unified_rounds_ahead()) &&
+                (!s.transposed || t >= 2 * s.cus || s.S >= 16 || t < s.cus);
      }},
     // 8 < m <= 16, one phase group with two 64 KB stages: 7-26 % ahead of the gathered 64 x 256 tiles on the BERT-large
     // layer shapes at N = 16384 (64:2:16 and 64:2:10, both layouts); on long k-loops ahead at 1.5 rounds too (12288 x 12288
@@ -186,7 +198,10 @@ const Rule kRules[] = {
     // (GPT-3 block at 128:2:8, 96 k-steps: 6.95 ms against 8.26 ms; GPT-2-large FFN-down, 40 k-steps: dense staging 20 % ahead)
     // (m <= 5: every dense row is a gathered row or nearly so, dense staging leads at any k: 1280 x 5120 x 4096 at 2:4, 80
     // k-steps, 45 against 65 us on 128 x 128 tiles; 12288 x 12288 x 512 at 2:4 115 against 127 us on 128 x 256 tiles)
-    {V_128, spatha::SPMM_VARIANT_DS256x128_S3_C8, [](const Shape& s) { return s.transposed && s.m <= 8 && (s.S <= 40 || s.m <= 5); }},
+    // (from 160 tiles on, as row-major: with fewer - 1024 x 4096 x 2048 / 4096, 1280 x 5120 x 2048: 64 .. 128 tiles - the
+    // gathered 128 x 128 tiles are 13-35 % ahead)
+    {V_128, spatha::SPMM_VARIANT_DS256x128_S3_C8,
+     [](const Shape& s) { return s.transposed && s.m <= 8 && (s.S <= 40 || s.m <= 5) && s.tiles(256, 128) >= 160; }},
     // row-major, m <= 8: dense staging leads the gathered tiles by 5-35 % as soon as its 256 x 128 tiles fill three quarters
     // of the CUs (BERT layer shapes, N = 2048 .. 16384; from 160 tiles on the GPT-2-large ones).  Up to 768 tiles the form in
     // two phase groups leads the eight-consumer form by 2-5 %; it has no fused write-out, and falls behind on long k-loops
@@ -202,9 +217,12 @@ const Rule kRules[] = {
      }},
     // transposed output, m > 8, more than one 128-column tile: 128 x 256 tiles at any tile count (5-15 % ahead of 128 x 128 on the BERT-large and
     // GPT-2-large layer shapes, N = 4096 and 16384); 64 x 64 consumer blocks up to 16 k-steps, else the tall consumers
-    {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m >= 16 && s.S <= 16; }},
-    {V_128, spatha::SPMM_VARIANT_T128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m > 8; }},
-    {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m > 8; }},
+    // (with fewer than 512 of them only where the rounds of tiles over the CUs say so: 1024 x 4096 x 2048, 1280 x 1280 x 2048,
+    // 1280 x 5120 x 2048 at 128:2:16 .. 32 - 64, 80, 80 tiles - run 24-41 % faster on 128 x 128 tiles)
+    {V_128, spatha::SPMM_VARIANT_W128x256_S3,
+     [](const Shape& s) { return s.transposed && s.N > 128 && s.m >= 16 && s.S <= 16 && s.wide_transposed(); }},
+    {V_128, spatha::SPMM_VARIANT_T128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m > 8 && s.wide_transposed(); }},
+    {V_128, spatha::SPMM_VARIANT_W128x256_S3, [](const Shape& s) { return s.transposed && s.N > 128 && s.m > 8 && s.wide_transposed(); }},
     // row-major, two or three k-steps per tile and more than two rounds of 128 x 128 tiles: the kernel with store waves (a finished tile
     // leaves while the next one's k-loop runs) leads the 128 x 256 tiles by 7-18 % and the plain 128 x 128 ones by 14-23 %
     // (4096 x 1024 x 16384 at 128:2:32, 3072 x 768 x 8192 at 128:2:40, 1024 x 1024 x 16384 at 128:2:32); with transposed output

@@ -151,14 +151,15 @@ struct Rule {
 };
 
 const Rule kRules[] = {
-    // few columns: streaming A is all that matters, one 64-row tile per workgroup with the k-steps split over its waves
-    // (N = 32: equal on the GPT-3 FFN matrix, 1.3-1.5x ahead on the BERT-large ones; N = 48, 64: behind the 128-wide tiles)
+    // few columns: streaming A is all that matters, one 64-row tile per workgroup with the k-steps split over its waves, B
+    // straight from the L2 with one load per gathered row whatever N (2, 4 or 8 bytes for 16, 32 or 64 columns).  Up to 32
+    // columns: 1.3-1.5x ahead of every tiled kernel on the BERT-large matrices, 31.7 us on the GPT-3 FFN matrix (5.6 TB/s;
+    // 128-wide tiles 39-41).  33 .. 64 columns, V a multiple of 64: 5.7 us on 4096 x 1024 at 64:2:8 and 128:2:8 (tiled
+    // kernels 6.8-7.7), 31.3 us on 12288 x 12288 at 64:2:8 (49.2), 7.4 us on 1024 x 4096 at 64:2:16 (equal); on the GPT-3 FFN
+    // matrix 40.5 us, level with the 128 x 128 tiles (39.4): there the 192 registers of its four column blocks leave two
+    // workgroups per CU for three tiles per CU.
     {V_HALF | V_128 | V_64, spatha::SPMM_VARIANT_SKINNY, [](const Shape& s) { return s.N <= 32; }},
-    // V a multiple of 64 only, m <= 8, up to 48 columns: still 9-22 % ahead of the dense-staged 256 x 128 tiles (4096 x 1024 and
-    // 12288 x 12288 at 64:2:8; at 64 columns ahead on the larger matrix only).  With V % 128 == 0 the 128 x 128 tiles lead it by
-    // 5-10 % from 40 columns on (m = 4 .. 32).  m > 8 with a dozen or more k-steps: up to 64 columns, 15-22 % ahead of the
-    // gathered 64 x 256 tiles (1024 x 4096 and 768 x 3072 at 64:2:16; with fewer k-steps 11-30 % behind them).
-    {V_64, spatha::SPMM_VARIANT_SKINNY, [](const Shape& s) { return s.m <= 8 ? s.N <= 48 : (s.N <= 64 && s.S >= 12); }},
+    {V_128 | V_64, spatha::SPMM_VARIANT_SKINNY, [](const Shape& s) { return s.N <= 64; }},
 
     // -- V % 64 != 0 (1024 x 4096 x 4096 and 4096 x 1024 x 16384, m = 8 .. 32) --
     // m <= 8: the dense B stage is shared by eight 32-row blocks, the fill does not grow with the smaller V

@@ -120,7 +120,11 @@ def test_half_tile_kernels_bit_exact(gpu, rows, cols, N, m, v, transposed):
         assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16)), (variant,)
     assert ran >= 4                          # automatic choice + three gathered tile shapes (+ dense-staged when it applies)
     if m <= 8 and rows % 256 == 0:
-        assert ran == 5 and "densestage" in plan.kernel_name(N, 1 if transposed else 0, 0)
+        assert ran == 5 and "densestage" in plan.kernel_name(N, 1 if transposed else 0, 17)
+        # dense staging is the automatic choice from 16 k-steps on or with 160 tiles or more; shorter, smaller products
+        # go to the gathered half-tile kernels
+        if (cols * 2 // m + 31) // 32 >= 16:
+            assert "densestage" in plan.kernel_name(N, 1 if transposed else 0, 0)
 
 
 def test_half_tile_gaussian_within_tolerance(gpu):

@@ -163,7 +163,10 @@ const Rule kRules[] = {
 
     // -- V % 64 != 0 (1024 x 4096 x 4096 and 4096 x 1024 x 16384, m = 8 .. 32) --
     // m <= 8: the dense B stage is shared by eight 32-row blocks, the fill does not grow with the smaller V
-    {V_HALF, spatha::SPMM_VARIANT_DSH256x128_S3_C8, [](const Shape&) { return true; }},
+    // (short k-loops - 8 or 10 k-steps - on 64 tiles or fewer, 1024 x 1024 up to 2048 tokens, 4096 x 1024 up to 512: the gathered
+    // half-tile kernels are 9-24 % ahead; with 32 k-steps or more dense staging leads at any tile count, 1.2-3.4x on 1024 x 4096,
+    // 1280 x 5120 and 12288 x 12288)
+    {V_HALF, spatha::SPMM_VARIANT_DSH256x128_S3_C8, [](const Shape& s) { return s.tiles(256, 128) >= 160 || s.S >= 16; }},
     // the 256-wide tile is never behind the 128-wide one with two stages by more than 7 %, and up to 2x ahead
     {V_HALF, spatha::SPMM_VARIANT_H64x256_S2, [](const Shape& s) { return s.N > 128; }},
     // (three stages of 128 leave two waves per CU)

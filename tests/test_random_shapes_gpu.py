@@ -114,3 +114,45 @@ def test_automatic_choice_on_random_shapes_bit_exact(gpu, chunk):
     print("kernels reached so far:", dict(kernels), flush=True)
     if chunk == 3 and sum(kernels.values()) > 150:
         assert len(kernels) >= 12          # the sweep is only worth its time if it reaches most of the registry
+
+
+@pytest.mark.gpu
+def test_every_kernel_id_on_random_shapes_bit_exact(gpu):
+    """The same draw with another seed, through EVERY kernel id that accepts the shape (a caller may name an id, and
+    spatha_spmm_tune runs them all): 120 shapes, about 900 launches, each equal to the oracle bit for bit."""
+    launches = 0
+    reached = set()
+    for i, (rows, cols, N, m, v, mode) in enumerate(draw_cases(120, seed=11)):
+        transposed = mode in ("transposed_bias", "fused_bias_transposed")
+        fused = mode.startswith("fused")
+        vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=5000 + i, integer_values=True)
+        rng = np.random.default_rng(7000 + i)
+        B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+        bias = None if mode == "row_major" else rng.integers(-8, 9, size=rows).astype(np.float16)
+        want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias, transposed_out=True) if bias is not None \
+            else oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B)
+        if bias is not None and not transposed:
+            want = np.ascontiguousarray(want.T)
+        plan = spatha.SpmmPlan(_dev(vals, gpu), _dev(meta, gpu), _dev(columns, gpu), rows, cols, 2, m, v)
+        dB, dbias = _dev(B, gpu), None if bias is None else _dev(bias, gpu)
+        for variant in range(1, spatha.num_variants()):
+            name = plan.kernel_name(N, 1 if transposed else 0, variant)
+            if name is None:
+                continue
+            print("case %d id %d: %d x %d x %d, %d:2:%d, %s -> %s" % (i, variant, rows, cols, N, v, m, mode, name), flush=True)
+            try:
+                got = plan.run(dB, bias=dbias, transposed_out=transposed, activation="none" if fused else None, variant=variant)
+            except RuntimeError as e:
+                assert fused and "no kernel" in str(e), (variant, str(e))    # ids without a fused write-out say so
+                continue
+            torch.cuda.synchronize()
+            got = got.cpu().numpy()
+            if not np.array_equal(got.view(np.uint16), want.view(np.uint16)):
+                bad = np.argwhere(got.view(np.uint16) != want.view(np.uint16))
+                pytest.fail("case %d id %d (%d x %d x %d, %d:2:%d, %s, kernel %s): %d entries differ, first at %s"
+                            % (i, variant, rows, cols, N, v, m, mode, name, len(bad), tuple(bad[0])))
+            launches += 1
+            reached.add(variant)
+        del plan
+    print("launches", launches, "ids", sorted(reached), flush=True)
+    assert launches > 600 and len(reached) >= 20

@@ -415,6 +415,37 @@ def test_full_size_checksums(gpu, rows, cols, N, m, v):
     assert torch.equal(Ct.t(), C)
 
 
+@pytest.mark.parametrize("m,v", [(8, 128), (16, 128), (8, 32)])
+def test_output_beyond_four_gib(gpu, m, v):
+    """C larger than 2^32 bytes (and 2^31 elements): 32768 x 69632 fp16 = 4.56 GB, so every address of the write-out
+    needs 64-bit arithmetic.  Row sums, column sums and the LAST rows against products the CPU can afford (exact for
+    small integers), row-major and transposed."""
+    rows, cols, N = 32768, 32 * m, 69632
+    assert rows * N * 2 > 2 ** 32 and rows * N > 2 ** 31
+    print("beyond 4 GiB", rows, cols, N, m, v, flush=True)
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=3, integer_values=True)
+    vals = np.clip(vals, -2, 2).astype(np.float16)
+    rng = np.random.default_rng(4)
+    B = rng.integers(-1, 2, size=(cols, N)).astype(np.float16)
+    dense = oracle.decode(vals, meta, columns, rows, cols, 2, m, v).astype(np.float64)
+    B64 = B.astype(np.float64)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    dB = _dev(B, gpu)
+    for transposed in (False, True):
+        print("   ", plan.kernel_name(N, 1 if transposed else 0, 0), flush=True)
+        C = plan.run(dB, transposed_out=transposed)
+        torch.cuda.synchronize()
+        assert C.numel() > 2 ** 31
+        row_sums = C.sum(dim=0 if transposed else 1, dtype=torch.float64).cpu().numpy()
+        col_sums = C.sum(dim=1 if transposed else 0, dtype=torch.float64).cpu().numpy()
+        assert np.array_equal(row_sums, dense @ B64.sum(axis=1))
+        assert np.array_equal(col_sums, dense.sum(axis=0) @ B64)
+        tail = (C[:, rows - 192:].t() if transposed else C[rows - 192:]).cpu().numpy().astype(np.float64)
+        assert np.array_equal(tail, dense[rows - 192:] @ B64)
+        del C
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("N", [16, 256, 2048])
 def test_gpt3_ffn_shape_blocks_within_tolerance(gpu, N):
     """GPT-3 feed-forward shape: A 49152 x 12288 in 128:2:16, values ~N(0, 0.02), B ~N(0, 1); N = 16 runs on the skinny

@@ -37,7 +37,7 @@ __global__ __launch_bounds__(WM* WN * 64) void spmm_kernel(SpmmParams p) {
     const int S = p.S, N = p.N;
 
     const int64_t wt = (int64_t)(m0 / 64 + wm);                       // wave tile index along rows
-    const char* a_blk = (const char*)p.apack + (wt * S) * APACK_BLOCK;   // + s*APACK_BLOCK
+    const char* a_blk = (const char*)p.apack + ((int64_t)wt * S) * APACK_BLOCK;   // + s*APACK_BLOCK
     const uint32_t* rt = p.rowtab + (int64_t)(m0 / p.v) * S * 64;
 
     // B loader coordinates

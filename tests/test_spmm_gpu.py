@@ -474,6 +474,36 @@ def test_gpt3_ffn_shape_blocks_within_tolerance(gpu, N):
 
 
 @pytest.mark.parametrize("transposed", [False, True])
+@pytest.mark.parametrize("N,cols,m", [(2048, 8192, 16), (1992, 2390, 20), (904, 4096, 32)])
+def test_a_round_and_a_half_runs_as_tiles_and_a_half(gpu, N, cols, m, transposed):
+    """Between one and one and a half rounds of 128 x 256 tiles over the compute units (m > 8): the automatic choice is the
+    kernel whose workgroups take one whole tile and a 128-column half of another.  Integer operands, bit-exact against the
+    oracle, with the bias of the transposed layout, with the fused bias in both layouts, ragged K and N, and equal to the
+    tall 128 x 256 kernel asked for by id."""
+    cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+    grid = cus // 8 * 8
+    v, tiles_n = 128, (N + 255) // 256
+    rows = (grid + grid // 2) // tiles_n * 128       # 1.5 rounds (or just under)
+    print("a round and a half", rows, cols, N, m, transposed, flush=True)
+    vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=6, integer_values=True)
+    rng = np.random.default_rng(12)
+    B = rng.integers(-4, 5, size=(cols, N)).astype(np.float16)
+    bias = rng.integers(-3, 4, size=rows).astype(np.float16)
+    plan = _plan(vals, meta, columns, rows, cols, m, v, gpu)
+    name = plan.kernel_name(N, 1 if transposed else 0, 0)
+    assert "tile_and_a_half" in name, name
+    want = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias if transposed else None, transposed_out=transposed)
+    got = plan.run(_dev(B, gpu), bias=_dev(bias, gpu) if transposed else None, transposed_out=transposed)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    tall = plan.run(_dev(B, gpu), bias=_dev(bias, gpu) if transposed else None, transposed_out=transposed, variant=10)
+    assert torch.equal(tall, got)
+    fused = plan.run(_dev(B, gpu), bias=_dev(bias, gpu), transposed_out=transposed, activation="none")
+    want_b = oracle.spmm(vals, meta, columns, rows, cols, 2, m, v, B, bias=bias, transposed_out=True)       # [N, rows]
+    want_b = want_b if transposed else np.ascontiguousarray(want_b.T)
+    assert np.array_equal(fused.cpu().numpy().view(np.uint16), want_b.view(np.uint16))
+
+
+@pytest.mark.parametrize("transposed", [False, True])
 def test_uneven_last_round_runs_as_two_launches(gpu, transposed):
     """More 128 x 256 tiles than compute units with a rest of at most half a round, long k-loops: the automatic choice runs the
     rest's row tiles as a second launch on 128 x 128 tiles.  Both launches together equal the oracle bit for bit (integer operands),
@@ -482,7 +512,7 @@ def test_uneven_last_round_runs_as_two_launches(gpu, transposed):
     cus = torch.cuda.get_device_properties(gpu).multi_processor_count
     grid = cus // 8 * 8
     N, m, v, cols = 2048, 16, 128, 8192               # 32 k-steps per tile: with shorter k-loops a second launch does not pay
-    rows = (grid // 8 + grid // 16) * 128            # 1.5 rounds of 128 x 256 tiles (8 column tiles)
+    rows = (2 * (grid // 8) + grid // 16) * 128      # 2.5 rounds of 128 x 256 tiles (8 column tiles)
     print("uneven last round", rows, cols, N, transposed, flush=True)
     vals, meta, columns = F.synthetic_vnm(rows, cols, 2, m, v, seed=5, integer_values=True)
     rng = np.random.default_rng(11)

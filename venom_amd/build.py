@@ -28,7 +28,7 @@ CXX_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-fopenmp", "-Wall"]
 
 # the SpMM kernels, one source per family (spmm_device.h holds what they share)
 KERNEL_SOURCES = ["spmm_gathered.hip", "spmm_warpspec.hip", "spmm_densestage.hip", "spmm_unified.hip", "spmm_pingpong.hip",
-                  "spmm_skinny.hip"]
+                  "spmm_skinny.hip", "spmm_onehalf.hip"]
 HIP_SOURCES = KERNEL_SOURCES + ["spmm_pack.hip", "spmm_dispatch.hip", "dense_gemm.hip", "transpose.hip", "layernorm.hip",
                                 "select_gpu.hip", "spmm_static.hip", "spatha_api.cpp"]
 CXX_SOURCES = ["vnm_format.cpp"]

@@ -33,7 +33,7 @@ bool variant_has_fused_writeout(int variant) {
         case SPMM_VARIANT_W128x128_S3: case SPMM_VARIANT_W128x256_S3: case SPMM_VARIANT_W64x256_S3:
         case SPMM_VARIANT_T128x256_S3: case SPMM_VARIANT_DS256x128_S3_C8: case SPMM_VARIANT_DSH256x128_S3_C8:
         case SPMM_VARIANT_UP512x128_S3: case SPMM_VARIANT_DU512x128_M16: case SPMM_VARIANT_WS128x128_S3:
-        case SPMM_VARIANT_WS64x256_S3: case SPMM_VARIANT_H64x256_S2: case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2:
+        case SPMM_VARIANT_WS64x256_S3: case SPMM_VARIANT_OH192x256: case SPMM_VARIANT_H64x256_S2: case SPMM_VARIANT_H64x128_S3: case SPMM_VARIANT_H64x128_S2:
             return true;
         default:
             return false;
@@ -138,6 +138,22 @@ struct Shape {
     // count (1280 x 5120 at 64:2:10, 4096 .. 16384 tokens, 320 .. 1280 tiles: 45 / 66 / 108 against 56 / 84 / 139 us;
     // 12288 x 12288 x 512 at 64:2:16 and 64:2:10: 66 / 100 against 86 / 132 us)
     bool long_k() const { return S >= 32; }
+    // More than one round of 128 x 256 tiles over the CUs and at most a round and a half: F = ceil(2T / 3) workgroups per
+    // 256-column tile, each with one whole tile and a 128-column half of another, run them in ONE round of equal workgroups
+    // that stay in step through k (kernel 22).  Every kernel id on 49152 / 40960 / 36864 / 34816 x 12288 (GPT-3 FFN matrix and
+    // fewer rows of it; 384 .. 272 row tiles on 256 CUs) at 136 .. 256 tokens, 128:2:16, Gaussian data: 53-57 / 52 / 50 / 50 us
+    // against 61-66 us for 256 tall tiles + the rest on 128 x 128 tiles in a second launch; the same rows x 1024 .. 6144
+    // columns (4 .. 24 k-steps), where the 128 x 128 tiles with store waves were chosen: 1.06-1.36x ahead row-major from 8
+    // k-steps on (4 k-steps: 0.94-1.06x), 1.19-1.53x transposed; 128:2:40 1.28-1.70x; 16128 x 12288 x 768 and 12288^2 x
+    // 1024 (three and four column tiles) 57 us against 59-70.  Not for m <= 8 (dense staging: 1.07-1.09x at 2:8 on the long
+    // k-loop only, behind at 2:4), not when the last column tile has no columns for the second half, not beyond one round of
+    // such workgroups (8192 x 4096 x 1536: 41 against 27 us).
+    bool tile_and_a_half() const {
+        if (m <= 8 || rows % 128 != 0 || S < 4 || (S < 8 && !transposed)) return false;
+        const int64_t T = rows / 128, tn = (N + 255) / 256, F = (2 * T + 2) / 3, grid = (cus / 8) * 8;
+        const int last = N - (int)(tn - 1) * 256;
+        return T * tn > grid && F * tn <= grid && last > 128;
+    }
     // 64 x 256 tiles: many tiles of few k-steps, m >= 32, row-major
     bool short_k_many() const { return m >= 32 && !transposed && tiles(64, 256) >= 2048 && S <= 8; }
 };
@@ -219,6 +235,8 @@ const Rule kRules[] = {
      [](const Shape& s) {
          return !s.transposed && s.m <= 8 && s.rows % 256 == 0 && s.tiles(256, 128) >= 160 && (s.S <= 64 || s.m <= 5);
      }},
+    // m > 8, between one and one and a half rounds of 128 x 256 tiles: one whole tile and a column half of another per workgroup
+    {V_128, spatha::SPMM_VARIANT_OH192x256, [](const Shape& s) { return s.tile_and_a_half(); }},
     // transposed output, m > 8, more than one 128-column tile: 128 x 256 tiles at any tile count (5-15 % ahead of 128 x 128 on the BERT-large and
     // GPT-2-large layer shapes, N = 4096 and 16384); 64 x 64 consumer blocks up to 16 k-steps, else the tall consumers
     // (with fewer than 512 of them only where the rounds of tiles over the CUs say so: 1024 x 4096 x 2048, 1280 x 1280 x 2048,

@@ -369,6 +369,19 @@ struct WswCfg {
     static constexpr uint32_t RT_BASE = EPI_BASE + EPI_BYTES;
 };
 
+// LDS layout of the tile-and-a-half kernel (spmm_onehalf.hip): per k-step an F sub-stage (64 gathered B rows of 256 columns
+// + two operand blocks) and an H sub-stage (64 gathered B rows of 128 columns + two operand blocks), two of each, and a
+// row-table ring of four slots.
+struct OhCfg {
+    static constexpr int ROW_BYTES = 512, HROW_BYTES = 256;
+    static constexpr int B_BYTES = 64 * ROW_BYTES, HB_BYTES = 64 * HROW_BYTES;
+    static constexpr int F_BYTES = B_BYTES + 2 * APACK_BLOCK;
+    static constexpr int H_BYTES = HB_BYTES + 2 * APACK_BLOCK;
+    static constexpr int PAIR = F_BYTES + H_BYTES;
+    static constexpr int RT_BASE = 2 * PAIR;
+    static constexpr int LDS_BYTES = RT_BASE + 4 * 256;
+};
+
 // Tile walk shared by both roles: XCD x (= workgroup id % 8) owns a contiguous range of tile
 // ids (id -> n-tile major, m-tile minor) and its workgroups take them round robin; the
 // coordinates advance by a fixed (dm, dn) with carry, so no division per tile.

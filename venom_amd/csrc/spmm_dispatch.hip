@@ -15,6 +15,7 @@ struct VariantInfo {
 };
 
 const VariantInfo kVariants[] = {
+    {SPMM_VARIANT_OH192x256, "smfmac16x16x64_warpspec_tile_and_a_half_192x256_4slots", 128, 256, OhCfg::LDS_BYTES, 0, launch_onehalf},
     {SPMM_VARIANT_128x128, "smfmac16x16x64_wg256_tile128x128", 128, 128, 1, 0, launch_gathered},
     {SPMM_VARIANT_64x256, "smfmac16x16x64_wg256_tile64x256", 64, 256, 1, 0, launch_gathered},
     {SPMM_VARIANT_P128x128_S3, "smfmac16x16x64_ldsdirect_tile128x128_3stage", 128, 128, 3 * (64 * 128 * 2 + 2 * APACK_BLOCK), 256,

@@ -66,7 +66,8 @@ enum {
     SPMM_VARIANT_DU512x128_M16 = 19,    // 8 < m <= 16: one phase group, 64 KB stages, two of them
     SPMM_VARIANT_WS128x128_S3 = 20,     // id 6 with store waves: finished tiles leave through an LDS staging buffer and a third role
     SPMM_VARIANT_WS64x256_S3 = 21,      // id 8 with store waves
-    SPMM_VARIANT_COUNT = 22
+    SPMM_VARIANT_OH192x256 = 22,        // V % 128 == 0: a whole 128 x 256 tile and a 64-row half of another one per workgroup, one k-loop
+    SPMM_VARIANT_COUNT = 23
 };
 
 const char* spmm_variant_name(int variant);
@@ -77,13 +78,14 @@ int spmm_variant_lds(int variant, int S);
 hipError_t launch_spmm(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 
 // one launch switch per kernel family (spmm_gathered.hip, spmm_warpspec.hip, spmm_densestage.hip, spmm_unified.hip,
-// spmm_skinny.hip, spmm_pingpong.hip); hipErrorInvalidValue for an id of another family
+// spmm_skinny.hip, spmm_pingpong.hip, spmm_onehalf.hip); hipErrorInvalidValue for an id of another family
 hipError_t launch_gathered(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 hipError_t launch_warpspec(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 hipError_t launch_densestage(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 hipError_t launch_unified(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 hipError_t launch_skinny_family(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 hipError_t launch_pingpong(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
+hipError_t launch_onehalf(int variant, int out_layout, const SpmmParams& p, hipStream_t stream);
 
 hipError_t launch_pack(const uint16_t* values, const uint32_t* metadata, const uint32_t* columns, int rows, int cols,
                        int m, int v, int ksp, int S, int half_tiles, uint16_t* apack, uint32_t* rowtab, hipStream_t stream);

@@ -45,8 +45,8 @@ MEASURED_TRAFFIC = {
         (61_530_000, "profiles/spmm_wsw_kernel_tile128x128_config1_128-2-8.md"),
     ("smfmac16x16x64_skinny_tile64xN_splitk4", 49152, 12288, 16, 16, 128):
         (184_100_000, "profiles/spmm_skinny_kernel_gpt3_ffn_n16.md"),
-    ("smfmac16x16x64_warpspec_tall_tile128x256_3stage+rest_on_tile128x128", 49152, 12288, 256, 16, 128):
-        (300_800_000, "profiles/spmm_wst_ws_kernels_gpt3_ffn_n256_128-2-16.md"),
+    ("smfmac16x16x64_warpspec_tile_and_a_half_192x256_4slots", 49152, 12288, 256, 16, 128):
+        (251_500_000, "profiles/spmm_oh_kernel_gpt3_ffn_n256_128-2-16.md"),
     ("smfmac16x16x64_warpspec_tall_tile128x256_3stage", 49152, 12288, 2048, 16, 128):
         (2_202_100_000, "profiles/spmm_wst_kernel_tile128x256_gpt3_ffn_n2048.md"),
 }

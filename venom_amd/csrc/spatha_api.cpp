@@ -147,12 +147,14 @@ struct Shape {
     // k-steps on (4 k-steps: 0.94-1.06x), 1.19-1.53x transposed; 128:2:40 1.28-1.70x; 16128 x 12288 x 768 and 12288^2 x
     // 1024 (three and four column tiles) 57 us against 59-70.  Not for m <= 8 (dense staging: 1.07-1.09x at 2:8 on the long
     // k-loop only, behind at 2:4), not when the last column tile has no columns for the second half, not beyond one round of
-    // such workgroups (8192 x 4096 x 1536: 41 against 27 us).
+    // such workgroups (8192 x 4096 x 1536: 41 against 27 us), and for at most four column tiles: with many of them (few row
+    // tiles, a large output: 1536 x 4096 x 8192, 1280 x 5120 x 8192, 768 x 3072 x 16384, 3072 x 4096 x 3584) the 128 x 128 tiles
+    // with store waves, which write a tile out under the next tile's k-loop, are level (transposed) or 3-12 % ahead (row-major).
     bool tile_and_a_half() const {
         if (m <= 8 || rows % 128 != 0 || S < 4 || (S < 8 && !transposed)) return false;
         const int64_t T = rows / 128, tn = (N + 255) / 256, F = (2 * T + 2) / 3, grid = (cus / 8) * 8;
         const int last = N - (int)(tn - 1) * 256;
-        return T * tn > grid && F * tn <= grid && last > 128;
+        return tn <= 4 && T * tn > grid && F * tn <= grid && last > 128;
     }
     // 64 x 256 tiles: many tiles of few k-steps, m >= 32, row-major
     bool short_k_many() const { return m >= 32 && !transposed && tiles(64, 256) >= 2048 && S <= 8; }
